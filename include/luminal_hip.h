@@ -1,0 +1,146 @@
+/*
+ * luminal_hip.h — C ABI of libluminal_hip.so, the MI355X (gfx950) backend for the
+ * attention hot path of Luminal.jl.
+ *
+ * Every entry point is `extern "C"`, takes plain pointers and sizes, never throws, never
+ * aborts, and returns LMH_OK (0) or a negative LMH_E_* code; lmh_last_error() then holds a
+ * human-readable message (thread-local). The library keeps no pointer past a call and
+ * allocates nothing inside the attention entry points: outputs and the decode workspace are
+ * caller-owned, exactly like the pre-allocated node buffers the reference's compiled graph
+ * hands to execute_op! (reference src/Compiler.jl:218-255).
+ *
+ * Tensor layout: row-major [B, H, S, D] addressed through element strides for (b, h, s);
+ * the innermost (D) stride must be 1. A Julia (B,H,S,D) array is column-major, so the Julia
+ * glue uploads permutedims(x, (4,3,2,1)).
+ */
+#ifndef LUMINAL_HIP_H
+#define LUMINAL_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define LMH_VERSION 100 /* major*10000 + minor*100 + patch */
+
+/* status codes */
+#define LMH_OK 0
+#define LMH_E_NULL (-1)        /* a required pointer is null */
+#define LMH_E_SHAPE (-2)       /* non-positive or inconsistent dimension / stride */
+#define LMH_E_UNSUPPORTED (-3) /* head dim / dtype / head map not implemented */
+#define LMH_E_WORKSPACE (-4)   /* decode workspace missing or too small */
+#define LMH_E_HIP (-5)         /* a HIP runtime call failed */
+#define LMH_E_NODEVICE (-6)    /* no usable gfx950 device */
+
+/* element type of q/k/v/out; accumulation is always fp32 */
+#define LMH_F32 0
+#define LMH_F16 1
+#define LMH_BF16 2
+/* out_f32 (a field of both parameter blocks): 0 writes the result in the input element type,
+ * 1 writes fp32. A bf16 result carries a rounding error of up to 2^-8 of its magnitude on its
+ * own, more than the 2e-3 parity budget of the half-precision configurations, so bf16 callers
+ * that need that budget ask for fp32. */
+
+/* which KV head a query head reads.
+ * INTERLEAVED: hq % Hkv — what the reference's repeat_kv produces, because its
+ *   Expand(dim 3) + Reshape run on column-major arrays (reference src/NN.jl:305-317,
+ *   src/Execution.jl:238-248, :228).
+ * BLOCKED: hq / (Hq/Hkv) — the row-major (HuggingFace) convention. */
+#define LMH_HEADMAP_INTERLEAVED 0
+#define LMH_HEADMAP_BLOCKED 1
+
+/* ---- runtime plumbing: replaces CUDA.functional()/CuArray()/Array() in the reference's
+ * device layer (reference src/Device.jl:31-74 get_device, :82-96 to_device, :103-105
+ * from_device). ---- */
+int lmh_version(void);
+const char *lmh_last_error(void);
+/* number of visible gfx950 devices; 0 when there is none (never an error) */
+int lmh_device_count(void);
+/* select the device and run the health check get_device() does (a 4-byte alloc+free) */
+int lmh_init(int device);
+int lmh_device_name(char *buf, size_t buf_bytes);
+int lmh_malloc(void **dev_ptr, size_t bytes);
+int lmh_free(void *dev_ptr);
+int lmh_memset(void *dev_ptr, int byte_value, size_t bytes, void *stream);
+int lmh_memcpy_h2d(void *dst_dev, const void *src_host, size_t bytes, void *stream);
+/* copies and then synchronises the stream, like Array(::CuArray) */
+int lmh_memcpy_d2h(void *dst_host, const void *src_dev, size_t bytes, void *stream);
+int lmh_memcpy_d2d(void *dst_dev, const void *src_dev, size_t bytes, void *stream);
+int lmh_sync(void *stream);
+/* HIP-event timing on a stream (for benchmarks) */
+int lmh_event_create(void **event);
+int lmh_event_destroy(void *event);
+int lmh_event_record(void *event, void *stream);
+int lmh_event_elapsed_ms(float *ms, void *start, void *stop);
+
+/* ---- flash attention forward: replaces
+ *   execute_op!(out, op::FlashAttentionOp, q, k, v)   reference src/Execution.jl:565-578
+ *   flash_attn_cpu(q, k, v, scale, causal)            reference src/Execution.jl:453-479
+ * generalised to Sq != Sk (cross attention, reference src/Whisper.jl:299-316) and to
+ * Hkv < Hq (GQA, reference src/NN.jl:305-317, :362-382).
+ *
+ * out[b,hq,i,:] = sum_j softmax_j(scale * q[b,hq,i,:] . k[b,kvh,j,:]) v[b,kvh,j,:]
+ * with j restricted to j <= i when causal != 0 (the reference skips j > i,
+ * src/Execution.jl:462), and to j < kv_len[b] when kv_len is non-null. ---- */
+typedef struct lmh_attn_params {
+  void *out;          /* [B,Hq,Sq,D] device */
+  const void *q;      /* [B,Hq,Sq,D] device */
+  const void *k;      /* [B,Hkv,Sk,D] device */
+  const void *v;      /* [B,Hkv,Sk,D] device */
+  const int32_t *kv_len; /* optional device int32[B]: valid keys per sequence (1..Sk); null = Sk */
+  int32_t B, Hq, Hkv, Sq, Sk, D;
+  int64_t q_stride[3]; /* element strides for (b, h, s); all-zero = contiguous */
+  int64_t k_stride[3];
+  int64_t v_stride[3];
+  int64_t o_stride[3];
+  int32_t dtype;    /* element type of q, k, v: LMH_F32 / LMH_F16 / LMH_BF16 */
+  float scale;      /* FlashAttentionOp.scale, reference src/Ops.jl:104-107 */
+  int32_t causal;   /* FlashAttentionOp.causal */
+  int32_t head_map; /* LMH_HEADMAP_* */
+  int32_t out_f32;  /* 0: out has element type `dtype`; 1: out is fp32 */
+  void *stream;     /* hipStream_t, null = default stream */
+} lmh_attn_params;
+
+int lmh_flash_attn_fwd(const lmh_attn_params *p);
+
+/* ---- single-token decode attention over a KV cache: replaces the un-fused subgraph
+ *   whisper_self_attn_cached  reference src/Whisper.jl:584-620 (slice 0:step_pos+1, matmul,
+ *   softmax, matmul) and whisper_cross_attn_cached :628-645, over a cache laid out like
+ *   KVCacheState :519-540, i.e. (B, H, max_seq, D); with GQA per reference src/NN.jl:305-317.
+ *
+ * out[b,hq,:] = sum_{j < kv_len[b]} softmax_j(scale * q[b,hq,:] . K[b,kvh,j,:]) V[b,kvh,j,:]
+ * Rows j >= kv_len[b] of the cache are never read into the result. ---- */
+typedef struct lmh_decode_params {
+  void *out;             /* [B,Hq,D] device */
+  const void *q;         /* [B,Hq,D] device */
+  const void *k_cache;   /* [B,Hkv,Lmax,D] device */
+  const void *v_cache;   /* [B,Hkv,Lmax,D] device */
+  const int32_t *kv_len; /* device int32[B], each in 1..Lmax; null = Lmax for every b */
+  int32_t B, Hq, Hkv, Lmax, D;
+  int64_t q_stride[2];   /* (b, h); all-zero = contiguous */
+  int64_t o_stride[2];
+  int64_t k_stride[3];   /* (b, h, s); all-zero = contiguous */
+  int64_t v_stride[3];
+  int32_t dtype;         /* element type of q and the caches */
+  float scale;
+  int32_t head_map;
+  int32_t out_f32;       /* 0: out has element type `dtype`; 1: out is fp32 */
+  int32_t num_splits;    /* KV splits per (b, kv head); 0 = choose */
+  void *workspace;       /* device, >= lmh_decode_workspace_bytes(...) */
+  size_t workspace_bytes;
+  void *stream;
+} lmh_decode_params;
+
+/* bytes of split-KV partial storage lmh_decode_attn needs for these sizes (0 on bad input) */
+size_t lmh_decode_workspace_bytes(int32_t B, int32_t Hq, int32_t Hkv, int32_t Lmax, int32_t D,
+                                  int32_t num_splits);
+/* the split count lmh_decode_attn uses when num_splits == 0 */
+int32_t lmh_decode_auto_splits(int32_t B, int32_t Hkv, int32_t Lmax);
+int lmh_decode_attn(const lmh_decode_params *p);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* LUMINAL_HIP_H */

@@ -1,0 +1,191 @@
+"""ctypes binding of libluminal_hip.so — one Python function per C-ABI entry point of
+include/luminal_hip.h, with LMH_E_* codes turned into LuminalHipError (the Julia glue does the
+same with error(unsafe_string(lmh_last_error()))).
+
+There is no CPU fallback: if the shared library is missing, load() raises.
+"""
+import ctypes
+import os
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(HERE, "lib", "libluminal_hip.so")
+
+LMH_F32, LMH_F16, LMH_BF16 = 0, 1, 2
+HEADMAP_INTERLEAVED, HEADMAP_BLOCKED = 0, 1
+DTYPE_CODES = {"f32": LMH_F32, "f16": LMH_F16, "bf16": LMH_BF16}
+DTYPE_BYTES = {"f32": 4, "f16": 2, "bf16": 2}
+
+LMH_OK = 0
+LMH_E_NULL, LMH_E_SHAPE, LMH_E_UNSUPPORTED, LMH_E_WORKSPACE, LMH_E_HIP, LMH_E_NODEVICE = -1, -2, -3, -4, -5, -6
+
+# every symbol include/luminal_hip.h declares
+EXPORTS = [
+    "lmh_version", "lmh_last_error", "lmh_device_count", "lmh_init", "lmh_device_name", "lmh_malloc", "lmh_free",
+    "lmh_memset", "lmh_memcpy_h2d", "lmh_memcpy_d2h", "lmh_memcpy_d2d", "lmh_sync", "lmh_event_create",
+    "lmh_event_destroy", "lmh_event_record", "lmh_event_elapsed_ms", "lmh_flash_attn_fwd",
+    "lmh_decode_workspace_bytes", "lmh_decode_auto_splits", "lmh_decode_attn",
+]
+
+
+class LuminalHipError(RuntimeError):
+    def __init__(self, code, message):
+        super().__init__("libluminal_hip error %d: %s" % (code, message))
+        self.code = code
+
+
+class AttnParams(ctypes.Structure):
+    _fields_ = [
+        ("out", ctypes.c_void_p), ("q", ctypes.c_void_p), ("k", ctypes.c_void_p), ("v", ctypes.c_void_p),
+        ("kv_len", ctypes.c_void_p),
+        ("B", ctypes.c_int32), ("Hq", ctypes.c_int32), ("Hkv", ctypes.c_int32), ("Sq", ctypes.c_int32),
+        ("Sk", ctypes.c_int32), ("D", ctypes.c_int32),
+        ("q_stride", ctypes.c_int64 * 3), ("k_stride", ctypes.c_int64 * 3), ("v_stride", ctypes.c_int64 * 3),
+        ("o_stride", ctypes.c_int64 * 3),
+        ("dtype", ctypes.c_int32), ("scale", ctypes.c_float), ("causal", ctypes.c_int32),
+        ("head_map", ctypes.c_int32), ("out_f32", ctypes.c_int32), ("stream", ctypes.c_void_p),
+    ]
+
+
+class DecodeParams(ctypes.Structure):
+    _fields_ = [
+        ("out", ctypes.c_void_p), ("q", ctypes.c_void_p), ("k_cache", ctypes.c_void_p), ("v_cache", ctypes.c_void_p),
+        ("kv_len", ctypes.c_void_p),
+        ("B", ctypes.c_int32), ("Hq", ctypes.c_int32), ("Hkv", ctypes.c_int32), ("Lmax", ctypes.c_int32),
+        ("D", ctypes.c_int32),
+        ("q_stride", ctypes.c_int64 * 2), ("o_stride", ctypes.c_int64 * 2), ("k_stride", ctypes.c_int64 * 3),
+        ("v_stride", ctypes.c_int64 * 3),
+        ("dtype", ctypes.c_int32), ("scale", ctypes.c_float), ("head_map", ctypes.c_int32),
+        ("out_f32", ctypes.c_int32), ("num_splits", ctypes.c_int32), ("workspace", ctypes.c_void_p), ("workspace_bytes", ctypes.c_size_t),
+        ("stream", ctypes.c_void_p),
+    ]
+
+
+_lib = None
+
+
+def load():
+    """Load the shared library (once). Raises if it has not been built."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise RuntimeError(
+            "libluminal_hip.so is not built (%s missing); run `python luminal.jl_amd/build.py`. "
+            "This backend has no CPU fallback." % LIB_PATH)
+    L = ctypes.CDLL(LIB_PATH)
+    vp = ctypes.c_void_p
+    L.lmh_version.restype = ctypes.c_int
+    L.lmh_last_error.restype = ctypes.c_char_p
+    L.lmh_device_count.restype = ctypes.c_int
+    L.lmh_init.argtypes = [ctypes.c_int]
+    L.lmh_device_name.argtypes = [ctypes.c_char_p, ctypes.c_size_t]
+    L.lmh_malloc.argtypes = [ctypes.POINTER(vp), ctypes.c_size_t]
+    L.lmh_free.argtypes = [vp]
+    L.lmh_memset.argtypes = [vp, ctypes.c_int, ctypes.c_size_t, vp]
+    L.lmh_memcpy_h2d.argtypes = [vp, vp, ctypes.c_size_t, vp]
+    L.lmh_memcpy_d2h.argtypes = [vp, vp, ctypes.c_size_t, vp]
+    L.lmh_memcpy_d2d.argtypes = [vp, vp, ctypes.c_size_t, vp]
+    L.lmh_sync.argtypes = [vp]
+    L.lmh_event_create.argtypes = [ctypes.POINTER(vp)]
+    L.lmh_event_destroy.argtypes = [vp]
+    L.lmh_event_record.argtypes = [vp, vp]
+    L.lmh_event_elapsed_ms.argtypes = [ctypes.POINTER(ctypes.c_float), vp, vp]
+    L.lmh_flash_attn_fwd.argtypes = [ctypes.POINTER(AttnParams)]
+    L.lmh_decode_attn.argtypes = [ctypes.POINTER(DecodeParams)]
+    L.lmh_decode_workspace_bytes.restype = ctypes.c_size_t
+    L.lmh_decode_workspace_bytes.argtypes = [ctypes.c_int32] * 6
+    L.lmh_decode_auto_splits.restype = ctypes.c_int32
+    L.lmh_decode_auto_splits.argtypes = [ctypes.c_int32] * 3
+    for name in ("lmh_init", "lmh_device_name", "lmh_malloc", "lmh_free", "lmh_memset", "lmh_memcpy_h2d",
+                 "lmh_memcpy_d2h", "lmh_memcpy_d2d", "lmh_sync", "lmh_event_create", "lmh_event_destroy",
+                 "lmh_event_record", "lmh_event_elapsed_ms", "lmh_flash_attn_fwd", "lmh_decode_attn"):
+        getattr(L, name).restype = ctypes.c_int
+    _lib = L
+    return L
+
+
+def check(rc):
+    if rc != LMH_OK:
+        raise LuminalHipError(rc, load().lmh_last_error().decode("utf-8", "replace"))
+
+
+def device_count():
+    return int(load().lmh_device_count())
+
+
+def init(device=0):
+    check(load().lmh_init(device))
+
+
+def device_name():
+    buf = ctypes.create_string_buffer(256)
+    check(load().lmh_device_name(buf, 256))
+    return buf.value.decode()
+
+
+def malloc(nbytes):
+    p = ctypes.c_void_p()
+    check(load().lmh_malloc(ctypes.byref(p), nbytes))
+    return p.value or 0
+
+
+def free(ptr):
+    check(load().lmh_free(ptr))
+
+
+def memset(ptr, value, nbytes, stream=None):
+    check(load().lmh_memset(ptr, value, nbytes, stream))
+
+
+def memcpy_h2d(dst, src_host_ptr, nbytes, stream=None):
+    check(load().lmh_memcpy_h2d(dst, src_host_ptr, nbytes, stream))
+
+
+def memcpy_d2h(dst_host_ptr, src, nbytes, stream=None):
+    check(load().lmh_memcpy_d2h(dst_host_ptr, src, nbytes, stream))
+
+
+def memcpy_d2d(dst, src, nbytes, stream=None):
+    check(load().lmh_memcpy_d2d(dst, src, nbytes, stream))
+
+
+def sync(stream=None):
+    check(load().lmh_sync(stream))
+
+
+class Event:
+    def __init__(self):
+        p = ctypes.c_void_p()
+        check(load().lmh_event_create(ctypes.byref(p)))
+        self.ptr = p.value
+
+    def record(self, stream=None):
+        check(load().lmh_event_record(self.ptr, stream))
+
+    def elapsed_ms_since(self, start):
+        ms = ctypes.c_float()
+        check(load().lmh_event_elapsed_ms(ctypes.byref(ms), start.ptr, self.ptr))
+        return float(ms.value)
+
+    def __del__(self):
+        try:
+            if self.ptr:
+                load().lmh_event_destroy(self.ptr)
+        except Exception:
+            pass
+
+
+def flash_attn_fwd(params):
+    check(load().lmh_flash_attn_fwd(ctypes.byref(params)))
+
+
+def decode_attn(params):
+    check(load().lmh_decode_attn(ctypes.byref(params)))
+
+
+def decode_workspace_bytes(B, Hq, Hkv, Lmax, D, num_splits=0):
+    return int(load().lmh_decode_workspace_bytes(B, Hq, Hkv, Lmax, D, num_splits))
+
+
+def decode_auto_splits(B, Hkv, Lmax):
+    return int(load().lmh_decode_auto_splits(B, Hkv, Lmax))

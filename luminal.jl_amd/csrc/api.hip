@@ -1,0 +1,301 @@
+// C-ABI layer of libluminal_hip.so: argument validation, dispatch to the kernel launchers, and
+// the small device-runtime surface (allocation, copies, sync, events) that stands in for the
+// CuArray()/Array() calls of the reference's device layer (reference src/Device.jl:82-105).
+#include <stdarg.h>
+#include <stdio.h>
+#include <string.h>
+
+#include "common.hpp"
+
+namespace lmh {
+
+static thread_local char g_last_error[512] = "";
+
+int fail(int code, const char *fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_last_error, sizeof(g_last_error), fmt, ap);
+  va_end(ap);
+  return code;
+}
+
+int hip_fail(hipError_t e, const char *what) {
+  return fail(LMH_E_HIP, "HIP error %d (%s) in %s", (int)e, hipGetErrorString(e), what);
+}
+
+namespace {
+
+bool all_zero(const int64_t *s, int n) {
+  for (int i = 0; i < n; i++)
+    if (s[i] != 0) return false;
+  return true;
+}
+
+size_t elem_bytes(int dtype) { return dtype == LMH_F32 ? 4 : 2; }
+
+bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+}  // namespace
+}  // namespace lmh
+
+using namespace lmh;
+
+extern "C" {
+
+int lmh_version(void) { return LMH_VERSION; }
+
+const char *lmh_last_error(void) { return g_last_error; }
+
+int lmh_device_count(void) {
+  int n = 0;
+  if (hipGetDeviceCount(&n) != hipSuccess) {
+    (void)hipGetLastError();
+    return 0;
+  }
+  int usable = 0;
+  for (int i = 0; i < n; i++) {
+    hipDeviceProp_t prop;
+    if (hipGetDeviceProperties(&prop, i) == hipSuccess && strncmp(prop.gcnArchName, "gfx950", 6) == 0) usable++;
+  }
+  return usable;
+}
+
+int lmh_init(int device) {
+  int n = 0;
+  if (hipGetDeviceCount(&n) != hipSuccess || n <= 0) {
+    (void)hipGetLastError();
+    return fail(LMH_E_NODEVICE, "no HIP device visible");
+  }
+  if (device < 0 || device >= n) return fail(LMH_E_NODEVICE, "device %d out of range (have %d)", device, n);
+  hipDeviceProp_t prop;
+  LMH_HIP_TRY(hipGetDeviceProperties(&prop, device));
+  if (strncmp(prop.gcnArchName, "gfx950", 6) != 0)
+    return fail(LMH_E_NODEVICE, "device %d is %s; this library carries gfx950 code only", device, prop.gcnArchName);
+  LMH_HIP_TRY(hipSetDevice(device));
+  void *probe = nullptr;  // same health check as get_device(): a tiny allocation
+  LMH_HIP_TRY(hipMalloc(&probe, 4));
+  LMH_HIP_TRY(hipFree(probe));
+  return LMH_OK;
+}
+
+int lmh_device_name(char *buf, size_t buf_bytes) {
+  if (!buf || buf_bytes == 0) return fail(LMH_E_NULL, "lmh_device_name: null buffer");
+  int dev = 0;
+  LMH_HIP_TRY(hipGetDevice(&dev));
+  hipDeviceProp_t prop;
+  LMH_HIP_TRY(hipGetDeviceProperties(&prop, dev));
+  snprintf(buf, buf_bytes, "%s (%s, %d CUs)", prop.name, prop.gcnArchName, prop.multiProcessorCount);
+  return LMH_OK;
+}
+
+int lmh_malloc(void **dev_ptr, size_t bytes) {
+  if (!dev_ptr) return fail(LMH_E_NULL, "lmh_malloc: null result pointer");
+  *dev_ptr = nullptr;
+  if (bytes == 0) return LMH_OK;
+  LMH_HIP_TRY(hipMalloc(dev_ptr, bytes));
+  return LMH_OK;
+}
+
+int lmh_free(void *dev_ptr) {
+  if (!dev_ptr) return LMH_OK;
+  LMH_HIP_TRY(hipFree(dev_ptr));
+  return LMH_OK;
+}
+
+int lmh_memset(void *dev_ptr, int byte_value, size_t bytes, void *stream) {
+  if (bytes == 0) return LMH_OK;
+  if (!dev_ptr) return fail(LMH_E_NULL, "lmh_memset: null pointer");
+  LMH_HIP_TRY(hipMemsetAsync(dev_ptr, byte_value, bytes, (hipStream_t)stream));
+  return LMH_OK;
+}
+
+int lmh_memcpy_h2d(void *dst_dev, const void *src_host, size_t bytes, void *stream) {
+  if (bytes == 0) return LMH_OK;
+  if (!dst_dev || !src_host) return fail(LMH_E_NULL, "lmh_memcpy_h2d: null pointer");
+  LMH_HIP_TRY(hipMemcpyAsync(dst_dev, src_host, bytes, hipMemcpyHostToDevice, (hipStream_t)stream));
+  LMH_HIP_TRY(hipStreamSynchronize((hipStream_t)stream));  // the host buffer may be reused at once
+  return LMH_OK;
+}
+
+int lmh_memcpy_d2h(void *dst_host, const void *src_dev, size_t bytes, void *stream) {
+  if (bytes == 0) return LMH_OK;
+  if (!dst_host || !src_dev) return fail(LMH_E_NULL, "lmh_memcpy_d2h: null pointer");
+  LMH_HIP_TRY(hipMemcpyAsync(dst_host, src_dev, bytes, hipMemcpyDeviceToHost, (hipStream_t)stream));
+  LMH_HIP_TRY(hipStreamSynchronize((hipStream_t)stream));
+  return LMH_OK;
+}
+
+int lmh_memcpy_d2d(void *dst_dev, const void *src_dev, size_t bytes, void *stream) {
+  if (bytes == 0) return LMH_OK;
+  if (!dst_dev || !src_dev) return fail(LMH_E_NULL, "lmh_memcpy_d2d: null pointer");
+  LMH_HIP_TRY(hipMemcpyAsync(dst_dev, src_dev, bytes, hipMemcpyDeviceToDevice, (hipStream_t)stream));
+  return LMH_OK;
+}
+
+int lmh_sync(void *stream) {
+  LMH_HIP_TRY(hipStreamSynchronize((hipStream_t)stream));
+  return LMH_OK;
+}
+
+int lmh_event_create(void **event) {
+  if (!event) return fail(LMH_E_NULL, "lmh_event_create: null result pointer");
+  hipEvent_t e;
+  LMH_HIP_TRY(hipEventCreate(&e));
+  *event = e;
+  return LMH_OK;
+}
+
+int lmh_event_destroy(void *event) {
+  if (!event) return LMH_OK;
+  LMH_HIP_TRY(hipEventDestroy((hipEvent_t)event));
+  return LMH_OK;
+}
+
+int lmh_event_record(void *event, void *stream) {
+  if (!event) return fail(LMH_E_NULL, "lmh_event_record: null event");
+  LMH_HIP_TRY(hipEventRecord((hipEvent_t)event, (hipStream_t)stream));
+  return LMH_OK;
+}
+
+int lmh_event_elapsed_ms(float *ms, void *start, void *stop) {
+  if (!ms || !start || !stop) return fail(LMH_E_NULL, "lmh_event_elapsed_ms: null argument");
+  LMH_HIP_TRY(hipEventSynchronize((hipEvent_t)stop));
+  LMH_HIP_TRY(hipEventElapsedTime(ms, (hipEvent_t)start, (hipEvent_t)stop));
+  return LMH_OK;
+}
+
+// --------------------------------------------------------------------------------------------
+// flash attention forward
+// --------------------------------------------------------------------------------------------
+int lmh_flash_attn_fwd(const lmh_attn_params *p) {
+  if (!p) return fail(LMH_E_NULL, "lmh_flash_attn_fwd: null params");
+  if (!p->out || !p->q || !p->k || !p->v) return fail(LMH_E_NULL, "lmh_flash_attn_fwd: null tensor pointer");
+  if (p->B <= 0 || p->Hq <= 0 || p->Hkv <= 0 || p->Sq <= 0 || p->Sk <= 0 || p->D <= 0)
+    return fail(LMH_E_SHAPE, "lmh_flash_attn_fwd: non-positive dimension (B=%d Hq=%d Hkv=%d Sq=%d Sk=%d D=%d)", p->B,
+                p->Hq, p->Hkv, p->Sq, p->Sk, p->D);
+  if (p->Hq % p->Hkv != 0)
+    return fail(LMH_E_SHAPE, "lmh_flash_attn_fwd: Hq=%d is not a multiple of Hkv=%d", p->Hq, p->Hkv);
+  if (p->dtype != LMH_F32 && p->dtype != LMH_F16 && p->dtype != LMH_BF16)
+    return fail(LMH_E_UNSUPPORTED, "lmh_flash_attn_fwd: unknown dtype %d", p->dtype);
+  if (p->head_map != LMH_HEADMAP_INTERLEAVED && p->head_map != LMH_HEADMAP_BLOCKED)
+    return fail(LMH_E_UNSUPPORTED, "lmh_flash_attn_fwd: unknown head_map %d", p->head_map);
+  if (p->D > 128) return fail(LMH_E_UNSUPPORTED, "lmh_flash_attn_fwd: head dim %d > 128 is not supported", p->D);
+  if (!(p->scale == p->scale)) return fail(LMH_E_SHAPE, "lmh_flash_attn_fwd: scale is NaN");
+
+  PrefillArgs a;
+  a.out = p->out; a.q = p->q; a.k = p->k; a.v = p->v; a.kv_len = p->kv_len;
+  a.B = p->B; a.Hq = p->Hq; a.Hkv = p->Hkv; a.Sq = p->Sq; a.Sk = p->Sk; a.D = p->D;
+  a.scale = p->scale; a.causal = p->causal ? 1 : 0; a.head_map = p->head_map;
+  a.out_f32 = (p->out_f32 != 0 || p->dtype == LMH_F32) ? 1 : 0;
+  auto fill = [&](int64_t *dst, const int64_t *src, int64_t H, int64_t S) {
+    if (all_zero(src, 3)) {
+      dst[0] = H * S * p->D; dst[1] = S * p->D; dst[2] = p->D;
+    } else {
+      dst[0] = src[0]; dst[1] = src[1]; dst[2] = src[2];
+    }
+  };
+  fill(a.qs, p->q_stride, p->Hq, p->Sq);
+  fill(a.os, p->o_stride, p->Hq, p->Sq);
+  fill(a.ks, p->k_stride, p->Hkv, p->Sk);
+  fill(a.vs, p->v_stride, p->Hkv, p->Sk);
+  for (int i = 0; i < 3; i++)
+    if (a.qs[i] < 0 || a.os[i] < 0 || a.ks[i] < 0 || a.vs[i] < 0)
+      return fail(LMH_E_SHAPE, "lmh_flash_attn_fwd: negative stride");
+  if (a.qs[2] < p->D || a.os[2] < p->D || a.ks[2] < p->D || a.vs[2] < p->D)
+    return fail(LMH_E_SHAPE, "lmh_flash_attn_fwd: row stride smaller than head dim (rows overlap)");
+
+  // The matrix-core kernel does 128-bit accesses and tracks the max on raw scores (needs scale>0).
+  bool mfma_ok = prefill_mfma_supported(p->dtype, p->D) && p->scale > 0.f && aligned16(p->q) && aligned16(p->k) &&
+                 aligned16(p->v) && aligned16(p->out);
+  for (int i = 0; i < 3 && mfma_ok; i++)
+    mfma_ok = (a.qs[i] % 8 == 0) && (a.ks[i] % 8 == 0) && (a.vs[i] % 8 == 0) && (a.os[i] % 8 == 0);
+  if (mfma_ok) return launch_prefill_mfma(a, p->dtype, (hipStream_t)p->stream);
+  return launch_prefill_valu(a, p->dtype, (hipStream_t)p->stream);
+}
+
+// --------------------------------------------------------------------------------------------
+// decode attention
+// --------------------------------------------------------------------------------------------
+int32_t lmh_decode_auto_splits(int32_t B, int32_t Hkv, int32_t Lmax) {
+  if (B <= 0 || Hkv <= 0 || Lmax <= 0) return 0;
+  // Aim for >= 4096 workgroups (16 per CU) but keep 256..1024 keys per split: shorter splits
+  // spend their time in the prologue/merge, longer ones balance ragged batches badly.
+  const int64_t pairs = (int64_t)B * Hkv;
+  int64_t want = (4096 + pairs - 1) / pairs;
+  int64_t chunk = (Lmax + want - 1) / want;
+  if (chunk < 256) chunk = 256;
+  if (chunk > 1024) chunk = 1024;
+  chunk = (chunk + 63) / 64 * 64;
+  int64_t splits = (Lmax + chunk - 1) / chunk;
+  return (int32_t)(splits < 1 ? 1 : splits);
+}
+
+size_t lmh_decode_workspace_bytes(int32_t B, int32_t Hq, int32_t Hkv, int32_t Lmax, int32_t D, int32_t num_splits) {
+  if (B <= 0 || Hq <= 0 || Hkv <= 0 || Lmax <= 0 || D <= 0 || num_splits < 0) return 0;
+  if (num_splits == 0) num_splits = lmh_decode_auto_splits(B, Hkv, Lmax);
+  if (num_splits == 1) return 0;
+  return (size_t)B * Hq * num_splits * (size_t)(D + 2) * sizeof(float);
+}
+
+int lmh_decode_attn(const lmh_decode_params *p) {
+  if (!p) return fail(LMH_E_NULL, "lmh_decode_attn: null params");
+  if (!p->out || !p->q || !p->k_cache || !p->v_cache) return fail(LMH_E_NULL, "lmh_decode_attn: null tensor pointer");
+  if (p->B <= 0 || p->Hq <= 0 || p->Hkv <= 0 || p->Lmax <= 0 || p->D <= 0)
+    return fail(LMH_E_SHAPE, "lmh_decode_attn: non-positive dimension (B=%d Hq=%d Hkv=%d Lmax=%d D=%d)", p->B, p->Hq,
+                p->Hkv, p->Lmax, p->D);
+  if (p->Hq % p->Hkv != 0) return fail(LMH_E_SHAPE, "lmh_decode_attn: Hq=%d is not a multiple of Hkv=%d", p->Hq, p->Hkv);
+  if (p->dtype != LMH_F32 && p->dtype != LMH_F16 && p->dtype != LMH_BF16)
+    return fail(LMH_E_UNSUPPORTED, "lmh_decode_attn: unknown dtype %d", p->dtype);
+  if (p->head_map != LMH_HEADMAP_INTERLEAVED && p->head_map != LMH_HEADMAP_BLOCKED)
+    return fail(LMH_E_UNSUPPORTED, "lmh_decode_attn: unknown head_map %d", p->head_map);
+  const int vec = p->dtype == LMH_F32 ? 4 : 8;
+  if (p->D % vec != 0 || p->D > 256)
+    return fail(LMH_E_UNSUPPORTED, "lmh_decode_attn: head dim %d must be a multiple of %d and <= 256", p->D, vec);
+  if (p->num_splits < 0) return fail(LMH_E_SHAPE, "lmh_decode_attn: negative num_splits");
+  if (!(p->scale == p->scale)) return fail(LMH_E_SHAPE, "lmh_decode_attn: scale is NaN");
+
+  DecodeArgs a;
+  a.out = p->out; a.q = p->q; a.k = p->k_cache; a.v = p->v_cache; a.kv_len = p->kv_len;
+  a.B = p->B; a.Hq = p->Hq; a.Hkv = p->Hkv; a.Lmax = p->Lmax; a.D = p->D;
+  a.scale = p->scale; a.head_map = p->head_map;
+  a.out_f32 = (p->out_f32 != 0 || p->dtype == LMH_F32) ? 1 : 0;
+  if (all_zero(p->q_stride, 2)) { a.qs[0] = (int64_t)p->Hq * p->D; a.qs[1] = p->D; }
+  else { a.qs[0] = p->q_stride[0]; a.qs[1] = p->q_stride[1]; }
+  if (all_zero(p->o_stride, 2)) { a.os[0] = (int64_t)p->Hq * p->D; a.os[1] = p->D; }
+  else { a.os[0] = p->o_stride[0]; a.os[1] = p->o_stride[1]; }
+  auto fill3 = [&](int64_t *dst, const int64_t *src) {
+    if (all_zero(src, 3)) {
+      dst[0] = (int64_t)p->Hkv * p->Lmax * p->D; dst[1] = (int64_t)p->Lmax * p->D; dst[2] = p->D;
+    } else {
+      dst[0] = src[0]; dst[1] = src[1]; dst[2] = src[2];
+    }
+  };
+  fill3(a.ks, p->k_stride);
+  fill3(a.vs, p->v_stride);
+  // 128-bit loads: every row start must be 16-byte aligned
+  const int64_t align_elems = 16 / (int64_t)elem_bytes(p->dtype);
+  if (!aligned16(p->k_cache) || !aligned16(p->v_cache))
+    return fail(LMH_E_SHAPE, "lmh_decode_attn: cache pointers must be 16-byte aligned");
+  for (int i = 0; i < 3; i++)
+    if (a.ks[i] < 0 || a.vs[i] < 0 || a.ks[i] % align_elems != 0 || a.vs[i] % align_elems != 0)
+      return fail(LMH_E_SHAPE, "lmh_decode_attn: cache strides must be non-negative multiples of %lld elements",
+                  (long long)align_elems);
+  if (a.ks[2] < p->D || a.vs[2] < p->D) return fail(LMH_E_SHAPE, "lmh_decode_attn: cache row stride smaller than head dim");
+  if (a.qs[0] < 0 || a.qs[1] < 0 || a.os[0] < 0 || a.os[1] < 0) return fail(LMH_E_SHAPE, "lmh_decode_attn: negative stride");
+
+  a.num_splits = p->num_splits == 0 ? lmh_decode_auto_splits(p->B, p->Hkv, p->Lmax) : p->num_splits;
+  a.chunk = decode_chunk_for(p->Lmax, a.num_splits);
+  a.ws_o = nullptr;
+  a.ws_ml = nullptr;
+  if (a.num_splits > 1) {
+    const size_t need = lmh_decode_workspace_bytes(p->B, p->Hq, p->Hkv, p->Lmax, p->D, a.num_splits);
+    if (!p->workspace || p->workspace_bytes < need)
+      return fail(LMH_E_WORKSPACE, "lmh_decode_attn: workspace of %zu bytes needed for %d splits, got %zu", need,
+                  a.num_splits, p->workspace ? p->workspace_bytes : (size_t)0);
+    a.ws_o = reinterpret_cast<float *>(p->workspace);
+    a.ws_ml = a.ws_o + (size_t)p->B * p->Hq * a.num_splits * p->D;
+  }
+  return launch_decode(a, p->dtype, (hipStream_t)p->stream);
+}
+
+}  // extern "C"

@@ -1,0 +1,73 @@
+// Shared declarations of libluminal_hip.so: error reporting, launch argument blocks and the
+// kernel launchers each .hip file exports to the C-ABI layer in api.hip.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/luminal_hip.h"
+
+namespace lmh {
+
+// Records a message for lmh_last_error() and returns `code`, so call sites read
+// `return fail(LMH_E_SHAPE, "...")`.
+int fail(int code, const char *fmt, ...) __attribute__((format(printf, 2, 3)));
+int hip_fail(hipError_t e, const char *what);
+
+#define LMH_HIP_TRY(expr)                                \
+  do {                                                   \
+    hipError_t lmh_e_ = (expr);                          \
+    if (lmh_e_ != hipSuccess) return ::lmh::hip_fail(lmh_e_, #expr); \
+  } while (0)
+
+// Prefill (flash attention forward) launch arguments; strides are in elements.
+struct PrefillArgs {
+  void *out;
+  const void *q, *k, *v;
+  const int32_t *kv_len;
+  int32_t B, Hq, Hkv, Sq, Sk, D;
+  int64_t qs[3], ks[3], vs[3], os[3];
+  float scale;
+  int32_t causal;
+  int32_t head_map;
+  int32_t out_f32;  // out is fp32 whatever the input element type
+};
+
+// Decode launch arguments.
+struct DecodeArgs {
+  void *out;
+  const void *q, *k, *v;
+  const int32_t *kv_len;
+  int32_t B, Hq, Hkv, Lmax, D;
+  int64_t qs[2], os[2], ks[3], vs[3];
+  float scale;
+  int32_t head_map;
+  int32_t out_f32;  // out is fp32 whatever the input element type
+  int32_t num_splits;
+  int32_t chunk;  // keys per split
+  float *ws_o;    // [B][Hq][num_splits][D] un-normalised partial outputs
+  float *ws_ml;   // [B][Hq][num_splits][2] (running max in log2 units, partial sum)
+};
+
+__host__ __device__ inline int kv_head_of(int hq, int Hq, int Hkv, int head_map) {
+  if (Hq == Hkv) return hq;
+  return head_map == LMH_HEADMAP_BLOCKED ? hq / (Hq / Hkv) : hq % Hkv;
+}
+
+// Query head number `g` (0..G-1) of KV head `kvh`.
+__host__ __device__ inline int q_head_of(int kvh, int g, int Hq, int Hkv, int head_map) {
+  if (Hq == Hkv) return kvh;
+  return head_map == LMH_HEADMAP_BLOCKED ? kvh * (Hq / Hkv) + g : kvh + Hkv * g;
+}
+
+// Launchers: validate nothing (api.hip already did), pick an instantiation, enqueue on `stream`.
+// Return LMH_OK or LMH_E_UNSUPPORTED / LMH_E_HIP.
+bool prefill_mfma_supported(int dtype, int D);
+int launch_prefill_mfma(const PrefillArgs &a, int dtype, hipStream_t stream);
+int launch_prefill_valu(const PrefillArgs &a, int dtype, hipStream_t stream);
+int launch_decode(const DecodeArgs &a, int dtype, hipStream_t stream);
+
+// Keys per split used for a given (Lmax, num_splits); always a multiple of 64.
+int decode_chunk_for(int Lmax, int num_splits);
+
+}  // namespace lmh

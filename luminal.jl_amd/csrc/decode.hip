@@ -1,0 +1,294 @@
+// Single-token decode attention over a KV cache, flash-decoding style.
+//
+// Semantics: the cached attention of reference src/Whisper.jl:584-620 (attend over rows
+// 0 .. step_pos of a (B, H, max_seq, D) cache, plain softmax) with the GQA head sharing of
+// reference src/NN.jl:305-317, per-sequence lengths and no cache rewrite.
+//
+// The op is HBM-bound: every K and V element has to cross the memory bus once and is used for
+// 2*G flops. The design follows from that:
+//   * one workgroup per (sequence, KV head, KV split): the G query heads that share a KV head are
+//     processed together from registers, so K/V are read once per KV head, not once per query
+//     head;
+//   * a key row is covered by LPK adjacent lanes, each issuing one 128-bit load, so a wave's load
+//     instruction touches 64/LPK complete, contiguous rows;
+//   * U independent K loads and U V loads are in flight per lane before the first use;
+//   * ragged lengths: grid.x spans ceil(Lmax/chunk) splits, a workgroup whose split starts past
+//     kv_len[b] exits at once, and the merge kernel reads only the splits that exist;
+//   * split partials (running max, sum, un-normalised output) go to a caller-owned workspace and
+//     a second small kernel merges them with the log-sum-exp identity.
+#include "common.hpp"
+#include "dtypes.hpp"
+
+namespace lmh {
+namespace {
+
+constexpr int kWaves = 4;
+constexpr int kUnroll = 4;  // key steps per wave per iteration
+constexpr float kLog2e = 1.4426950408889634f;
+
+// Sum over the LPK lanes that share a key (lane bits below LPK).
+template <int LPK>
+__device__ inline float sum_within_key(float x) {
+#pragma unroll
+  for (int off = 1; off < LPK; off <<= 1) x += __shfl_xor(x, off);
+  return x;
+}
+// Reduce over the key slots of a wave (lane bits at and above LPK).
+template <int LPK>
+__device__ inline float sum_across_slots(float x) {
+#pragma unroll
+  for (int off = LPK; off < 64; off <<= 1) x += __shfl_xor(x, off);
+  return x;
+}
+template <int LPK>
+__device__ inline float max_across_slots(float x) {
+#pragma unroll
+  for (int off = LPK; off < 64; off <<= 1) x = fmaxf(x, __shfl_xor(x, off));
+  return x;
+}
+
+// E: element type; LPK: lanes per key row (power of two, LPK * E::kVec >= D); G: query heads
+// handled per workgroup (the GQA group, or a slice of it).
+template <typename E, int LPK, int G>
+__global__ __launch_bounds__(kWaves * 64) void decode_split_kernel(DecodeArgs a, int g_chunks) {
+  using raw = typename E::raw;
+  constexpr int VEC = E::kVec;
+  constexpr int KPW = 64 / LPK;                       // keys per wave per load step
+  constexpr int KEYS_PER_ITER = kWaves * kUnroll * KPW;  // keys per workgroup iteration
+
+  const int split = blockIdx.x;
+  const int kvh = blockIdx.y / g_chunks;
+  const int g0 = (blockIdx.y % g_chunks) * G;  // first group member handled here
+  const int b = blockIdx.z;
+  const int group = a.Hq / a.Hkv;
+
+  int L = a.kv_len ? a.kv_len[b] : a.Lmax;
+  L = min(max(L, 0), a.Lmax);
+  const int start = split * a.chunk;
+  if (start >= L) return;  // ragged tail: this split does not exist for sequence b
+  const int end = min(L, start + a.chunk);
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63, wave = tid >> 6;
+  const int slot = lane / LPK;
+  const int c = lane % LPK;
+  const int d0 = c * VEC;
+  const bool lane_active = d0 < a.D;  // D is a multiple of VEC (checked on the host)
+
+  // q, pre-multiplied by scale*log2(e) so that softmax runs on exp2
+  float qf[G][VEC];
+  const float qmul = a.scale * kLog2e;
+#pragma unroll
+  for (int g = 0; g < G; g++) {
+    const int gi = g0 + g;
+    const bool head_ok = gi < group;
+    const int hq = q_head_of(kvh, head_ok ? gi : 0, a.Hq, a.Hkv, a.head_map);
+    const raw *qp = reinterpret_cast<const raw *>(a.q) + b * a.qs[0] + hq * a.qs[1];
+#pragma unroll
+    for (int e = 0; e < VEC; e++) qf[g][e] = (lane_active && head_ok) ? E::ld(qp[d0 + e]) * qmul : 0.f;
+  }
+
+  const raw *kbase = reinterpret_cast<const raw *>(a.k) + b * a.ks[0] + kvh * a.ks[1] + d0;
+  const raw *vbase = reinterpret_cast<const raw *>(a.v) + b * a.vs[0] + kvh * a.vs[1] + d0;
+
+  float m[G], l[G], acc[G][VEC];
+#pragma unroll
+  for (int g = 0; g < G; g++) {
+    m[g] = -INFINITY;
+    l[g] = 0.f;
+#pragma unroll
+    for (int e = 0; e < VEC; e++) acc[g][e] = 0.f;
+  }
+
+  for (int it0 = start; it0 < end; it0 += KEYS_PER_ITER) {
+    Vec128<E> kr[kUnroll], vr[kUnroll];
+    bool valid[kUnroll];
+#pragma unroll
+    for (int u = 0; u < kUnroll; u++) {
+      const int key = it0 + (wave * kUnroll + u) * KPW + slot;
+      valid[u] = key < end;
+      if (valid[u] && lane_active) {
+        kr[u].load(kbase + (int64_t)key * a.ks[2]);
+      } else {
+        kr[u].zero();
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < kUnroll; u++) {
+      const int key = it0 + (wave * kUnroll + u) * KPW + slot;
+      if (valid[u] && lane_active) {
+        vr[u].load(vbase + (int64_t)key * a.vs[2]);
+      } else {
+        vr[u].zero();
+      }
+    }
+
+    float s[kUnroll][G];
+    float blk_max[G];
+#pragma unroll
+    for (int g = 0; g < G; g++) blk_max[g] = -INFINITY;
+#pragma unroll
+    for (int u = 0; u < kUnroll; u++) {
+      float kf[VEC];
+      kr[u].unpack(kf);
+#pragma unroll
+      for (int g = 0; g < G; g++) {
+        float dot = 0.f;
+#pragma unroll
+        for (int e = 0; e < VEC; e++) dot += qf[g][e] * kf[e];
+        dot = sum_within_key<LPK>(dot);
+        s[u][g] = valid[u] ? dot : -INFINITY;
+        blk_max[g] = fmaxf(blk_max[g], s[u][g]);
+      }
+    }
+#pragma unroll
+    for (int g = 0; g < G; g++) {
+      const float bm = max_across_slots<LPK>(blk_max[g]);
+      const float m_new = fmaxf(m[g], bm);
+      // m_new is -inf only when this wave has seen no valid key yet; then everything stays 0.
+      const float alpha = (m[g] == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(m[g] - m_new);
+      m[g] = m_new;
+      l[g] *= alpha;
+#pragma unroll
+      for (int e = 0; e < VEC; e++) acc[g][e] *= alpha;
+    }
+#pragma unroll
+    for (int u = 0; u < kUnroll; u++) {
+      float vf[VEC];
+      vr[u].unpack(vf);
+#pragma unroll
+      for (int g = 0; g < G; g++) {
+        const float p = valid[u] ? __builtin_amdgcn_exp2f(s[u][g] - m[g]) : 0.f;
+        l[g] += p;
+#pragma unroll
+        for (int e = 0; e < VEC; e++) acc[g][e] += p * vf[e];
+      }
+    }
+  }
+
+  // Merge the key slots of each wave, then the waves of the workgroup.
+  __shared__ float sm_m[kWaves][G];
+  __shared__ float sm_l[kWaves][G];
+  __shared__ float sm_acc[kWaves][G][LPK * VEC];
+#pragma unroll
+  for (int g = 0; g < G; g++) {
+    l[g] = sum_across_slots<LPK>(l[g]);
+#pragma unroll
+    for (int e = 0; e < VEC; e++) acc[g][e] = sum_across_slots<LPK>(acc[g][e]);
+    if (slot == 0) {
+#pragma unroll
+      for (int e = 0; e < VEC; e++) sm_acc[wave][g][d0 + e] = acc[g][e];
+      if (c == 0) {
+        sm_m[wave][g] = m[g];
+        sm_l[wave][g] = l[g];
+      }
+    }
+  }
+  __syncthreads();
+
+  for (int idx = tid; idx < G * a.D; idx += kWaves * 64) {
+    const int g = idx / a.D, d = idx % a.D;
+    const int gi = g0 + g;
+    if (gi >= group) continue;
+    float M = -INFINITY;
+#pragma unroll
+    for (int w = 0; w < kWaves; w++) M = fmaxf(M, sm_m[w][g]);
+    float lsum = 0.f, o = 0.f;
+#pragma unroll
+    for (int w = 0; w < kWaves; w++) {
+      const float f = (sm_m[w][g] == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(sm_m[w][g] - M);
+      lsum += sm_l[w][g] * f;
+      o += sm_acc[w][g][d] * f;
+    }
+    const int hq = q_head_of(kvh, gi, a.Hq, a.Hkv, a.head_map);
+    if (a.num_splits == 1) {
+      const int64_t off = b * a.os[0] + hq * a.os[1] + d;
+      if (a.out_f32) reinterpret_cast<float *>(a.out)[off] = o / lsum;
+      else reinterpret_cast<raw *>(a.out)[off] = E::st(o / lsum);
+    } else {
+      const int64_t row = ((int64_t)b * a.Hq + hq) * a.num_splits + split;
+      a.ws_o[row * a.D + d] = o;
+      if (d == 0) {
+        a.ws_ml[row * 2 + 0] = M;
+        a.ws_ml[row * 2 + 1] = lsum;
+      }
+    }
+  }
+}
+
+// out[b,hq,:] = sum_s o_s 2^(m_s - M) / sum_s l_s 2^(m_s - M) over the splits that exist.
+template <typename E>
+__global__ __launch_bounds__(128) void decode_merge_kernel(DecodeArgs a) {
+  using raw = typename E::raw;
+  const int hq = blockIdx.x, b = blockIdx.y;
+  int L = a.kv_len ? a.kv_len[b] : a.Lmax;
+  L = min(max(L, 0), a.Lmax);
+  const int n = (L + a.chunk - 1) / a.chunk;
+  const int64_t off = b * a.os[0] + hq * a.os[1];
+  const int64_t row0 = ((int64_t)b * a.Hq + hq) * a.num_splits;
+  float M = -INFINITY;
+  for (int s = 0; s < n; s++) M = fmaxf(M, a.ws_ml[(row0 + s) * 2]);
+  float lsum = 0.f;
+  for (int s = 0; s < n; s++) lsum += a.ws_ml[(row0 + s) * 2 + 1] * __builtin_amdgcn_exp2f(a.ws_ml[(row0 + s) * 2] - M);
+  const float inv = 1.f / lsum;
+  for (int d = threadIdx.x; d < a.D; d += blockDim.x) {
+    float o = 0.f;
+    for (int s = 0; s < n; s++) o += a.ws_o[(row0 + s) * a.D + d] * __builtin_amdgcn_exp2f(a.ws_ml[(row0 + s) * 2] - M);
+    if (a.out_f32) reinterpret_cast<float *>(a.out)[off + d] = o * inv;
+    else reinterpret_cast<raw *>(a.out)[off + d] = E::st(o * inv);
+  }
+}
+
+template <typename E, int LPK>
+int launch_for_lpk(const DecodeArgs &a, hipStream_t stream) {
+  const int group = a.Hq / a.Hkv;
+  dim3 block(kWaves * 64);
+#define LMH_DECODE_LAUNCH(GG)                                                               \
+  do {                                                                                      \
+    const int g_chunks = (group + (GG)-1) / (GG);                                           \
+    dim3 grid(a.num_splits, a.Hkv * g_chunks, a.B);                                         \
+    hipLaunchKernelGGL((decode_split_kernel<E, LPK, GG>), grid, block, 0, stream, a, g_chunks); \
+  } while (0)
+  if (group == 1) LMH_DECODE_LAUNCH(1);
+  else if (group == 2) LMH_DECODE_LAUNCH(2);
+  else if (group <= 4) LMH_DECODE_LAUNCH(4);
+  else LMH_DECODE_LAUNCH(8);
+#undef LMH_DECODE_LAUNCH
+  LMH_HIP_TRY(hipGetLastError());
+  if (a.num_splits > 1) {
+    hipLaunchKernelGGL((decode_merge_kernel<E>), dim3(a.Hq, a.B), dim3(128), 0, stream, a);
+    LMH_HIP_TRY(hipGetLastError());
+  }
+  return LMH_OK;
+}
+
+template <typename E>
+int launch_for_dtype(const DecodeArgs &a, hipStream_t stream) {
+  const int chunks = (a.D + E::kVec - 1) / E::kVec;
+  if (chunks <= 4) return launch_for_lpk<E, 4>(a, stream);
+  if (chunks <= 8) return launch_for_lpk<E, 8>(a, stream);
+  if (chunks <= 16) return launch_for_lpk<E, 16>(a, stream);
+  if (chunks <= 32) return launch_for_lpk<E, 32>(a, stream);
+  if (chunks <= 64) return launch_for_lpk<E, 64>(a, stream);
+  return fail(LMH_E_UNSUPPORTED, "decode attention: head dim %d too large", a.D);
+}
+
+}  // namespace
+
+int decode_chunk_for(int Lmax, int num_splits) {
+  if (num_splits < 1) num_splits = 1;
+  int chunk = (Lmax + num_splits - 1) / num_splits;
+  chunk = (chunk + 63) / 64 * 64;
+  return chunk < 64 ? 64 : chunk;
+}
+
+int launch_decode(const DecodeArgs &a, int dtype, hipStream_t stream) {
+  switch (dtype) {
+    case LMH_F32: return launch_for_dtype<F32>(a, stream);
+    case LMH_F16: return launch_for_dtype<F16>(a, stream);
+    case LMH_BF16: return launch_for_dtype<BF16>(a, stream);
+  }
+  return fail(LMH_E_UNSUPPORTED, "decode attention: unknown dtype %d", dtype);
+}
+
+}  // namespace lmh

@@ -1,0 +1,89 @@
+// Element types of the attention tensors and their conversion to/from the fp32 the kernels
+// accumulate in.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace lmh {
+
+typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
+typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x4_t __attribute__((ext_vector_type(4)));
+typedef float floatx16_t __attribute__((ext_vector_type(16)));
+typedef float floatx4_t __attribute__((ext_vector_type(4)));
+typedef short shortx4_t __attribute__((ext_vector_type(4)));
+
+__device__ inline float bf16_bits_to_f32(uint32_t bits16) { return __uint_as_float(bits16 << 16); }
+
+// round-to-nearest-even, NaN kept quiet
+__device__ inline uint16_t f32_to_bf16_bits(float x) {
+  uint32_t u = __float_as_uint(x);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x40u);
+  u += 0x7fffu + ((u >> 16) & 1u);
+  return (uint16_t)(u >> 16);
+}
+
+struct F32 {
+  using raw = float;
+  static constexpr int kVec = 4;  // elements per 128-bit access
+  __device__ static float ld(raw x) { return x; }
+  __device__ static raw st(float x) { return x; }
+};
+struct F16 {
+  using raw = _Float16;
+  static constexpr int kVec = 8;
+  __device__ static float ld(raw x) { return (float)x; }
+  __device__ static raw st(float x) { return (_Float16)x; }
+};
+struct BF16 {
+  using raw = uint16_t;
+  static constexpr int kVec = 8;
+  __device__ static float ld(raw x) { return bf16_bits_to_f32(x); }
+  __device__ static raw st(float x) { return f32_to_bf16_bits(x); }
+};
+
+// Unpack one 128-bit global load into fp32 lanes.
+template <typename E>
+struct Vec128;
+
+template <>
+struct Vec128<F32> {
+  float4 r;
+  __device__ void load(const void *p) { r = *reinterpret_cast<const float4 *>(p); }
+  __device__ void zero() { r = make_float4(0.f, 0.f, 0.f, 0.f); }
+  __device__ void unpack(float *f) const { f[0] = r.x; f[1] = r.y; f[2] = r.z; f[3] = r.w; }
+};
+template <>
+struct Vec128<F16> {
+  uint4 r;
+  __device__ void load(const void *p) { r = *reinterpret_cast<const uint4 *>(p); }
+  __device__ void zero() { r = make_uint4(0, 0, 0, 0); }
+  __device__ void unpack(float *f) const {
+    const uint32_t w[4] = {r.x, r.y, r.z, r.w};
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+      h2 h = __builtin_bit_cast(h2, w[i]);
+      f[2 * i] = (float)h[0];
+      f[2 * i + 1] = (float)h[1];
+    }
+  }
+};
+template <>
+struct Vec128<BF16> {
+  uint4 r;
+  __device__ void load(const void *p) { r = *reinterpret_cast<const uint4 *>(p); }
+  __device__ void zero() { r = make_uint4(0, 0, 0, 0); }
+  __device__ void unpack(float *f) const {
+    const uint32_t w[4] = {r.x, r.y, r.z, r.w};
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      f[2 * i] = __uint_as_float(w[i] << 16);
+      f[2 * i + 1] = __uint_as_float(w[i] & 0xffff0000u);
+    }
+  }
+};
+
+}  // namespace lmh

@@ -1,0 +1,298 @@
+// Flash attention forward on the gfx950 matrix cores (fp16 / bf16 in, fp32 accumulate).
+//
+// Same mathematics as flash_attn_cpu (reference src/Execution.jl:453-479) — online softmax with a
+// running max m, running sum l and an un-normalised output row — evaluated 64 keys at a time for
+// 128 query rows per workgroup instead of one (i, j) pair at a time.
+//
+// Tiling (wave64, v_mfma_f32_32x32x16):
+//   * workgroup = 4 waves = 128 query rows of one (b, hq); each wave owns 32 query rows and keeps
+//     their Q fragments in registers for the whole kernel;
+//   * the scores are computed TRANSPOSED, S^T = K Q^T (M = keys, N = queries). In the MFMA
+//     accumulator layout a lane then holds one query column (n = lane % 32) and 16 of the 32 keys
+//     of a block, so the softmax statistics (max, sum, rescale factor) are per-lane scalars and
+//     the only cross-lane traffic is one exchange with lane ^ 32;
+//   * the same registers, converted to half precision, are directly the B operand of the second
+//     product O^T = V^T P^T (M = head dim, N = queries, contraction over keys), so P never
+//     touches LDS;
+//   * K and V tiles (64 keys) are staged row-major in LDS; the K fragment is a plain 128-bit LDS
+//     read (contraction over the contiguous head dim), the V^T fragment uses the gfx950 transposing
+//     LDS read ds_read_b64_tr_b16, which hands each lane 4 consecutive keys of its head-dim column;
+//   * causal: key tiles beyond the workgroup's last query are never loaded, a wave skips tiles (and
+//     32-key blocks) that lie entirely above its diagonal, and only diagonal tiles pay for masking;
+//   * blockIdx -> work mapping keeps all query tiles of a head on one XCD (private L2) and, for
+//     causal, issues the long rows first.
+#include "common.hpp"
+#include "dtypes.hpp"
+
+namespace lmh {
+namespace {
+
+constexpr int BM = 128;  // query rows per workgroup
+constexpr int BN = 64;   // keys per tile
+constexpr int kPad = 8;  // LDS row padding in elements (16 B): spreads rows over the banks
+constexpr float kLog2e = 1.4426950408889634f;
+
+typedef short shortx8_t __attribute__((ext_vector_type(8)));
+typedef __attribute__((address_space(3))) shortx4_t lds_shortx4_t;
+
+struct MfmaF16 {
+  using vec8 = half8_t;
+  __device__ static floatx16_t mfma(vec8 a, vec8 b, floatx16_t c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+  }
+  __device__ static uint16_t cvt_bits(float x) { return __builtin_bit_cast(uint16_t, (_Float16)x); }
+  __device__ static _Float16 cvt(float x) { return (_Float16)x; }
+};
+struct MfmaBF16 {
+  using vec8 = bf16x8_t;
+  __device__ static floatx16_t mfma(vec8 a, vec8 b, floatx16_t c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+  }
+  __device__ static uint16_t cvt_bits(float x) { return f32_to_bf16_bits(x); }
+  __device__ static __bf16 cvt(float x) { return (__bf16)x; }
+};
+
+template <typename MT, int D, bool CAUSAL>
+__global__ __launch_bounds__(256, 2) void prefill_mfma_kernel(PrefillArgs a, int n_q_tiles, int n_bh_groups) {
+  using vec8 = typename MT::vec8;
+  constexpr int KS = D / 16;       // k-steps of the S^T product
+  constexpr int DB = D / 32;       // 32-row blocks of O^T
+  constexpr int CPR = D / 8;       // 16-byte chunks per K/V row
+  constexpr int CH = BN * CPR / 256;  // chunks per thread per tile
+  constexpr int LDW = D + kPad;    // LDS row stride in elements
+
+  __shared__ __attribute__((aligned(16))) uint16_t Ks[BN * LDW];
+  __shared__ __attribute__((aligned(16))) uint16_t Vs[BN * LDW];
+
+  // ---- which (b, hq, query tile) this workgroup owns ----
+  const int bid = blockIdx.x;
+  const int xcd = bid & 7;
+  const int idx = bid >> 3;
+  const int tile_rank = idx / n_bh_groups;
+  const int bh = (idx % n_bh_groups) * 8 + xcd;
+  if (bh >= a.B * a.Hq) return;
+  const int b = bh / a.Hq, hq = bh % a.Hq;
+  const int kvh = kv_head_of(hq, a.Hq, a.Hkv, a.head_map);
+  const int q_tile = CAUSAL ? (n_q_tiles - 1 - tile_rank) : tile_rank;
+  const int q0 = q_tile * BM;
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63, wave = tid >> 6;
+  const int n = lane & 31, g = lane >> 5;
+  const int wave_q_lo = q0 + wave * 32;
+  const int wave_q_hi = wave_q_lo + 31;
+  const int qi = wave_q_lo + n;
+
+  int n_keys = a.kv_len ? a.kv_len[b] : a.Sk;
+  n_keys = min(max(n_keys, 0), a.Sk);
+  int k_end = n_keys;
+  if (CAUSAL) k_end = min(k_end, q0 + BM);
+  const int n_kv_tiles = (k_end + BN - 1) / BN;
+
+  const uint16_t *qp = reinterpret_cast<const uint16_t *>(a.q) + b * a.qs[0] + hq * a.qs[1];
+  const uint16_t *kp = reinterpret_cast<const uint16_t *>(a.k) + b * a.ks[0] + kvh * a.ks[1];
+  const uint16_t *vp = reinterpret_cast<const uint16_t *>(a.v) + b * a.vs[0] + kvh * a.vs[1];
+
+  // ---- Q fragments: B operand of S^T = K Q^T; lane (n, g) holds q[qi][16*ks + 8*g .. +7] ----
+  vec8 qreg[KS];
+#pragma unroll
+  for (int ks = 0; ks < KS; ks++) {
+    uint4 raw = make_uint4(0, 0, 0, 0);
+    if (qi < a.Sq) raw = *reinterpret_cast<const uint4 *>(qp + (int64_t)qi * a.qs[2] + 16 * ks + 8 * g);
+    qreg[ks] = __builtin_bit_cast(vec8, raw);
+  }
+
+  floatx16_t oacc[DB];
+#pragma unroll
+  for (int db = 0; db < DB; db++)
+#pragma unroll
+    for (int i = 0; i < 16; i++) oacc[db][i] = 0.f;
+  float m_i = -INFINITY;  // running max of the raw (unscaled) scores of query qi
+  float l_i = 0.f;        // this lane's half of the running sum
+  const float c = a.scale * kLog2e;
+
+  // ---- tile staging: global -> registers (prefetch) -> LDS ----
+  uint4 kreg[CH], vreg[CH];
+  auto load_tile = [&](int kt) {
+    const int k0 = kt * BN;
+#pragma unroll
+    for (int r = 0; r < CH; r++) {
+      const int id = tid + 256 * r;
+      const int row = id / CPR, col = id % CPR;
+      const int key = k0 + row;
+      kreg[r] = make_uint4(0, 0, 0, 0);
+      vreg[r] = make_uint4(0, 0, 0, 0);
+      if (key < n_keys) {
+        kreg[r] = *reinterpret_cast<const uint4 *>(kp + (int64_t)key * a.ks[2] + col * 8);
+        vreg[r] = *reinterpret_cast<const uint4 *>(vp + (int64_t)key * a.vs[2] + col * 8);
+      }
+    }
+  };
+  auto store_tile = [&]() {
+#pragma unroll
+    for (int r = 0; r < CH; r++) {
+      const int id = tid + 256 * r;
+      const int row = id / CPR, col = id % CPR;
+      *reinterpret_cast<uint4 *>(&Ks[row * LDW + col * 8]) = kreg[r];
+      *reinterpret_cast<uint4 *>(&Vs[row * LDW + col * 8]) = vreg[r];
+    }
+  };
+
+  // lane-constant pieces of the LDS addresses
+  const int k_frag_off = n * LDW + 8 * g;  // + kb*32*LDW + 16*ks
+  // transposing V read: within each 16-lane block, lane i supplies row (i / 4) and 4-column group
+  // (i % 4) of a 4-key x 16-column patch and receives the 4 keys of column i.
+  const int i16 = lane & 15;
+  const int v_frag_off = (4 * g + (i16 >> 2)) * LDW + 16 * ((lane >> 4) & 1) + 4 * (i16 & 3);
+  // + (kb*32 + 16*t [+8]) * LDW + db*32
+
+  if (n_kv_tiles > 0) load_tile(0);
+
+  for (int kt = 0; kt < n_kv_tiles; kt++) {
+    __syncthreads();  // every wave is done reading the previous tile
+    store_tile();
+    __syncthreads();
+    if (kt + 1 < n_kv_tiles) load_tile(kt + 1);  // in flight while this tile is computed
+
+    const int k0 = kt * BN;
+    if (CAUSAL && k0 > wave_q_hi) continue;  // whole tile above this wave's diagonal
+    const bool blk1_active = !(CAUSAL && k0 + 32 > wave_q_hi);
+
+    // ---- S^T = K Q^T for two 32-key blocks ----
+    floatx16_t sacc[2];
+#pragma unroll
+    for (int kb = 0; kb < 2; kb++) {
+#pragma unroll
+      for (int i = 0; i < 16; i++) sacc[kb][i] = 0.f;
+      if (kb == 0 || blk1_active) {
+#pragma unroll
+        for (int ks = 0; ks < KS; ks++) {
+          const vec8 kf = *reinterpret_cast<const vec8 *>(&Ks[k_frag_off + kb * 32 * LDW + 16 * ks]);
+          sacc[kb] = MT::mfma(kf, qreg[ks], sacc[kb]);
+        }
+      }
+    }
+
+    // ---- masking (diagonal tiles and the ragged last tile only) ----
+    const bool need_mask = (k0 + BN > n_keys) || (CAUSAL && k0 + BN - 1 > wave_q_lo);
+    if (need_mask) {
+#pragma unroll
+      for (int kb = 0; kb < 2; kb++)
+#pragma unroll
+        for (int i = 0; i < 16; i++) {
+          const int key = k0 + kb * 32 + 8 * (i >> 2) + 4 * g + (i & 3);
+          if (key >= n_keys || (CAUSAL && key > qi)) sacc[kb][i] = -INFINITY;
+        }
+    }
+
+    // ---- online softmax; all statistics are per lane (one query column) ----
+    float mx = sacc[0][0];
+#pragma unroll
+    for (int kb = 0; kb < 2; kb++)
+#pragma unroll
+      for (int i = 0; i < 16; i++) mx = fmaxf(mx, sacc[kb][i]);
+    mx = fmaxf(mx, __shfl_xor(mx, 32));
+    const float m_new = fmaxf(m_i, mx);  // finite: key 0 is visible to every query
+    const float alpha = __builtin_amdgcn_exp2f((m_i - m_new) * c);
+    const float mc = m_new * c;
+    m_i = m_new;
+    float psum = 0.f;
+#pragma unroll
+    for (int kb = 0; kb < 2; kb++)
+#pragma unroll
+      for (int i = 0; i < 16; i++) {
+        const float p = __builtin_amdgcn_exp2f(sacc[kb][i] * c - mc);
+        sacc[kb][i] = p;
+        psum += p;
+      }
+    l_i = l_i * alpha + psum;
+#pragma unroll
+    for (int db = 0; db < DB; db++)
+#pragma unroll
+      for (int i = 0; i < 16; i++) oacc[db][i] *= alpha;
+
+    // ---- O^T += V^T P^T ----
+#pragma unroll
+    for (int kb = 0; kb < 2; kb++) {
+      if (kb == 1 && !blk1_active) continue;
+#pragma unroll
+      for (int t = 0; t < 2; t++) {
+        vec8 pf;
+#pragma unroll
+        for (int e = 0; e < 8; e++) pf[e] = MT::cvt(sacc[kb][8 * t + e]);
+#pragma unroll
+        for (int db = 0; db < DB; db++) {
+          const uint16_t *vaddr = &Vs[v_frag_off + (kb * 32 + 16 * t) * LDW + db * 32];
+          const shortx4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_shortx4_t *)(vaddr));
+          const shortx4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_shortx4_t *)(vaddr + 8 * LDW));
+          const shortx8_t v8 = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+          oacc[db] = MT::mfma(__builtin_bit_cast(vec8, v8), pf, oacc[db]);
+        }
+      }
+    }
+  }
+
+  // ---- epilogue: out[qi][d] = O^T[d][qi] / l ----
+  const float l_tot = l_i + __shfl_xor(l_i, 32);
+  const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
+  if (qi < a.Sq) {
+    const int64_t off = b * a.os[0] + hq * a.os[1] + (int64_t)qi * a.os[2];
+    uint16_t *op = reinterpret_cast<uint16_t *>(a.out) + off;
+    float *op32 = reinterpret_cast<float *>(a.out) + off;
+#pragma unroll
+    for (int db = 0; db < DB; db++)
+#pragma unroll
+      for (int i4 = 0; i4 < 4; i4++) {
+        const int d = db * 32 + 8 * i4 + 4 * g;
+        if (a.out_f32) {
+          *reinterpret_cast<float4 *>(op32 + d) =
+              make_float4(oacc[db][4 * i4 + 0] * inv, oacc[db][4 * i4 + 1] * inv, oacc[db][4 * i4 + 2] * inv,
+                          oacc[db][4 * i4 + 3] * inv);
+          continue;
+        }
+        uint2 packed;
+        packed.x = (uint32_t)MT::cvt_bits(oacc[db][4 * i4 + 0] * inv) |
+                   ((uint32_t)MT::cvt_bits(oacc[db][4 * i4 + 1] * inv) << 16);
+        packed.y = (uint32_t)MT::cvt_bits(oacc[db][4 * i4 + 2] * inv) |
+                   ((uint32_t)MT::cvt_bits(oacc[db][4 * i4 + 3] * inv) << 16);
+        *reinterpret_cast<uint2 *>(op + d) = packed;
+      }
+  }
+}
+
+template <typename MT, int D>
+int launch_for_d(const PrefillArgs &a, hipStream_t stream) {
+  const int n_q_tiles = (a.Sq + BM - 1) / BM;
+  const int n_bh_groups = (a.B * a.Hq + 7) / 8;
+  dim3 grid(8 * n_bh_groups * n_q_tiles), block(256);
+  if (a.causal)
+    hipLaunchKernelGGL((prefill_mfma_kernel<MT, D, true>), grid, block, 0, stream, a, n_q_tiles, n_bh_groups);
+  else
+    hipLaunchKernelGGL((prefill_mfma_kernel<MT, D, false>), grid, block, 0, stream, a, n_q_tiles, n_bh_groups);
+  LMH_HIP_TRY(hipGetLastError());
+  return LMH_OK;
+}
+
+template <typename MT>
+int launch_for_type(const PrefillArgs &a, hipStream_t stream) {
+  switch (a.D) {
+    case 64: return launch_for_d<MT, 64>(a, stream);
+    case 96: return launch_for_d<MT, 96>(a, stream);
+    case 128: return launch_for_d<MT, 128>(a, stream);
+  }
+  return fail(LMH_E_UNSUPPORTED, "MFMA flash attention: head dim %d not tiled", a.D);
+}
+
+}  // namespace
+
+bool prefill_mfma_supported(int dtype, int D) {
+  return (dtype == LMH_F16 || dtype == LMH_BF16) && (D == 64 || D == 96 || D == 128);
+}
+
+int launch_prefill_mfma(const PrefillArgs &a, int dtype, hipStream_t stream) {
+  if (dtype == LMH_F16) return launch_for_type<MfmaF16>(a, stream);
+  if (dtype == LMH_BF16) return launch_for_type<MfmaBF16>(a, stream);
+  return fail(LMH_E_UNSUPPORTED, "MFMA flash attention: dtype %d has no matrix-core path", dtype);
+}
+
+}  // namespace lmh

@@ -1,0 +1,447 @@
+"""Host-side mirror of the slice of Luminal.jl's API that the attention hot path goes through.
+
+The reference's host is Julia; its toolchain is not available where this backend is built and
+tested, so the same interface is mirrored here in Python over the same C ABI the Julia glue
+(julia/LuminalHIP.jl) calls. Names, argument meaning and error behaviour follow the reference:
+
+  Graph, GraphTensor, tensor, add_op             reference src/Graph.jl:4-82
+  FlashAttentionOp(scale, causal)                reference src/Ops.jl:104-107
+  flash_attention(q, k, v; scale, causal)        reference src/HighLevelOps.jl:377-388
+  execute_op / execute_op_inplace                reference src/Execution.jl:252-255, :565-578
+  execute(graph, ids, inputs, device)            reference src/Execution.jl:620-670
+  compile(graph) -> CompiledGraph(inputs, dev)   reference src/Compiler.jl:75-100, :181-255
+  HIPDevice, get_device, to_device, from_device  reference src/Device.jl:9-16, :31-74, :82-105
+
+Additions the reference has only as un-fused subgraphs:
+  DecodeAttentionOp / decode_attention           reference src/Whisper.jl:584-620, :628-645
+  GQA (Hkv < Hq) inside the fused ops            reference src/NN.jl:305-317, :362-366
+
+Arrays here are row-major [B, H, S, D] (numpy order), which is the layout the C ABI takes. There
+is no CPU execution path in this backend: running an attention op on host arrays raises.
+"""
+import ctypes
+import math
+
+import numpy as np
+
+from . import binding
+from .binding import HEADMAP_BLOCKED, HEADMAP_INTERLEAVED, LuminalHipError  # noqa: F401
+
+
+# ---------------------------------------------------------------------------------------------
+# element types
+# ---------------------------------------------------------------------------------------------
+def f32_to_bf16_bits(x):
+    """fp32 array -> uint16 bf16 bit patterns, round-to-nearest-even."""
+    u = np.ascontiguousarray(x, dtype=np.float32).view(np.uint32)
+    nan = (u & np.uint32(0x7FFFFFFF)) > np.uint32(0x7F800000)
+    r = (u + np.uint32(0x7FFF) + ((u >> np.uint32(16)) & np.uint32(1))) >> np.uint32(16)
+    r = np.where(nan, (u >> np.uint32(16)) | np.uint32(0x40), r)
+    return r.astype(np.uint16)
+
+
+def bf16_bits_to_f32(bits):
+    return (np.ascontiguousarray(bits, dtype=np.uint16).astype(np.uint32) << np.uint32(16)).view(np.float32)
+
+
+def encode(x, dtype):
+    """fp32 numpy array -> the byte representation of `dtype` ('f32' | 'f16' | 'bf16')."""
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    if dtype == "f32":
+        return x
+    if dtype == "f16":
+        return x.astype(np.float16)
+    if dtype == "bf16":
+        return f32_to_bf16_bits(x)
+    raise ValueError("unknown dtype %r" % (dtype,))
+
+
+def decode(raw, dtype):
+    if dtype == "f32":
+        return np.asarray(raw, dtype=np.float32)
+    if dtype == "f16":
+        return np.asarray(raw).view(np.float16).astype(np.float32)
+    if dtype == "bf16":
+        return bf16_bits_to_f32(np.asarray(raw).view(np.uint16))
+    raise ValueError("unknown dtype %r" % (dtype,))
+
+
+_NP_STORAGE = {"f32": np.float32, "f16": np.float16, "bf16": np.uint16, "i32": np.int32}
+
+
+# ---------------------------------------------------------------------------------------------
+# devices and arrays
+# ---------------------------------------------------------------------------------------------
+class AbstractDevice:
+    pass
+
+
+class CPUDevice(AbstractDevice):
+    def __repr__(self):
+        return "CPUDevice()"
+
+
+class HIPDevice(AbstractDevice):
+    """An MI355X reached through libluminal_hip.so (not through AMDGPU.jl-style array packages)."""
+
+    def __init__(self, index=0):
+        self.index = index
+
+    def __repr__(self):
+        return "HIPDevice(%d)" % self.index
+
+
+_initialised = set()
+
+
+def get_device():
+    """Best available device; same try-then-fall-through shape as the reference's get_device()
+    (health check = lmh_init's tiny allocation). Falls through to CPUDevice, on which the attention
+    ops refuse to run."""
+    try:
+        if binding.device_count() > 0:
+            binding.init(0)
+            _initialised.add(0)
+            return HIPDevice(0)
+    except (LuminalHipError, RuntimeError, OSError):
+        pass
+    return CPUDevice()
+
+
+def _ensure_init(device):
+    if device.index not in _initialised:
+        binding.init(device.index)
+        _initialised.add(device.index)
+
+
+class HipArray:
+    """Device buffer + shape + element type; frees its memory when collected (the Julia glue's
+    HipArray does it in a finalizer)."""
+
+    def __init__(self, shape, dtype="f32", device=None):
+        self.shape = tuple(int(s) for s in shape)
+        self.dtype = dtype
+        self.device = device or HIPDevice(0)
+        _ensure_init(self.device)
+        itemsize = 4 if dtype == "i32" else binding.DTYPE_BYTES[dtype]
+        self.nbytes = int(np.prod(self.shape, dtype=np.int64)) * itemsize
+        self.ptr = binding.malloc(max(self.nbytes, 1))
+
+    @property
+    def size(self):
+        return int(np.prod(self.shape, dtype=np.int64))
+
+    def copy_from_host(self, arr):
+        """arr: fp32 values (converted to this array's dtype) or already-encoded storage."""
+        if self.dtype == "i32":
+            raw = np.ascontiguousarray(arr, dtype=np.int32)
+        elif np.asarray(arr).dtype == _NP_STORAGE[self.dtype] and self.dtype != "f32":
+            raw = np.ascontiguousarray(arr)
+        else:
+            raw = encode(arr, self.dtype)
+        if raw.size != self.size:
+            raise ValueError("Input length mismatch: expected %d, got %d" % (self.size, raw.size))
+        binding.memcpy_h2d(self.ptr, raw.ctypes.data, self.nbytes)
+        return self
+
+    def to_host_raw(self):
+        raw = np.empty(self.shape, dtype=_NP_STORAGE[self.dtype])
+        binding.memcpy_d2h(raw.ctypes.data, self.ptr, self.nbytes)
+        return raw
+
+    def to_host(self):
+        raw = self.to_host_raw()
+        return raw if self.dtype == "i32" else decode(raw, self.dtype).reshape(self.shape)
+
+    def fill_bytes(self, value):
+        binding.memset(self.ptr, value, self.nbytes)
+        return self
+
+    def free(self):
+        if getattr(self, "ptr", 0):
+            binding.free(self.ptr)
+            self.ptr = 0
+
+    def __del__(self):
+        try:
+            self.free()
+        except Exception:
+            pass
+
+
+def to_device(data, device, dtype="f32"):
+    """Move data to `device`; dicts are mapped value-wise (reference src/Device.jl:82-96)."""
+    if isinstance(data, dict):
+        return {k: to_device(v, device, dtype) for k, v in data.items()}
+    if isinstance(device, HIPDevice):
+        if isinstance(data, HipArray):
+            return data
+        if isinstance(data, np.ndarray):
+            if data.dtype == np.int32:
+                return HipArray(data.shape, "i32", device).copy_from_host(data)
+            return HipArray(data.shape, dtype, device).copy_from_host(data)
+    return data
+
+
+def from_device(data):
+    """Move data back to the host (reference src/Device.jl:103-105)."""
+    if isinstance(data, HipArray):
+        return data.to_host()
+    return data
+
+
+# ---------------------------------------------------------------------------------------------
+# graph IR (only what the attention path touches)
+# ---------------------------------------------------------------------------------------------
+class Op:
+    pass
+
+
+class InputTensor(Op):
+    name = "InputTensor"
+
+
+class FlashAttentionOp(Op):
+    """Fused flash attention node (reference src/Ops.jl:104-107), plus the GQA head map."""
+
+    def __init__(self, scale, causal, head_map=HEADMAP_INTERLEAVED, out_dtype=None):
+        self.scale = float(np.float32(scale))
+        self.causal = bool(causal)
+        self.head_map = head_map
+        self.out_dtype = out_dtype  # None = q's element type; "f32" = full-precision result
+
+
+class DecodeAttentionOp(Op):
+    """Single-token attention over a KV cache; inputs (q, k_cache, v_cache, kv_len)."""
+
+    def __init__(self, scale, head_map=HEADMAP_INTERLEAVED, num_splits=0, out_dtype=None):
+        self.scale = float(np.float32(scale))
+        self.head_map = head_map
+        self.num_splits = num_splits
+        self.out_dtype = out_dtype
+
+
+class Node:
+    def __init__(self, op, inputs):
+        self.op = op
+        self.inputs = inputs  # list of (node_id, output_index, shape)
+
+
+class GraphTensor:
+    def __init__(self, id, shape, graph_ref):
+        self.id = id
+        self.shape = tuple(shape)
+        self.graph_ref = graph_ref
+
+
+class Graph:
+    def __init__(self):
+        self.nodes = []
+        self.shapes = []
+        self.dtypes = []
+        self.tensors = {}
+
+
+def add_op(graph, op, inputs, output_shape, dtype="f32"):
+    graph.nodes.append(Node(op, inputs))
+    graph.shapes.append(tuple(output_shape))
+    graph.dtypes.append(dtype)
+    return GraphTensor(len(graph.nodes) - 1, output_shape, graph)
+
+
+def tensor(graph, shape, dtype="f32"):
+    """Define a new input tensor on the graph (reference src/Graph.jl:56-61)."""
+    if isinstance(shape, np.ndarray):
+        shape = shape.shape
+    return add_op(graph, InputTensor(), [], tuple(shape), dtype)
+
+
+def flash_attention(q, k, v, scale=None, causal=False, head_map=HEADMAP_INTERLEAVED, out_dtype=None):
+    """q, k, v: (Batch, Head, Seq, HeadDim). Output has q's shape; scale defaults to 1/sqrt(D)
+    computed in fp32 (reference src/HighLevelOps.jl:377-388)."""
+    if scale is None:
+        scale = np.float32(1.0) / np.sqrt(np.float32(q.shape[-1]))
+    inputs = [(q.id, 0, q.shape), (k.id, 0, k.shape), (v.id, 0, v.shape)]
+    return add_op(q.graph_ref, FlashAttentionOp(np.float32(scale), causal, head_map, out_dtype), inputs, q.shape,
+                  out_dtype or q.graph_ref.dtypes[q.id])
+
+
+def decode_attention(q, k_cache, v_cache, kv_len, scale=None, head_map=HEADMAP_INTERLEAVED, num_splits=0,
+                     out_dtype=None):
+    """q: (Batch, Head, HeadDim); caches: (Batch, KVHead, MaxSeq, HeadDim); kv_len: (Batch,) int32."""
+    if scale is None:
+        scale = np.float32(1.0) / np.sqrt(np.float32(q.shape[-1]))
+    inputs = [(q.id, 0, q.shape), (k_cache.id, 0, k_cache.shape), (v_cache.id, 0, v_cache.shape),
+              (kv_len.id, 0, kv_len.shape)]
+    return add_op(q.graph_ref, DecodeAttentionOp(np.float32(scale), head_map, num_splits, out_dtype), inputs, q.shape,
+                  out_dtype or q.graph_ref.dtypes[q.id])
+
+
+# ---------------------------------------------------------------------------------------------
+# execution
+# ---------------------------------------------------------------------------------------------
+def _require_hip(*arrays):
+    for a in arrays:
+        if not isinstance(a, HipArray):
+            raise TypeError("attention ops run on HipArray inputs only; this backend has no CPU path "
+                            "(got %s)" % type(a).__name__)
+
+
+class _Workspaces:
+    """Decode split-KV scratch, grown on demand and reused (caller-owned from the library's view)."""
+
+    def __init__(self):
+        self.buf = None
+
+    def get(self, nbytes, device):
+        if nbytes == 0:
+            return 0, 0
+        if self.buf is None or self.buf.nbytes < nbytes:
+            if self.buf is not None:
+                binding.sync()
+                self.buf.free()
+            self.buf = HipArray(((nbytes + 3) // 4,), "f32", device)
+        return self.buf.ptr, self.buf.nbytes
+
+
+_workspaces = _Workspaces()
+
+
+def execute_op_inplace(out, op, *inputs, stream=None):
+    """execute_op!(out, op, inputs...) (reference src/Execution.jl:565-578) for the two attention ops."""
+    if isinstance(op, FlashAttentionOp):
+        q, k, v = inputs[:3]
+        kv_len = inputs[3] if len(inputs) > 3 else None
+        _require_hip(out, q, k, v)
+        if len(q.shape) != 4 or len(k.shape) != 4 or k.shape != v.shape:
+            raise ValueError("flash attention expects q (B,H,S,D) and k, v (B,Hkv,Sk,D); got %s %s %s" %
+                             (q.shape, k.shape, v.shape))
+        if out.shape != q.shape:
+            raise ValueError("output shape %s differs from q shape %s" % (out.shape, q.shape))
+        if not (q.dtype == k.dtype == v.dtype) or out.dtype not in (q.dtype, "f32"):
+            raise ValueError("q, k, v must share one element type; out has that type or f32")
+        if k.shape[0] != q.shape[0] or k.shape[3] != q.shape[3]:
+            raise ValueError("k/v batch or head dim differ from q's")
+        p = binding.AttnParams()
+        p.out, p.q, p.k, p.v = out.ptr, q.ptr, k.ptr, v.ptr
+        p.kv_len = kv_len.ptr if kv_len is not None else None
+        p.B, p.Hq, p.Sq, p.D = q.shape
+        p.Hkv, p.Sk = k.shape[1], k.shape[2]
+        p.dtype = binding.DTYPE_CODES[q.dtype]
+        p.scale, p.causal, p.head_map = op.scale, int(op.causal), op.head_map
+        p.out_f32 = int(out.dtype == "f32")
+        p.stream = stream
+        binding.flash_attn_fwd(p)
+        return out
+    if isinstance(op, DecodeAttentionOp):
+        q, kc, vc = inputs[:3]
+        kv_len = inputs[3] if len(inputs) > 3 else None
+        _require_hip(out, q, kc, vc)
+        if len(q.shape) != 3 or len(kc.shape) != 4 or kc.shape != vc.shape:
+            raise ValueError("decode attention expects q (B,H,D) and caches (B,Hkv,Lmax,D); got %s %s %s" %
+                             (q.shape, kc.shape, vc.shape))
+        if out.shape != q.shape:
+            raise ValueError("output shape %s differs from q shape %s" % (out.shape, q.shape))
+        if not (q.dtype == kc.dtype == vc.dtype) or out.dtype not in (q.dtype, "f32"):
+            raise ValueError("q and the caches must share one element type; out has that type or f32")
+        p = binding.DecodeParams()
+        p.out, p.q, p.k_cache, p.v_cache = out.ptr, q.ptr, kc.ptr, vc.ptr
+        p.kv_len = kv_len.ptr if kv_len is not None else None
+        p.B, p.Hq, p.D = q.shape
+        p.Hkv, p.Lmax = kc.shape[1], kc.shape[2]
+        p.dtype = binding.DTYPE_CODES[q.dtype]
+        p.scale, p.head_map = op.scale, op.head_map
+        p.out_f32 = int(out.dtype == "f32")
+        p.num_splits = op.num_splits or binding.decode_auto_splits(p.B, p.Hkv, p.Lmax)
+        need = binding.decode_workspace_bytes(p.B, p.Hq, p.Hkv, p.Lmax, p.D, p.num_splits)
+        p.workspace, p.workspace_bytes = _workspaces.get(need, q.device)
+        p.stream = stream
+        binding.decode_attn(p)
+        return out
+    raise TypeError("no HIP kernel for op %s" % type(op).__name__)
+
+
+def execute_op(op, *inputs):
+    """Allocating form: out = similar(q); execute_op!(out, ...) (reference src/Execution.jl:252-255)."""
+    q = inputs[0]
+    _require_hip(q)
+    out = HipArray(q.shape, getattr(op, "out_dtype", None) or q.dtype, q.device)
+    return execute_op_inplace(out, op, *inputs)
+
+
+def execute(graph, output_ids, initial_inputs, device=None, dtype=None):
+    """Interpreter (reference src/Execution.jl:620-670): upload inputs, run nodes in order, download
+    the requested outputs. `output_ids` may be one id or a list."""
+    device = device or get_device()
+    single = isinstance(output_ids, int)
+    ids = [output_ids] if single else list(output_ids)
+    results = {}
+    for k, v in initial_inputs.items():
+        results[k] = to_device(v, device, dtype or graph.dtypes[k])
+    for (node_id, out_idx), data in graph.tensors.items():
+        if node_id not in results and out_idx == 0:
+            results[node_id] = to_device(data, device, graph.dtypes[node_id])
+    for node_id, node in enumerate(graph.nodes):
+        if node_id in results:
+            continue
+        if isinstance(node.op, InputTensor):
+            raise KeyError("no value given for input tensor %d" % node_id)
+        results[node_id] = execute_op(node.op, *[results[i] for (i, _, _) in node.inputs])
+    final = {i: from_device(results[i]) for i in ids}
+    return final[ids[0]] if single else final
+
+
+class CompiledGraph:
+    """Pre-allocated node buffers + a step list (reference src/Compiler.jl:75-100). Calling it copies the
+    inputs into their buffers, runs the steps in place and returns the buffer list; nothing is
+    allocated per call."""
+
+    def __init__(self, steps, results):
+        self.steps = steps
+        self.results = results
+
+    def __call__(self, inputs, device=None):
+        for k, v in inputs.items():
+            if k >= len(self.results) or self.results[k] is None:
+                raise KeyError("Input node %d not found in compiled graph results." % k)
+            if isinstance(v, HipArray):
+                if v.nbytes != self.results[k].nbytes:
+                    raise ValueError("Input length mismatch for node %d" % k)
+                binding.memcpy_d2d(self.results[k].ptr, v.ptr, v.nbytes)
+            else:
+                self.results[k].copy_from_host(v)
+        for step in self.steps:
+            step()
+        return self.results
+
+
+def compile(graph, device=None):
+    """compile(graph) (reference src/Compiler.jl:181-255) for graphs of attention ops: one persistent
+    device buffer per node, one in-place step per op. Unlike the reference, which allocates host
+    arrays for every non-CUDA device (src/Compiler.jl:224-228), buffers live on the HIP device."""
+    device = device or get_device()
+    if not isinstance(device, HIPDevice):
+        raise RuntimeError("compile: no HIP device available and this backend has no CPU path")
+    results = []
+    for node_id, node in enumerate(graph.nodes):
+        dt = "i32" if graph.dtypes[node_id] == "i32" else graph.dtypes[node_id]
+        results.append(HipArray(graph.shapes[node_id], dt, device).fill_bytes(0))
+    steps = []
+    for node_id, node in enumerate(graph.nodes):
+        if isinstance(node.op, InputTensor):
+            continue
+        args = [results[i] for (i, _, _) in node.inputs]
+        steps.append(lambda out=results[node_id], op=node.op, args=args: execute_op_inplace(out, op, *args))
+    return CompiledGraph(steps, results)
+
+
+def default_scale(D):
+    return float(np.float32(1.0) / np.sqrt(np.float32(D)))
+
+
+__all__ = [
+    "AbstractDevice", "CPUDevice", "HIPDevice", "HipArray", "get_device", "to_device", "from_device", "Graph",
+    "GraphTensor", "tensor", "add_op", "FlashAttentionOp", "DecodeAttentionOp", "flash_attention", "decode_attention",
+    "execute_op", "execute_op_inplace", "execute", "compile", "CompiledGraph", "HEADMAP_INTERLEAVED",
+    "HEADMAP_BLOCKED", "LuminalHipError", "encode", "decode", "f32_to_bf16_bits", "bf16_bits_to_f32", "default_scale",
+]

@@ -1,0 +1,119 @@
+"""CPU-side checks of the C ABI: the built library loads, exports every function the header
+declares, and validates arguments (returning LMH_E_* with a message) before touching a GPU."""
+import ctypes
+import os
+import re
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def header_functions():
+    text = open(os.path.join(ROOT, "include", "luminal_hip.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(lmh_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_header_and_binding_list_the_same_symbols(lm):
+    assert header_functions() == sorted(lm.binding.EXPORTS)
+
+
+def test_library_exports_every_declared_symbol(lm):
+    lib = lm.binding.load()
+    for name in header_functions():
+        assert hasattr(lib, name), name
+    assert lib.lmh_version() == 100
+
+
+def test_struct_layout_matches_header(lm):
+    # field order/size must match the C struct: compare against sizes computed by hand from the header
+    assert ctypes.sizeof(lm.binding.AttnParams) == 5 * 8 + 6 * 4 + 4 * 24 + 5 * 4 + 4 + 8
+    assert ctypes.sizeof(lm.binding.DecodeParams) == 5 * 8 + 5 * 4 + 4 + 2 * 16 + 2 * 24 + 5 * 4 + 4 + 8 + 8 + 8
+
+
+def _attn(lm, **kw):
+    p = lm.binding.AttnParams()
+    p.out, p.q, p.k, p.v = 0x1000, 0x2000, 0x3000, 0x4000  # never dereferenced: validation fails first
+    p.B, p.Hq, p.Hkv, p.Sq, p.Sk, p.D = 1, 4, 2, 8, 8, 64
+    p.dtype, p.scale, p.causal, p.head_map = 0, 0.125, 1, 0
+    for k, v in kw.items():
+        setattr(p, k, v)
+    return p
+
+
+@pytest.mark.parametrize("kw,code", [
+    (dict(q=None), -1), (dict(out=None), -1), (dict(B=0), -2), (dict(D=-3), -2), (dict(Hq=5), -2),
+    (dict(dtype=7), -3), (dict(head_map=9), -3), (dict(D=256), -3), (dict(scale=float("nan")), -2),
+])
+def test_flash_attn_argument_errors(lm, kw, code):
+    with pytest.raises(lm.LuminalHipError) as e:
+        lm.binding.flash_attn_fwd(_attn(lm, **kw))
+    assert e.value.code == code
+    assert "lmh_flash_attn_fwd" in str(e.value)
+
+
+def test_flash_attn_rejects_overlapping_rows(lm):
+    p = _attn(lm)
+    p.k_stride[0], p.k_stride[1], p.k_stride[2] = 1024, 512, 32  # row stride < D
+    with pytest.raises(lm.LuminalHipError) as e:
+        lm.binding.flash_attn_fwd(p)
+    assert e.value.code == lm.binding.LMH_E_SHAPE
+
+
+def _dec(lm, **kw):
+    p = lm.binding.DecodeParams()
+    p.out, p.q, p.k_cache, p.v_cache = 0x1000, 0x2000, 0x3000, 0x4000
+    p.B, p.Hq, p.Hkv, p.Lmax, p.D = 2, 8, 2, 1024, 128
+    p.dtype, p.scale, p.head_map, p.num_splits = 2, 0.088, 0, 4
+    for k, v in kw.items():
+        setattr(p, k, v)
+    return p
+
+
+@pytest.mark.parametrize("kw,code", [
+    (dict(k_cache=None), -1), (dict(Lmax=0), -2), (dict(Hkv=3), -2), (dict(dtype=5), -3), (dict(D=100), -3),
+    (dict(D=512), -3), (dict(num_splits=-1), -2), (dict(k_cache=0x3004), -2),
+    (dict(), -4),                                   # 4 splits but no workspace
+    (dict(workspace=0x5000, workspace_bytes=16), -4),  # workspace too small
+])
+def test_decode_argument_errors(lm, kw, code):
+    with pytest.raises(lm.LuminalHipError) as e:
+        lm.binding.decode_attn(_dec(lm, **kw))
+    assert e.value.code == code
+    assert "lmh_decode_attn" in str(e.value)
+
+
+def test_decode_workspace_and_split_heuristic(lm):
+    b = lm.binding
+    assert b.decode_workspace_bytes(2, 8, 2, 1024, 128, 1) == 0
+    assert b.decode_workspace_bytes(2, 8, 2, 1024, 128, 4) == 2 * 8 * 4 * 130 * 4
+    assert b.decode_workspace_bytes(0, 8, 2, 1024, 128, 4) == 0
+    for (B, Hkv, L) in [(16, 8, 4096), (64, 8, 32768), (1, 1, 17), (1, 8, 100000)]:
+        s = b.decode_auto_splits(B, Hkv, L)
+        assert s >= 1
+        chunk = -(-L // s)
+        assert s == 1 or chunk >= 200  # never shreds the cache into tiny splits
+        assert b.decode_workspace_bytes(B, 4 * Hkv, Hkv, L, 128, 0) == b.decode_workspace_bytes(B, 4 * Hkv, Hkv, L, 128, s)
+
+
+def test_no_device_is_reported_not_fatal(lm):
+    # Device probing never raises: the host's get_device() relies on it to fall through
+    # (reference src/Device.jl:31-74 does the same with try/catch around a tiny allocation).
+    n = lm.binding.device_count()
+    assert n >= 0
+    if n == 0:
+        with pytest.raises(lm.LuminalHipError) as e:
+            lm.binding.init(0)
+        assert e.value.code == lm.binding.LMH_E_NODEVICE
+        assert isinstance(lm.get_device(), lm.CPUDevice)
+
+
+def test_null_and_zero_size_plumbing(lm):
+    b = lm.binding
+    with pytest.raises(lm.LuminalHipError):
+        b.check(b.load().lmh_malloc(None, 16))
+    assert b.load().lmh_free(None) == 0
+    assert b.load().lmh_memcpy_h2d(None, None, 0, None) == 0
+    with pytest.raises(lm.LuminalHipError):
+        b.check(b.load().lmh_memcpy_h2d(None, None, 8, None))

@@ -1,0 +1,317 @@
+"""Parity of the HIP kernels (called through the C ABI) against the CPU oracle and the golden
+vectors, on an MI355X. Tolerances are the contract's: max|err| / max|oracle| <= 1e-5 for fp32 and
+<= 2e-3 for fp16 / bf16, with the oracle evaluated in fp32 on inputs already rounded to the
+element type."""
+import numpy as np
+import pytest
+
+from conftest import TOL, rel_err
+
+pytestmark = pytest.mark.gpu
+
+NT = 16  # oracle threads (rows are independent; results do not depend on it)
+
+
+def out_type(dtype, out_dtype):
+    """bf16 results are taken in fp32 unless a test asks otherwise: rounding a result to bf16 costs up
+    to 2^-8 of its magnitude by itself, more than the 2e-3 budget (test_bf16_output_is_rounded_fp32
+    covers the bf16-out path)."""
+    if out_dtype is not None:
+        return out_dtype
+    return "f32" if dtype == "bf16" else dtype
+
+
+def run_flash(lm, hip, q, k, v, dtype, causal, scale=None, head_map=0, kv_len=None, out_dtype=None):
+    od = out_type(dtype, out_dtype)
+    g = lm.Graph()
+    tq, tk, tv = lm.tensor(g, q.shape, dtype), lm.tensor(g, k.shape, dtype), lm.tensor(g, v.shape, dtype)
+    if kv_len is None:
+        out = lm.flash_attention(tq, tk, tv, scale=scale, causal=causal, head_map=head_map, out_dtype=od)
+        return lm.execute(g, out.id, {tq.id: q, tk.id: k, tv.id: v}, hip)
+    # kv_len is an extension of the op: call the in-place executor directly
+    dq, dk, dv = (lm.to_device(x, hip, dtype) for x in (q, k, v))
+    dl = lm.to_device(np.asarray(kv_len, np.int32), hip)
+    op = lm.FlashAttentionOp(lm.default_scale(q.shape[-1]) if scale is None else scale, causal, head_map)
+    out = lm.HipArray(q.shape, od, hip)
+    lm.host.execute_op_inplace(out, op, dq, dk, dv, dl)
+    return out.to_host()
+
+
+def run_decode(lm, hip, q, kc, vc, dtype, kv_len=None, scale=None, head_map=0, num_splits=0, out_dtype=None):
+    dq, dk, dv = (lm.to_device(x, hip, dtype) for x in (q, kc, vc))
+    dl = None if kv_len is None else lm.to_device(np.asarray(kv_len, np.int32), hip)
+    op = lm.DecodeAttentionOp(lm.default_scale(q.shape[-1]) if scale is None else scale, head_map, num_splits)
+    out = lm.HipArray(q.shape, out_type(dtype, out_dtype), hip)
+    args = (dq, dk, dv) if dl is None else (dq, dk, dv, dl)
+    lm.host.execute_op_inplace(out, op, *args)
+    return out.to_host()
+
+
+def inputs(oracle, shape_q, shape_kv, dtype, seed, mul=1.0):
+    q = oracle.round_to(oracle.gen_normal(shape_q, seed, mul), dtype)
+    k = oracle.round_to(oracle.gen_normal(shape_kv, seed + 1, mul), dtype)
+    v = oracle.round_to(oracle.gen_normal(shape_kv, seed + 2, mul), dtype)
+    return q, k, v
+
+
+# ---------------------------------------------------------------------------------------------
+# golden vectors (independent numpy float64), every element type
+# ---------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("dtype", ["f32", "f16", "bf16"])
+def test_golden_vectors(lm, hip, golden, dtype):
+    for name, c in golden.items():
+        print("case", name, dtype, flush=True)
+        if name.startswith("decode"):
+            got = run_decode(lm, hip, c["q"][:, :, 0], c["k"], c["v"], dtype, kv_len=c["kv_len"], scale=c["scale"])
+            want = c["out"][:, :, 0]
+        else:
+            got = run_flash(lm, hip, c["q"], c["k"], c["v"], dtype, c["causal"], scale=c["scale"], kv_len=c["kv_len"])
+            want = c["out"]
+        assert rel_err(got, want) <= TOL[dtype], (name, dtype)
+
+
+def test_reference_test_shape_criterion(lm, hip, oracle):
+    # the reference's own check: flash ~= manual attention at rtol 1e-4 on B=H=1, S=8, D=16
+    # (reference tests/test_flash_attention_verification.jl:24-49)
+    q, k, v = inputs(oracle, (1, 1, 8, 16), (1, 1, 8, 16), "f32", 100)
+    for causal in (False, True):
+        got = run_flash(lm, hip, q, k, v, "f32", causal)
+        np.testing.assert_allclose(got, oracle.naive_attention_np(q, k, v, causal=causal), rtol=1e-4, atol=1e-6)
+        assert rel_err(got, oracle.flash_attn(q, k, v, causal=causal)) <= 1e-5
+
+
+# ---------------------------------------------------------------------------------------------
+# the five benchmark configurations at full size
+# ---------------------------------------------------------------------------------------------
+def test_config1_llama_example_fp32_causal(lm, hip, oracle):
+    q, k, v = inputs(oracle, (1, 8, 128, 64), (1, 8, 128, 64), "f32", 1000)
+    got = run_flash(lm, hip, q, k, v, "f32", True, scale=0.125)
+    assert rel_err(got, oracle.flash_attn(q, k, v, scale=0.125, causal=True)) <= 1e-5
+    np.testing.assert_array_equal(got[:, :, 0], v[:, :, 0])  # first causal row is V[0] exactly
+
+
+def test_config2_phi3_prefill_fp16_causal_d96(lm, hip, oracle):
+    shape = (1, 32, 4096, 96)
+    q, k, v = inputs(oracle, shape, shape, "f16", 2000, mul=0.5)
+    got = run_flash(lm, hip, q, k, v, "f16", True)
+    want = oracle.flash_attn(q, k, v, causal=True, nthreads=NT)
+    assert rel_err(got, want) <= 2e-3
+
+
+def test_config3_whisper_cross_attention_fp16(lm, hip, oracle):
+    q, k, v = inputs(oracle, (4, 20, 448, 64), (4, 20, 1500, 64), "f16", 3000)
+    got = run_flash(lm, hip, q, k, v, "f16", False)
+    want = oracle.flash_attn(q, k, v, causal=False, nthreads=NT)
+    assert rel_err(got, want) <= 2e-3
+
+
+@pytest.mark.parametrize("head_map", [0, 1])
+def test_config4_llama_gqa_decode_bf16(lm, hip, oracle, head_map):
+    B, Hq, Hkv, L, D = 16, 32, 8, 4096, 128
+    q, k, v = inputs(oracle, (B, Hq, D), (B, Hkv, L, D), "bf16", 4000)
+    lens = np.full(B, L, np.int32)
+    got = run_decode(lm, hip, q, k, v, "bf16", kv_len=lens, head_map=head_map)
+    want = oracle.decode_attn(q, k, v, kv_len=lens, head_map=head_map, nthreads=NT)
+    assert rel_err(got, want) <= 2e-3
+    # the two head maps are different functions of the same inputs
+    other = oracle.decode_attn(q, k, v, kv_len=lens, head_map=1 - head_map, nthreads=NT)
+    assert rel_err(got, other) > 1e-2
+
+
+def test_config5_long_ragged_gqa_decode_bf16(lm, hip, oracle):
+    """B=64, Hq=32, Hkv=8, D=128, kv_len ~ U[8192, 32768]; the cache tail past kv_len[b] is NaN."""
+    B, Hq, Hkv, Lmax, D = 64, 32, 8, 32768, 128
+    lens = oracle.gen_uniform_int(B, 5000, 8192, 32768)
+    q = oracle.round_to(oracle.gen_normal((B, Hq, D), 5001), "bf16")
+    dk = lm.HipArray((B, Hkv, Lmax, D), "bf16", hip).fill_bytes(0xFF)  # 0xFFFF = NaN
+    dv = lm.HipArray((B, Hkv, Lmax, D), "bf16", hip).fill_bytes(0xFF)
+    want = np.empty((B, Hq, D), np.float32)
+    row_bytes = D * 2
+    for b in range(B):
+        n = int(lens[b])
+        kb = oracle.round_to(oracle.gen_normal((1, Hkv, n, D), 6000 + 2 * b), "bf16")
+        vb = oracle.round_to(oracle.gen_normal((1, Hkv, n, D), 6001 + 2 * b), "bf16")
+        want[b] = oracle.decode_attn(q[b:b + 1], kb, vb, nthreads=NT)[0]
+        kbits, vbits = lm.encode(kb, "bf16"), lm.encode(vb, "bf16")
+        for h in range(Hkv):
+            off = ((b * Hkv + h) * Lmax) * row_bytes
+            lm.binding.memcpy_h2d(dk.ptr + off, kbits[0, h].ctypes.data, n * row_bytes)
+            lm.binding.memcpy_h2d(dv.ptr + off, vbits[0, h].ctypes.data, n * row_bytes)
+    dq = lm.to_device(q, hip, "bf16")
+    dl = lm.to_device(lens, hip)
+    results = {}
+    for splits in (0, 8, 57):
+        out = lm.HipArray((B, Hq, D), "f32", hip)
+        lm.host.execute_op_inplace(out, lm.DecodeAttentionOp(lm.default_scale(D), 0, splits), dq, dk, dv, dl)
+        results[splits] = out.to_host()
+        assert rel_err(results[splits], want) <= 2e-3, splits
+    # split-count invariance (log-sum-exp merge identity): same answer up to fp32 reassociation
+    assert rel_err(results[8], results[0]) <= 1e-5
+    assert rel_err(results[57], results[0]) <= 1e-5
+
+
+# ---------------------------------------------------------------------------------------------
+# shape / feature sweeps
+# ---------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("D", [16, 24, 32, 64, 80, 96, 128])
+@pytest.mark.parametrize("causal", [False, True])
+def test_fp32_head_dims(lm, hip, oracle, D, causal):
+    q, k, v = inputs(oracle, (2, 3, 70, D), (2, 3, 70, D), "f32", 7000 + D)
+    assert rel_err(run_flash(lm, hip, q, k, v, "f32", causal), oracle.flash_attn(q, k, v, causal=causal)) <= 1e-5
+
+
+@pytest.mark.parametrize("Sq,Sk", [(1, 1), (1, 77), (7, 7), (64, 64), (65, 130), (130, 65), (257, 300)])
+@pytest.mark.parametrize("causal", [False, True])
+def test_fp32_sequence_shapes(lm, hip, oracle, Sq, Sk, causal):
+    q, k, v = inputs(oracle, (1, 2, Sq, 64), (1, 2, Sk, 64), "f32", 7100 + Sq)
+    assert rel_err(run_flash(lm, hip, q, k, v, "f32", causal), oracle.flash_attn(q, k, v, causal=causal)) <= 1e-5
+
+
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
+@pytest.mark.parametrize("D", [64, 96, 128])
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("Sq,Sk", [(1, 1), (1, 200), (64, 64), (127, 127), (128, 128), (129, 129), (300, 1000), (1000, 300), (513, 513)])
+def test_mfma_shapes(lm, hip, oracle, dtype, D, causal, Sq, Sk):
+    q, k, v = inputs(oracle, (2, 3, Sq, D), (2, 3, Sk, D), dtype, 7200 + Sq + D)
+    got = run_flash(lm, hip, q, k, v, dtype, causal)
+    assert rel_err(got, oracle.flash_attn(q, k, v, causal=causal, nthreads=NT)) <= 2e-3
+
+
+@pytest.mark.parametrize("dtype", ["f32", "f16", "bf16"])
+@pytest.mark.parametrize("head_map", [0, 1])
+def test_gqa_prefill_both_head_maps(lm, hip, oracle, dtype, head_map):
+    q, k, v = inputs(oracle, (2, 8, 150, 64), (2, 2, 150, 64), dtype, 7300)
+    got = run_flash(lm, hip, q, k, v, dtype, True, head_map=head_map)
+    assert rel_err(got, oracle.flash_attn(q, k, v, causal=True, head_map=head_map, nthreads=NT)) <= TOL[dtype]
+    assert rel_err(got, oracle.flash_attn(q, k, v, causal=True, head_map=1 - head_map, nthreads=NT)) > 1e-2
+
+
+@pytest.mark.parametrize("dtype", ["f32", "f16", "bf16"])
+def test_prefill_ragged_kv_len_with_poisoned_tail(lm, hip, oracle, dtype):
+    B, H, Sq, Sk, D = 3, 2, 40, 200, 64
+    q, k, v = inputs(oracle, (B, H, Sq, D), (B, H, Sk, D), dtype, 7400)
+    lens = np.array([200, 65, 1], np.int32)
+    kp, vp = k.copy(), v.copy()
+    for b, n in enumerate(lens):
+        kp[b, :, n:] = np.nan
+        vp[b, :, n:] = np.nan
+    got = run_flash(lm, hip, q, kp, vp, dtype, False, kv_len=lens)
+    assert rel_err(got, oracle.flash_attn(q, k, v, kv_len=lens)) <= TOL[dtype]
+
+
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
+def test_unusual_head_dim_and_scale_take_the_vector_path(lm, hip, oracle, dtype):
+    q, k, v = inputs(oracle, (1, 2, 90, 80), (1, 2, 90, 80), dtype, 7500)
+    assert rel_err(run_flash(lm, hip, q, k, v, dtype, True), oracle.flash_attn(q, k, v, causal=True)) <= 2e-3
+    q, k, v = inputs(oracle, (1, 2, 90, 64), (1, 2, 90, 64), dtype, 7501)
+    for scale in (-0.2, 0.0):
+        assert rel_err(run_flash(lm, hip, q, k, v, dtype, True, scale=scale),
+                       oracle.flash_attn(q, k, v, causal=True, scale=scale)) <= 2e-3
+
+
+def test_whisper_split_scale_equals_single_scale(lm, hip, oracle):
+    # Whisper multiplies q and k by D^-0.25 each (reference src/Whisper.jl:305-307); the fused op takes
+    # unscaled q, k and scale = 1/sqrt(D). Same function up to fp32 rounding.
+    q, k, v = inputs(oracle, (1, 4, 30, 64), (1, 4, 100, 64), "f32", 7600)
+    s = np.float32(64) ** np.float32(-0.25)
+    split = run_flash(lm, hip, q * s, k * s, v, "f32", False, scale=1.0)
+    fused = run_flash(lm, hip, q, k, v, "f32", False)
+    assert rel_err(split, fused) <= 1e-5
+
+
+@pytest.mark.parametrize("dtype,D", [("f32", 64), ("f32", 128), ("f16", 64), ("f16", 96), ("bf16", 128), ("bf16", 256), ("f16", 8)])
+@pytest.mark.parametrize("Hq,Hkv", [(4, 4), (8, 4), (8, 2), (8, 1), (12, 2), (16, 1)])
+def test_decode_group_sizes_and_dims(lm, hip, oracle, dtype, D, Hq, Hkv):
+    B, L = 3, 333
+    q, k, v = inputs(oracle, (B, Hq, D), (B, Hkv, L, D), dtype, 7700 + D + Hq)
+    lens = np.array([333, 100, 1], np.int32)
+    for hm in (0, 1):
+        for splits in (1, 3):
+            got = run_decode(lm, hip, q, k, v, dtype, kv_len=lens, head_map=hm, num_splits=splits)
+            want = oracle.decode_attn(q, k, v, kv_len=lens, head_map=hm)
+            assert rel_err(got, want) <= TOL[dtype], (hm, splits)
+
+
+def test_decode_equals_last_row_of_causal_prefill_on_gpu(lm, hip, oracle):
+    B, Hq, Hkv, L, D = 2, 8, 2, 257, 128
+    q, k, v = inputs(oracle, (B, Hq, L, D), (B, Hkv, L, D), "bf16", 7800)
+    full = run_flash(lm, hip, q, k, v, "bf16", True)
+    dec = run_decode(lm, hip, np.ascontiguousarray(q[:, :, L - 1]), k, v, "bf16")
+    assert rel_err(dec, full[:, :, L - 1]) <= 4e-3  # two results, each within 2e-3 of the oracle
+
+
+def test_decode_without_kv_len_and_poisoned_tail(lm, hip, oracle):
+    B, Hq, Hkv, L, D = 2, 8, 2, 1000, 128
+    q, k, v = inputs(oracle, (B, Hq, D), (B, Hkv, L, D), "bf16", 7900)
+    assert rel_err(run_decode(lm, hip, q, k, v, "bf16"), oracle.decode_attn(q, k, v)) <= 2e-3
+    lens = np.array([999, 130], np.int32)
+    kp, vp = k.copy(), v.copy()
+    for b, n in enumerate(lens):
+        kp[b, :, n:] = np.nan
+        vp[b, :, n:] = np.nan
+    for splits in (0, 1, 5):
+        got = run_decode(lm, hip, q, kp, vp, "bf16", kv_len=lens, num_splits=splits)
+        assert rel_err(got, oracle.decode_attn(q, k, v, kv_len=lens)) <= 2e-3
+
+
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
+def test_half_output_is_the_rounded_fp32_output(lm, hip, oracle, dtype):
+    """out_f32 = 0 writes the same result rounded once to the input element type. The two code paths
+    may differ in the last fp32 bit (the compiler schedules the final multiply separately), which
+    moves a value across a rounding boundary now and then: allow one unit in the last place on a
+    tiny fraction of the elements."""
+    ulp = 2.0 ** -10 if dtype == "f16" else 2.0 ** -7
+
+    def check(narrow, wide):
+        want = oracle.round_to(wide, dtype)
+        assert np.mean(narrow != want) < 1e-3
+        assert np.all(np.abs(narrow - want) <= ulp * np.maximum(np.abs(want), 2.0 ** -14))
+
+    q, k, v = inputs(oracle, (1, 4, 200, 128), (1, 4, 200, 128), dtype, 8500)
+    check(run_flash(lm, hip, q, k, v, dtype, True, out_dtype=dtype), run_flash(lm, hip, q, k, v, dtype, True, out_dtype="f32"))
+    qd, kd, vd = inputs(oracle, (3, 8, 128), (3, 2, 900, 128), dtype, 8600)
+    for splits in (1, 4):
+        check(run_decode(lm, hip, qd, kd, vd, dtype, num_splits=splits, out_dtype=dtype),
+              run_decode(lm, hip, qd, kd, vd, dtype, num_splits=splits, out_dtype="f32"))
+
+
+def test_strided_tensors(lm, hip, oracle):
+    # K and V interleaved in one [B, H, S, 2, D] buffer: row stride 2*D, exercised through explicit strides
+    B, H, S, D = 2, 4, 100, 64
+    q, k, v = inputs(oracle, (B, H, S, D), (B, H, S, D), "f16", 8000)
+    kv = np.stack([k, v], axis=3)  # [B,H,S,2,D]
+    dkv = lm.to_device(kv, hip, "f16")
+    dq = lm.to_device(q, hip, "f16")
+    out = lm.HipArray(q.shape, "f16", hip)
+    p = lm.binding.AttnParams()
+    p.out, p.q, p.k, p.v = out.ptr, dq.ptr, dkv.ptr, dkv.ptr + D * 2
+    p.B, p.Hq, p.Hkv, p.Sq, p.Sk, p.D = B, H, H, S, S, D
+    for arr in (p.k_stride, p.v_stride):
+        arr[0], arr[1], arr[2] = H * S * 2 * D, S * 2 * D, 2 * D
+    p.dtype, p.scale, p.causal, p.head_map = lm.binding.LMH_F16, lm.default_scale(D), 1, 0
+    lm.binding.flash_attn_fwd(p)
+    assert rel_err(out.to_host(), oracle.flash_attn(q, k, v, causal=True)) <= 2e-3
+
+
+def test_compiled_graph_reuses_buffers(lm, hip, oracle):
+    # compile() pre-allocates one buffer per node and runs in place (reference src/Compiler.jl:218-255)
+    B, H, S, D = 1, 4, 96, 64
+    g = lm.Graph()
+    tq, tk, tv = (lm.tensor(g, (B, H, S, D), "f16") for _ in range(3))
+    out = lm.flash_attention(tq, tk, tv, causal=True)
+    cg = lm.compile(g, hip)
+    ptr_before = cg.results[out.id].ptr
+    for seed in (8100, 8200):
+        q, k, v = inputs(oracle, (B, H, S, D), (B, H, S, D), "f16", seed)
+        res = cg({tq.id: q, tk.id: k, tv.id: v}, hip)
+        assert rel_err(lm.from_device(res[out.id]), oracle.flash_attn(q, k, v, causal=True)) <= 2e-3
+    assert cg.results[out.id].ptr == ptr_before
+
+
+def test_rerun_is_bitwise_deterministic(lm, hip, oracle):
+    q, k, v = inputs(oracle, (1, 4, 500, 96), (1, 4, 500, 96), "f16", 8300)
+    a = run_flash(lm, hip, q, k, v, "f16", True)
+    b = run_flash(lm, hip, q, k, v, "f16", True)
+    np.testing.assert_array_equal(a, b)
+    qd, kd, vd = inputs(oracle, (4, 8, 128), (4, 2, 3000, 128), "bf16", 8400)
+    np.testing.assert_array_equal(run_decode(lm, hip, qd, kd, vd, "bf16"), run_decode(lm, hip, qd, kd, vd, "bf16"))
