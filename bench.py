@@ -1,0 +1,313 @@
+#!/usr/bin/env python3
+"""Benchmark of the attention hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--only all|prefill|decode|copy]
+
+A step is one pass of the hot path over one batch of synthetic input, inputs resident in HBM:
+  prefill leg (the headline `value`): causal flash attention, Phi-3-mini shape
+      B=1, Hq=Hkv=32, S=4096, D=96, fp16 in/out, fp32 accumulate        -> TFLOP/s, MFMA roofline
+  decode leg (reported under "decode"): split-KV GQA decode, long ragged batch
+      B=64, Hq=32, Hkv=8, D=128, bf16, kv_len ~ U[8192, 32768]          -> GB/s, HBM roofline
+Other configurations of the contract (fp32 S=128, Whisper cross attention, B=16 L=4096 decode) are
+timed briefly and listed under "other_configs".
+
+Algorithmic work: prefill FLOPs = 4*B*Hq*D*S*(S+1)/2 (2 flops per MAC, QK^T and PV, unmasked pairs
+only); decode bytes = 2 * sum_b kv_len[b] * Hkv * D * 2 (K and V once per KV head) + q + out.
+
+Kernel time is measured with HIP events on the launch stream around the timed steps; the CPU
+baseline is the oracle (a C restatement of the reference's flash_attn_cpu) on a bounded sample of
+the same workload, whose output also serves as a parity check of the GPU result.
+One JSON line on stdout; progress on stderr.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK_FP16_TFLOPS = 2500.0  # MI355X dense fp16/bf16 MFMA
+PEAK_HBM_GBS = 8000.0      # MI355X HBM3E
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def time_steps(fn, steps, warmup, binding):
+    """warmup untimed calls, then `steps` timed calls bracketed by a device sync on both sides.
+    Returns (wall ms per step, HIP-event ms per step)."""
+    for _ in range(warmup):
+        fn()
+    binding.sync()
+    e0, e1 = binding.Event(), binding.Event()
+    t0 = time.perf_counter()
+    e0.record()
+    for _ in range(steps):
+        fn()
+    e1.record()
+    binding.sync()
+    t1 = time.perf_counter()
+    return (t1 - t0) * 1e3 / steps, e1.elapsed_ms_since(e0) / steps
+
+
+def attn_params(lm, out, q, k, v, dtype, causal, scale, head_map=0, kv_len=None):
+    p = lm.binding.AttnParams()
+    p.out, p.q, p.k, p.v = out.ptr, q.ptr, k.ptr, v.ptr
+    p.kv_len = kv_len.ptr if kv_len is not None else None
+    p.B, p.Hq, p.Sq, p.D = q.shape
+    p.Hkv, p.Sk = k.shape[1], k.shape[2]
+    p.dtype = lm.binding.DTYPE_CODES[dtype]
+    p.scale, p.causal, p.head_map = scale, int(causal), head_map
+    p.out_f32 = int(out.dtype == "f32")
+    return p
+
+
+def decode_params(lm, out, q, kc, vc, kv_len, dtype, scale, ws, head_map=0, num_splits=0):
+    b = lm.binding
+    p = b.DecodeParams()
+    p.out, p.q, p.k_cache, p.v_cache = out.ptr, q.ptr, kc.ptr, vc.ptr
+    p.kv_len = kv_len.ptr if kv_len is not None else None
+    p.B, p.Hq, p.D = q.shape
+    p.Hkv, p.Lmax = kc.shape[1], kc.shape[2]
+    p.dtype = b.DTYPE_CODES[dtype]
+    p.scale, p.head_map = scale, head_map
+    p.out_f32 = int(out.dtype == "f32")
+    p.num_splits = num_splits or b.decode_auto_splits(p.B, p.Hkv, p.Lmax)
+    p.workspace, p.workspace_bytes = ws.ptr, ws.nbytes
+    return p
+
+
+def rel_err(got, want):
+    return float(np.abs(np.asarray(got, np.float64) - want).max() / np.abs(want).max())
+
+
+# -------------------------------------------------------------------------------------------------
+def prefill_leg(lm, dev, steps, warmup, cpu_seconds):
+    B, H, S, D = 1, 32, 4096, 96
+    rng = np.random.default_rng(2)
+    host = [(rng.standard_normal((B, H, S, D), dtype=np.float32) * 0.5).astype(np.float16) for _ in range(3)]
+    dq, dk, dv = (lm.HipArray((B, H, S, D), "f16", dev).copy_from_host(x) for x in host)
+    out = lm.HipArray((B, H, S, D), "f16", dev)
+    scale = lm.default_scale(D)
+    p = attn_params(lm, out, dq, dk, dv, "f16", True, scale)
+    fn = lambda: lm.binding.flash_attn_fwd(p)
+    wall_ms, ev_ms = time_steps(fn, steps, warmup, lm.binding)
+    flops = 4.0 * B * H * D * S * (S + 1) / 2
+    tflops = flops / (wall_ms * 1e-3) / 1e12
+    kern_tflops = flops / (ev_ms * 1e-3) / 1e12
+    log("[prefill] C2 causal fp16 B=1 H=32 S=4096 D=96: %.1f us/step wall, %.1f us/launch events, %.1f TFLOP/s (%.1f%% of %g)"
+        % (wall_ms * 1e3, ev_ms * 1e3, kern_tflops, 100 * kern_tflops / PEAK_FP16_TFLOPS, PEAK_FP16_TFLOPS))
+    res = {
+        "ms_per_step": wall_ms, "value": tflops,
+        "roofline": {"bound": "mfma", "achieved": kern_tflops, "peak": PEAK_FP16_TFLOPS, "unit": "TFLOP/s",
+                     "frac": kern_tflops / PEAK_FP16_TFLOPS, "traffic": None,
+                     "kernel": "prefill_mfma_kernel<MfmaF16, 96, causal>", "launch_us": ev_ms * 1e3,
+                     "algorithmic_flops_per_launch": flops},
+    }
+    if cpu_seconds > 0:
+        # CPU baseline = the oracle on a head subset of the same workload, all host threads; the same
+        # output is the parity check of the GPU result for those heads.
+        import oracle
+        nthreads = oracle.max_threads()
+        got = out.to_host()
+        q32, k32, v32 = (x.astype(np.float32) for x in host)
+        heads, t_cpu, worst = 0, 0.0, 0.0
+        step_heads = 2
+        while heads < H and (heads == 0 or t_cpu * (heads + step_heads) / heads < cpu_seconds):
+            sl = slice(heads, heads + step_heads)
+            t0 = time.perf_counter()
+            want = oracle.flash_attn(q32[:, sl], k32[:, sl], v32[:, sl], scale=scale, causal=True, nthreads=nthreads)
+            t_cpu += time.perf_counter() - t0
+            worst = max(worst, rel_err(got[:, sl], want))
+            heads += step_heads
+        cpu_tflops = flops * heads / H / t_cpu / 1e12
+        log("[prefill] CPU oracle: %d of %d heads in %.1f s on %d threads = %.4f TFLOP/s; GPU vs oracle rel err %.2e"
+            % (heads, H, t_cpu, nthreads, cpu_tflops, worst))
+        res["cpu_baseline"] = {"value": cpu_tflops, "unit": "TFLOP/s", "cores": nthreads, "kind": "port",
+                               "sample": "heads 0..%d of %d, all %d query rows, %.1f s" % (heads - 1, H, S, t_cpu)}
+        res["parity"] = {"max_rel_err": worst, "tolerance": 2e-3, "checked": "heads 0..%d vs CPU oracle" % (heads - 1)}
+        if worst > 2e-3:
+            raise SystemExit("prefill parity check failed: rel err %.3g > 2e-3" % worst)
+    return res
+
+
+def fill_cache_from_pool(lm, cache, pool, lens, Hkv, Lmax, D, rng):
+    """cache[b, h, 0:lens[b]] <- a row-aligned window of `pool` (device-to-device); returns the windows."""
+    row_bytes = D * 2
+    pool_rows = pool.shape[0]
+    starts = np.zeros((len(lens), Hkv), np.int64)
+    for b, n in enumerate(lens):
+        for h in range(Hkv):
+            s = int(rng.integers(0, pool_rows - int(n)))
+            starts[b, h] = s
+            lm.binding.memcpy_d2d(cache.ptr + ((b * Hkv + h) * Lmax) * row_bytes, pool.ptr + s * row_bytes, int(n) * row_bytes)
+    return starts
+
+
+def decode_leg(lm, dev, steps, warmup, cpu_seconds):
+    B, Hq, Hkv, Lmax, D = 64, 32, 8, 32768, 128
+    rng = np.random.default_rng(5)
+    lens = rng.integers(8192, 32768, size=B, endpoint=True).astype(np.int32)
+    pool_rows = 1 << 18  # 256 Ki rows of 128 bf16 = 64 MiB per pool
+    pools_host = [lm.f32_to_bf16_bits(rng.standard_normal((pool_rows, D), dtype=np.float32)) for _ in range(2)]
+    kpool, vpool = (lm.HipArray((pool_rows, D), "bf16", dev).copy_from_host(x) for x in pools_host)
+    kc = lm.HipArray((B, Hkv, Lmax, D), "bf16", dev).fill_bytes(0xFF)  # tail past kv_len is NaN
+    vc = lm.HipArray((B, Hkv, Lmax, D), "bf16", dev).fill_bytes(0xFF)
+    kstart = fill_cache_from_pool(lm, kc, kpool, lens, Hkv, Lmax, D, rng)
+    vstart = fill_cache_from_pool(lm, vc, vpool, lens, Hkv, Lmax, D, rng)
+    q_host = lm.f32_to_bf16_bits(rng.standard_normal((B, Hq, D), dtype=np.float32))
+    dq = lm.HipArray((B, Hq, D), "bf16", dev).copy_from_host(q_host)
+    dl = lm.HipArray((B,), "i32", dev).copy_from_host(lens)
+    out = lm.HipArray((B, Hq, D), "f32", dev)
+    ws = lm.HipArray((max(lm.binding.decode_workspace_bytes(B, Hq, Hkv, Lmax, D, 0) // 4, 4),), "f32", dev)
+    scale = lm.default_scale(D)
+    p = decode_params(lm, out, dq, kc, vc, dl, "bf16", scale, ws)
+    fn = lambda: lm.binding.decode_attn(p)
+    wall_ms, ev_ms = time_steps(fn, steps, warmup, lm.binding)
+    algo_bytes = 2.0 * float(lens.sum()) * Hkv * D * 2 + B * Hq * D * 2 + B * Hq * D * 4
+    gbs = algo_bytes / (wall_ms * 1e-3) / 1e9
+    kern_gbs = algo_bytes / (ev_ms * 1e-3) / 1e9
+    log("[decode] C5 bf16 B=64 Hq=32 Hkv=8 D=128 sum(kv_len)=%d (%.2f GB): %.1f us/step wall, %.1f us events, %.0f GB/s (%.1f%% of %g); %d splits"
+        % (int(lens.sum()), algo_bytes / 1e9, wall_ms * 1e3, ev_ms * 1e3, kern_gbs, 100 * kern_gbs / PEAK_HBM_GBS, PEAK_HBM_GBS, p.num_splits))
+    res = {
+        "workload": "C5 long ragged GQA decode: B=64 Hq=32 Hkv=8 D=128 bf16, kv_len~U[8192,32768], sum=%d" % int(lens.sum()),
+        "value": gbs, "unit": "GB/s", "ms_per_step": wall_ms, "num_splits": int(p.num_splits),
+        "roofline": {"bound": "hbm", "achieved": kern_gbs, "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": kern_gbs / PEAK_HBM_GBS,
+                     "traffic": None, "kernel": "decode_split_kernel<BF16,16,4> + decode_merge_kernel",
+                     "launch_us": ev_ms * 1e3, "algorithmic_bytes_per_launch": algo_bytes},
+    }
+    if cpu_seconds > 0:
+        import oracle
+        nthreads = oracle.max_threads()
+        got = out.to_host()
+        qf = lm.bf16_bits_to_f32(q_host)
+        kp32, vp32 = (lm.bf16_bits_to_f32(x) for x in pools_host)
+        done, t_cpu, worst, bytes_done = 0, 0.0, 0.0, 0.0
+        while done < B and (done == 0 or t_cpu * (done + 1) / done < cpu_seconds):
+            b, n = done, int(lens[done])
+            kb = np.stack([kp32[kstart[b, h]:kstart[b, h] + n] for h in range(Hkv)])[None]
+            vb = np.stack([vp32[vstart[b, h]:vstart[b, h] + n] for h in range(Hkv)])[None]
+            t0 = time.perf_counter()
+            want = oracle.decode_attn(qf[b:b + 1], kb, vb, scale=scale, nthreads=nthreads)
+            t_cpu += time.perf_counter() - t0
+            worst = max(worst, rel_err(got[b:b + 1], want))
+            bytes_done += 2.0 * n * Hkv * D * 2
+            done += 1
+        cpu_gbs = bytes_done / t_cpu / 1e9
+        log("[decode] CPU oracle: %d of %d sequences in %.2f s on %d threads = %.2f GB/s (bf16-equivalent bytes); rel err %.2e"
+            % (done, B, t_cpu, nthreads, cpu_gbs, worst))
+        res["cpu_baseline"] = {"value": cpu_gbs, "unit": "GB/s", "cores": nthreads, "kind": "port",
+                               "sample": "sequences 0..%d of %d at their full kv_len, %.2f s" % (done - 1, B, t_cpu)}
+        res["parity"] = {"max_rel_err": worst, "tolerance": 2e-3, "checked": "sequences 0..%d vs CPU oracle" % (done - 1)}
+        if worst > 2e-3:
+            raise SystemExit("decode parity check failed: rel err %.3g > 2e-3" % worst)
+    for a in (kc, vc, kpool, vpool, ws):
+        a.free()
+    return res
+
+
+def other_configs(lm, dev):
+    """Short timings of the remaining contract configurations (20 launches each)."""
+    res = {}
+    rng = np.random.default_rng(9)
+
+    def flash(name, B, Hq, Hkv, Sq, Sk, D, dtype, causal, flops):
+        q = lm.HipArray((B, Hq, Sq, D), dtype, dev).copy_from_host(rng.standard_normal((B, Hq, Sq, D), dtype=np.float32))
+        k = lm.HipArray((B, Hkv, Sk, D), dtype, dev).copy_from_host(rng.standard_normal((B, Hkv, Sk, D), dtype=np.float32))
+        v = lm.HipArray((B, Hkv, Sk, D), dtype, dev).copy_from_host(rng.standard_normal((B, Hkv, Sk, D), dtype=np.float32))
+        o = lm.HipArray((B, Hq, Sq, D), dtype, dev)
+        p = attn_params(lm, o, q, k, v, dtype, causal, lm.default_scale(D))
+        _, ev = time_steps(lambda: lm.binding.flash_attn_fwd(p), 20, 5, lm.binding)
+        res[name] = {"launch_us": ev * 1e3, "TFLOP/s": flops / (ev * 1e-3) / 1e12}
+        log("[other] %s: %.1f us, %.2f TFLOP/s" % (name, ev * 1e3, res[name]["TFLOP/s"]))
+
+    flash("C1 causal fp32 B=1 H=8 S=128 D=64", 1, 8, 8, 128, 128, 64, "f32", True, 4.0 * 8 * 64 * 128 * 129 / 2)
+    flash("C3 cross fp16 B=4 H=20 Sq=448 Sk=1500 D=64", 4, 20, 20, 448, 1500, 64, "f16", False, 4.0 * 4 * 20 * 448 * 1500 * 64)
+
+    # C4: B=16 L=4096 decode; 268 MB would sit in the 256 MB last-level cache, so rotate over 4 caches
+    B, Hq, Hkv, L, D = 16, 32, 8, 4096, 128
+    pool = lm.f32_to_bf16_bits(rng.standard_normal((B * Hkv * L, D), dtype=np.float32))
+    caches = []
+    for i in range(4):
+        kc = lm.HipArray((B, Hkv, L, D), "bf16", dev).copy_from_host(np.roll(pool, 977 * i, axis=0))
+        vc = lm.HipArray((B, Hkv, L, D), "bf16", dev).copy_from_host(np.roll(pool, 977 * i + 401, axis=0))
+        caches.append((kc, vc))
+    q = lm.HipArray((B, Hq, D), "bf16", dev).copy_from_host(rng.standard_normal((B, Hq, D), dtype=np.float32))
+    o = lm.HipArray((B, Hq, D), "f32", dev)
+    ws = lm.HipArray((max(lm.binding.decode_workspace_bytes(B, Hq, Hkv, L, D, 0) // 4, 4),), "f32", dev)
+    ps = [decode_params(lm, o, q, kc, vc, None, "bf16", lm.default_scale(D), ws) for kc, vc in caches]
+    state = {"i": 0}
+
+    def step():
+        lm.binding.decode_attn(ps[state["i"] % 4])
+        state["i"] += 1
+
+    _, ev = time_steps(step, 40, 8, lm.binding)
+    nbytes = 2.0 * B * L * Hkv * D * 2 + B * Hq * D * 6
+    res["C4 decode bf16 B=16 Hq=32 Hkv=8 L=4096 D=128 (4 caches rotated)"] = {
+        "launch_us": ev * 1e3, "GB/s": nbytes / (ev * 1e-3) / 1e9, "frac_of_hbm_peak": nbytes / (ev * 1e-3) / 1e9 / PEAK_HBM_GBS}
+    log("[other] C4 decode: %.1f us, %.0f GB/s" % (ev * 1e3, nbytes / (ev * 1e-3) / 1e9))
+    return res
+
+
+def copy_leg(lm, dev, steps, warmup):
+    """The calibration copy kernel alone (profile this with --pmc FETCH_SIZE / WRITE_SIZE)."""
+    nbytes = 1 << 30
+    src = lm.HipArray((nbytes // 4,), "f32", dev).fill_bytes(1)
+    dst = lm.HipArray((nbytes // 4,), "f32", dev).fill_bytes(0)
+    _, ev = time_steps(lambda: lm.binding.calib_copy(dst.ptr, src.ptr, nbytes), steps, warmup, lm.binding)
+    log("[copy] %d bytes read + %d written per launch: %.1f us, %.0f GB/s" % (nbytes, nbytes, ev * 1e3, 2 * nbytes / (ev * 1e-3) / 1e9))
+    return {"bytes_read_per_launch": nbytes, "bytes_written_per_launch": nbytes, "launch_us": ev * 1e3}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--only", choices=["all", "prefill", "decode", "copy"], default="all")
+    ap.add_argument("--cpu-seconds", type=float, default=15.0, help="CPU-baseline budget per leg; 0 disables it")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: the attention path shards over (batch, KV head) with no exchange and "
+              "nothing here uses a second device; run with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+
+    import __graft_entry__
+    lm = __graft_entry__.load_package()
+    dev = lm.get_device()
+    if not isinstance(dev, lm.HIPDevice):
+        raise SystemExit("bench.py needs an MI355X: libluminal_hip.so found no gfx950 device (no CPU fallback exists)")
+    log("[bench] device:", lm.binding.device_name())
+
+    line = {
+        "metric": "attention TFLOP/s (prefill) + KV-read GB/s (decode), % roofline, 1xMI355X",
+        "value": None, "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": None, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f16",
+        "data": "synthetic",
+        "config": {"workload": "C2 Phi-3-mini causal prefill attention: B=1 Hq=Hkv=32 S=4096 D=96, fp16 in/out, fp32 accumulate, scale 1/sqrt(96)"},
+    }
+    if args.only == "copy":
+        line["calibration_copy"] = copy_leg(lm, dev, args.steps, args.warmup)
+        print(json.dumps(line))
+        return
+    if args.only in ("all", "prefill"):
+        r = prefill_leg(lm, dev, args.steps, args.warmup, args.cpu_seconds)
+        line["value"], line["ms_per_step"] = r["value"], r["ms_per_step"]
+        line["roofline"] = r["roofline"]
+        if "cpu_baseline" in r:
+            line["cpu_baseline"], line["parity"] = r["cpu_baseline"], r["parity"]
+    if args.only in ("all", "decode"):
+        line["decode"] = decode_leg(lm, dev, args.steps, args.warmup, args.cpu_seconds)
+    if args.only == "all":
+        line["other_configs"] = other_configs(lm, dev)
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

@@ -75,6 +75,11 @@ int lmh_event_destroy(void *event);
 int lmh_event_record(void *event, void *stream);
 int lmh_event_elapsed_ms(float *ms, void *start, void *stop);
 
+/* Measurement aid with no counterpart in the reference: a plain copy kernel (reads `bytes`,
+ * writes `bytes`; both pointers and the size multiples of 16) used to calibrate HBM traffic
+ * counters against a known transfer. */
+int lmh_calib_copy(void *dst_dev, const void *src_dev, size_t bytes, void *stream);
+
 /* ---- flash attention forward: replaces
  *   execute_op!(out, op::FlashAttentionOp, q, k, v)   reference src/Execution.jl:565-578
  *   flash_attn_cpu(q, k, v, scale, causal)            reference src/Execution.jl:453-479

@@ -23,7 +23,7 @@ EXPORTS = [
     "lmh_version", "lmh_last_error", "lmh_device_count", "lmh_init", "lmh_device_name", "lmh_malloc", "lmh_free",
     "lmh_memset", "lmh_memcpy_h2d", "lmh_memcpy_d2h", "lmh_memcpy_d2d", "lmh_sync", "lmh_event_create",
     "lmh_event_destroy", "lmh_event_record", "lmh_event_elapsed_ms", "lmh_flash_attn_fwd",
-    "lmh_decode_workspace_bytes", "lmh_decode_auto_splits", "lmh_decode_attn",
+    "lmh_decode_workspace_bytes", "lmh_decode_auto_splits", "lmh_decode_attn", "lmh_calib_copy",
 ]
 
 
@@ -96,7 +96,8 @@ def load():
     L.lmh_decode_workspace_bytes.argtypes = [ctypes.c_int32] * 6
     L.lmh_decode_auto_splits.restype = ctypes.c_int32
     L.lmh_decode_auto_splits.argtypes = [ctypes.c_int32] * 3
-    for name in ("lmh_init", "lmh_device_name", "lmh_malloc", "lmh_free", "lmh_memset", "lmh_memcpy_h2d",
+    L.lmh_calib_copy.argtypes = [vp, vp, ctypes.c_size_t, vp]
+    for name in ("lmh_calib_copy", "lmh_init", "lmh_device_name", "lmh_malloc", "lmh_free", "lmh_memset", "lmh_memcpy_h2d",
                  "lmh_memcpy_d2h", "lmh_memcpy_d2d", "lmh_sync", "lmh_event_create", "lmh_event_destroy",
                  "lmh_event_record", "lmh_event_elapsed_ms", "lmh_flash_attn_fwd", "lmh_decode_attn"):
         getattr(L, name).restype = ctypes.c_int
@@ -181,6 +182,10 @@ def flash_attn_fwd(params):
 
 def decode_attn(params):
     check(load().lmh_decode_attn(ctypes.byref(params)))
+
+
+def calib_copy(dst, src, nbytes, stream=None):
+    check(load().lmh_calib_copy(dst, src, nbytes, stream))
 
 
 def decode_workspace_bytes(B, Hq, Hkv, Lmax, D, num_splits=0):
