@@ -149,10 +149,12 @@ def fill_cache_from_pool(lm, cache, pool, lens, Hkv, Lmax, D, rng):
     return starts
 
 
-def decode_leg(lm, dev, steps, warmup, cpu_seconds):
+def decode_leg(lm, dev, steps, warmup, cpu_seconds, num_splits=0):
     B, Hq, Hkv, Lmax, D = 64, 32, 8, 32768, 128
     rng = np.random.default_rng(5)
     lens = rng.integers(8192, 32768, size=B, endpoint=True).astype(np.int32)
+    if os.environ.get("LMH_EXP_FULL_LENS"):
+        lens[:] = int(os.environ["LMH_EXP_FULL_LENS"])
     pool_rows = 1 << 18  # 256 Ki rows of 128 bf16 = 64 MiB per pool
     pools_host = [lm.f32_to_bf16_bits(rng.standard_normal((pool_rows, D), dtype=np.float32)) for _ in range(2)]
     kpool, vpool = (lm.HipArray((pool_rows, D), "bf16", dev).copy_from_host(x) for x in pools_host)
@@ -164,9 +166,9 @@ def decode_leg(lm, dev, steps, warmup, cpu_seconds):
     dq = lm.HipArray((B, Hq, D), "bf16", dev).copy_from_host(q_host)
     dl = lm.HipArray((B,), "i32", dev).copy_from_host(lens)
     out = lm.HipArray((B, Hq, D), "f32", dev)
-    ws = lm.HipArray((max(lm.binding.decode_workspace_bytes(B, Hq, Hkv, Lmax, D, 0) // 4, 4),), "f32", dev)
+    ws = lm.HipArray((max(lm.binding.decode_workspace_bytes(B, Hq, Hkv, Lmax, D, num_splits) // 4, 4),), "f32", dev)
     scale = lm.default_scale(D)
-    p = decode_params(lm, out, dq, kc, vc, dl, "bf16", scale, ws)
+    p = decode_params(lm, out, dq, kc, vc, dl, "bf16", scale, ws, num_splits=num_splits)
     fn = lambda: lm.binding.decode_attn(p)
     wall_ms, ev_ms = time_steps(fn, steps, warmup, lm.binding)
     algo_bytes = 2.0 * float(lens.sum()) * Hkv * D * 2 + B * Hq * D * 2 + B * Hq * D * 4
@@ -271,6 +273,7 @@ def main():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--only", choices=["all", "prefill", "decode", "copy"], default="all")
+    ap.add_argument("--decode-splits", type=int, default=0, help="KV splits for the decode leg (0 = library heuristic)")
     ap.add_argument("--cpu-seconds", type=float, default=15.0, help="CPU-baseline budget per leg; 0 disables it")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -303,7 +306,7 @@ def main():
         if "cpu_baseline" in r:
             line["cpu_baseline"], line["parity"] = r["cpu_baseline"], r["parity"]
     if args.only in ("all", "decode"):
-        line["decode"] = decode_leg(lm, dev, args.steps, args.warmup, args.cpu_seconds)
+        line["decode"] = decode_leg(lm, dev, args.steps, args.warmup, args.cpu_seconds, args.decode_splits)
     if args.only == "all":
         line["other_configs"] = other_configs(lm, dev)
     print(json.dumps(line))

@@ -12,14 +12,14 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIBDIR = os.path.join(HERE, "lib")
 LIBNAME = "libluminal_hip.so"
-SOURCES = ["api.hip", "prefill_valu.hip", "prefill_mfma.hip", "decode.hip", "calib.hip"]
+SOURCES = ["api.hip", "prefill_valu.hip", "prefill_mfma.hip", "decode.hip", "decode_mfma.hip", "calib.hip"]
 
 # -packed-fp32-ops: keep the compiler from forming v_pk_{add,mul,fma}_f32 out of scalar fp32 code.
 HIPCC_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fno-gpu-rdc",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wno-unused-command-line-argument",
-]
+] + os.environ.get("LMH_EXTRA_FLAGS", "").split()
 
 
 def hipcc_path():

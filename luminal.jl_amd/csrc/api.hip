@@ -283,6 +283,7 @@ int lmh_decode_attn(const lmh_decode_params *p) {
   if (a.ks[2] < p->D || a.vs[2] < p->D) return fail(LMH_E_SHAPE, "lmh_decode_attn: cache row stride smaller than head dim");
   if (a.qs[0] < 0 || a.qs[1] < 0 || a.os[0] < 0 || a.os[1] < 0) return fail(LMH_E_SHAPE, "lmh_decode_attn: negative stride");
 
+  a.mfma_ok = (p->scale > 0.f && aligned16(p->q) && a.qs[0] % 8 == 0 && a.qs[1] % 8 == 0) ? 1 : 0;
   a.num_splits = p->num_splits == 0 ? lmh_decode_auto_splits(p->B, p->Hkv, p->Lmax) : p->num_splits;
   a.chunk = decode_chunk_for(p->Lmax, a.num_splits);
   a.ws_o = nullptr;

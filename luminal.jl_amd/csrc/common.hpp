@@ -45,6 +45,7 @@ struct DecodeArgs {
   int32_t out_f32;  // out is fp32 whatever the input element type
   int32_t num_splits;
   int32_t chunk;  // keys per split
+  int32_t mfma_ok;  // q is 16-byte aligned with 8-element strides and scale > 0: the MFMA kernel may run
   float *ws_o;    // [B][Hq][num_splits][D] un-normalised partial outputs
   float *ws_ml;   // [B][Hq][num_splits][2] (running max in log2 units, partial sum)
 };
@@ -66,6 +67,8 @@ bool prefill_mfma_supported(int dtype, int D);
 int launch_prefill_mfma(const PrefillArgs &a, int dtype, hipStream_t stream);
 int launch_prefill_valu(const PrefillArgs &a, int dtype, hipStream_t stream);
 int launch_decode(const DecodeArgs &a, int dtype, hipStream_t stream);
+bool decode_mfma_supported(int dtype, int D);
+int launch_decode_mfma_split(const DecodeArgs &a, int dtype, hipStream_t stream);
 
 // Keys per split used for a given (Lmax, num_splits); always a multiple of 64.
 int decode_chunk_for(int Lmax, int num_splits);

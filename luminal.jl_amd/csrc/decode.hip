@@ -26,14 +26,30 @@ constexpr int kWaves = 4;
 constexpr int kUnroll = 4;  // key steps per wave per iteration
 constexpr float kLog2e = 1.4426950408889634f;
 
-// Sum over the LPK lanes that share a key (lane bits below LPK).
+// v_mov_b32_dpp with a compile-time lane pattern; the compiler folds it into the consuming VALU op.
+template <int CTRL>
+__device__ inline float dpp(float x) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), CTRL, 0xf, 0xf, true));
+}
+constexpr int kDppXor1 = 0xB1;        // quad_perm [1,0,3,2]
+constexpr int kDppXor2 = 0x4E;        // quad_perm [2,3,0,1]
+constexpr int kDppHalfMirror = 0x141; // lane i <- lane 7-i of its 8-lane half row
+constexpr int kDppMirror = 0x140;     // lane i <- lane 15-i of its 16-lane row
+
+// All-reduce (sum) over the LPK adjacent lanes that share a key. Up to 16 lanes this is pure DPP
+// (no LDS round trip): after the two quad steps every lane of a quad holds the quad sum, so the
+// mirror patterns, which pair quad 0 with 1 (and 2 with 3), then half row 0 with 1, finish it.
 template <int LPK>
 __device__ inline float sum_within_key(float x) {
-#pragma unroll
-  for (int off = 1; off < LPK; off <<= 1) x += __shfl_xor(x, off);
+  if (LPK >= 2) x += dpp<kDppXor1>(x);
+  if (LPK >= 4) x += dpp<kDppXor2>(x);
+  if (LPK >= 8) x += dpp<kDppHalfMirror>(x);
+  if (LPK >= 16) x += dpp<kDppMirror>(x);
+  if (LPK >= 32) x += __shfl_xor(x, 16);
+  if (LPK >= 64) x += __shfl_xor(x, 32);
   return x;
 }
-// Reduce over the key slots of a wave (lane bits at and above LPK).
+// Reductions over the key slots of a wave (lane bits at and above LPK); used once, after the loop.
 template <int LPK>
 __device__ inline float sum_across_slots(float x) {
 #pragma unroll
@@ -47,13 +63,66 @@ __device__ inline float max_across_slots(float x) {
   return x;
 }
 
+// q in the form the dot product wants: fp32 for fp32 tensors, the original packed 16-bit pairs for
+// fp16 / bf16 (v_dot2_f32_f16 / v_dot2_f32_bf16: two exact products + fp32 accumulate per op).
+template <typename E>
+struct QFrag;
+template <>
+struct QFrag<F32> {
+  float q[4];
+  __device__ void load(const float *p, bool ok) {
+#pragma unroll
+    for (int e = 0; e < 4; e++) q[e] = ok ? p[e] : 0.f;
+  }
+  __device__ float dot(const Vec128<F32> &k) const { return q[0] * k.r.x + q[1] * k.r.y + q[2] * k.r.z + q[3] * k.r.w; }
+};
+template <>
+struct QFrag<F16> {
+  uint32_t q[4];
+  __device__ void load(const _Float16 *p, bool ok) {
+    const uint16_t *u = reinterpret_cast<const uint16_t *>(p);
+#pragma unroll
+    for (int e = 0; e < 4; e++) q[e] = ok ? ((uint32_t)u[2 * e] | ((uint32_t)u[2 * e + 1] << 16)) : 0u;
+  }
+  __device__ float dot(const Vec128<F16> &k) const {
+    typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+    const uint32_t w[4] = {k.r.x, k.r.y, k.r.z, k.r.w};
+    float acc = 0.f;
+#pragma unroll
+    for (int e = 0; e < 4; e++)
+      acc = __builtin_amdgcn_fdot2(__builtin_bit_cast(h2, q[e]), __builtin_bit_cast(h2, w[e]), acc, false);
+    return acc;
+  }
+};
+template <>
+struct QFrag<BF16> {
+  uint32_t q[4];
+  __device__ void load(const uint16_t *u, bool ok) {
+#pragma unroll
+    for (int e = 0; e < 4; e++) q[e] = ok ? ((uint32_t)u[2 * e] | ((uint32_t)u[2 * e + 1] << 16)) : 0u;
+  }
+  __device__ float dot(const Vec128<BF16> &k) const {
+    typedef __bf16 b2 __attribute__((ext_vector_type(2)));
+    const uint32_t w[4] = {k.r.x, k.r.y, k.r.z, k.r.w};
+    float acc = 0.f;
+#pragma unroll
+    for (int e = 0; e < 4; e++)
+      acc = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(b2, q[e]), __builtin_bit_cast(b2, w[e]), acc, false);
+    return acc;
+  }
+};
+
 // E: element type; LPK: lanes per key row (power of two, LPK * E::kVec >= D); G: query heads
 // handled per workgroup (the GQA group, or a slice of it).
+//
+// Every key slot (a group of LPK lanes) runs its own online softmax over the keys it sees: the
+// running max, sum and output slice are slot-local, so the loop has no traffic between slots and,
+// for LPK <= 16, none through LDS at all. Slots, then waves, are merged once after the loop.
 template <typename E, int LPK, int G>
 __global__ __launch_bounds__(kWaves * 64) void decode_split_kernel(DecodeArgs a, int g_chunks) {
   using raw = typename E::raw;
   constexpr int VEC = E::kVec;
-  constexpr int KPW = 64 / LPK;                       // keys per wave per load step
+  constexpr int KPW = 64 / LPK;                          // keys per wave per load step
   constexpr int KEYS_PER_ITER = kWaves * kUnroll * KPW;  // keys per workgroup iteration
 
   const int split = blockIdx.x;
@@ -75,18 +144,16 @@ __global__ __launch_bounds__(kWaves * 64) void decode_split_kernel(DecodeArgs a,
   const int d0 = c * VEC;
   const bool lane_active = d0 < a.D;  // D is a multiple of VEC (checked on the host)
 
-  // q, pre-multiplied by scale*log2(e) so that softmax runs on exp2
-  float qf[G][VEC];
-  const float qmul = a.scale * kLog2e;
+  QFrag<E> qf[G];
 #pragma unroll
   for (int g = 0; g < G; g++) {
     const int gi = g0 + g;
     const bool head_ok = gi < group;
     const int hq = q_head_of(kvh, head_ok ? gi : 0, a.Hq, a.Hkv, a.head_map);
     const raw *qp = reinterpret_cast<const raw *>(a.q) + b * a.qs[0] + hq * a.qs[1];
-#pragma unroll
-    for (int e = 0; e < VEC; e++) qf[g][e] = (lane_active && head_ok) ? E::ld(qp[d0 + e]) * qmul : 0.f;
+    qf[g].load(qp + (lane_active ? d0 : 0), lane_active && head_ok);
   }
+  const float qmul = a.scale * kLog2e;  // scores in log2 units: softmax runs on exp2
 
   const raw *kbase = reinterpret_cast<const raw *>(a.k) + b * a.ks[0] + kvh * a.ks[1] + d0;
   const raw *vbase = reinterpret_cast<const raw *>(a.v) + b * a.vs[0] + kvh * a.vs[1] + d0;
@@ -129,23 +196,17 @@ __global__ __launch_bounds__(kWaves * 64) void decode_split_kernel(DecodeArgs a,
     for (int g = 0; g < G; g++) blk_max[g] = -INFINITY;
 #pragma unroll
     for (int u = 0; u < kUnroll; u++) {
-      float kf[VEC];
-      kr[u].unpack(kf);
 #pragma unroll
       for (int g = 0; g < G; g++) {
-        float dot = 0.f;
-#pragma unroll
-        for (int e = 0; e < VEC; e++) dot += qf[g][e] * kf[e];
-        dot = sum_within_key<LPK>(dot);
+        const float dot = sum_within_key<LPK>(qf[g].dot(kr[u])) * qmul;
         s[u][g] = valid[u] ? dot : -INFINITY;
         blk_max[g] = fmaxf(blk_max[g], s[u][g]);
       }
     }
 #pragma unroll
     for (int g = 0; g < G; g++) {
-      const float bm = max_across_slots<LPK>(blk_max[g]);
-      const float m_new = fmaxf(m[g], bm);
-      // m_new is -inf only when this wave has seen no valid key yet; then everything stays 0.
+      const float m_new = fmaxf(m[g], blk_max[g]);
+      // m_new is -inf only while this slot has seen no valid key; then everything stays 0.
       const float alpha = (m[g] == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(m[g] - m_new);
       m[g] = m_new;
       l[g] *= alpha;
@@ -166,20 +227,22 @@ __global__ __launch_bounds__(kWaves * 64) void decode_split_kernel(DecodeArgs a,
     }
   }
 
-  // Merge the key slots of each wave, then the waves of the workgroup.
+  // Merge the key slots of each wave (bring them to the wave's max first), then the waves.
   __shared__ float sm_m[kWaves][G];
   __shared__ float sm_l[kWaves][G];
   __shared__ float sm_acc[kWaves][G][LPK * VEC];
 #pragma unroll
   for (int g = 0; g < G; g++) {
-    l[g] = sum_across_slots<LPK>(l[g]);
+    const float m_wave = max_across_slots<LPK>(m[g]);
+    const float f = (m[g] == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(m[g] - m_wave);
+    l[g] = sum_across_slots<LPK>(l[g] * f);
 #pragma unroll
-    for (int e = 0; e < VEC; e++) acc[g][e] = sum_across_slots<LPK>(acc[g][e]);
+    for (int e = 0; e < VEC; e++) acc[g][e] = sum_across_slots<LPK>(acc[g][e] * f);
     if (slot == 0) {
 #pragma unroll
       for (int e = 0; e < VEC; e++) sm_acc[wave][g][d0 + e] = acc[g][e];
       if (c == 0) {
-        sm_m[wave][g] = m[g];
+        sm_m[wave][g] = m_wave;
         sm_l[wave][g] = l[g];
       }
     }
@@ -239,6 +302,15 @@ __global__ __launch_bounds__(128) void decode_merge_kernel(DecodeArgs a) {
   }
 }
 
+template <typename E>
+int launch_merge(const DecodeArgs &a, hipStream_t stream) {
+  if (a.num_splits > 1) {
+    hipLaunchKernelGGL((decode_merge_kernel<E>), dim3(a.Hq, a.B), dim3(128), 0, stream, a);
+    LMH_HIP_TRY(hipGetLastError());
+  }
+  return LMH_OK;
+}
+
 template <typename E, int LPK>
 int launch_for_lpk(const DecodeArgs &a, hipStream_t stream) {
   const int group = a.Hq / a.Hkv;
@@ -255,11 +327,7 @@ int launch_for_lpk(const DecodeArgs &a, hipStream_t stream) {
   else LMH_DECODE_LAUNCH(8);
 #undef LMH_DECODE_LAUNCH
   LMH_HIP_TRY(hipGetLastError());
-  if (a.num_splits > 1) {
-    hipLaunchKernelGGL((decode_merge_kernel<E>), dim3(a.Hq, a.B), dim3(128), 0, stream, a);
-    LMH_HIP_TRY(hipGetLastError());
-  }
-  return LMH_OK;
+  return launch_merge<E>(a, stream);
 }
 
 template <typename E>
@@ -283,6 +351,11 @@ int decode_chunk_for(int Lmax, int num_splits) {
 }
 
 int launch_decode(const DecodeArgs &a, int dtype, hipStream_t stream) {
+  if (a.mfma_ok && decode_mfma_supported(dtype, a.D)) {
+    const int rc = launch_decode_mfma_split(a, dtype, stream);
+    if (rc != LMH_OK) return rc;
+    return dtype == LMH_F16 ? launch_merge<F16>(a, stream) : launch_merge<BF16>(a, stream);
+  }
   switch (dtype) {
     case LMH_F32: return launch_for_dtype<F32>(a, stream);
     case LMH_F16: return launch_for_dtype<F16>(a, stream);
