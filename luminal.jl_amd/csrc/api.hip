@@ -218,13 +218,14 @@ int lmh_flash_attn_fwd(const lmh_attn_params *p) {
 // --------------------------------------------------------------------------------------------
 int32_t lmh_decode_auto_splits(int32_t B, int32_t Hkv, int32_t Lmax) {
   if (B <= 0 || Hkv <= 0 || Lmax <= 0) return 0;
-  // Aim for >= 4096 workgroups (16 per CU) but keep 256..1024 keys per split: shorter splits
-  // spend their time in the prologue/merge, longer ones balance ragged batches badly.
+  // The chunk (keys per split) is the unit the persistent decode kernel balances its workgroups
+  // with: aim for >= 2048 units (4 per resident workgroup) with 128..512 keys each. Shorter chunks
+  // only add partial-result slots; longer ones leave the last workgroups of a ragged batch idle.
   const int64_t pairs = (int64_t)B * Hkv;
-  int64_t want = (4096 + pairs - 1) / pairs;
+  int64_t want = (2048 + pairs - 1) / pairs;
   int64_t chunk = (Lmax + want - 1) / want;
-  if (chunk < 256) chunk = 256;
-  if (chunk > 1024) chunk = 1024;
+  if (chunk < 128) chunk = 128;
+  if (chunk > 512) chunk = 512;
   chunk = (chunk + 63) / 64 * 64;
   int64_t splits = (Lmax + chunk - 1) / chunk;
   return (int32_t)(splits < 1 ? 1 : splits);

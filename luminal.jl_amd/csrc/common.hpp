@@ -67,7 +67,7 @@ bool prefill_mfma_supported(int dtype, int D);
 int launch_prefill_mfma(const PrefillArgs &a, int dtype, hipStream_t stream);
 int launch_prefill_valu(const PrefillArgs &a, int dtype, hipStream_t stream);
 int launch_decode(const DecodeArgs &a, int dtype, hipStream_t stream);
-bool decode_mfma_supported(int dtype, int D);
+bool decode_mfma_supported(int dtype, int D, int B);
 int launch_decode_mfma_split(const DecodeArgs &a, int dtype, hipStream_t stream);
 
 // Keys per split used for a given (Lmax, num_splits); always a multiple of 64.

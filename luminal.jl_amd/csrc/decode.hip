@@ -292,11 +292,18 @@ __global__ __launch_bounds__(128) void decode_merge_kernel(DecodeArgs a) {
   float M = -INFINITY;
   for (int s = 0; s < n; s++) M = fmaxf(M, a.ws_ml[(row0 + s) * 2]);
   float lsum = 0.f;
-  for (int s = 0; s < n; s++) lsum += a.ws_ml[(row0 + s) * 2 + 1] * __builtin_amdgcn_exp2f(a.ws_ml[(row0 + s) * 2] - M);
+  for (int s = 0; s < n; s++) {
+    const float ms = a.ws_ml[(row0 + s) * 2];
+    if (ms != -INFINITY) lsum += a.ws_ml[(row0 + s) * 2 + 1] * __builtin_amdgcn_exp2f(ms - M);
+  }
   const float inv = 1.f / lsum;
   for (int d = threadIdx.x; d < a.D; d += blockDim.x) {
     float o = 0.f;
-    for (int s = 0; s < n; s++) o += a.ws_o[(row0 + s) * a.D + d] * __builtin_amdgcn_exp2f(a.ws_ml[(row0 + s) * 2] - M);
+    for (int s = 0; s < n; s++) {
+      const float ms = a.ws_ml[(row0 + s) * 2];
+      // a slot marked (-inf, 0) was folded into an earlier slot of the same run: its output row is unset
+      if (ms != -INFINITY) o += a.ws_o[(row0 + s) * a.D + d] * __builtin_amdgcn_exp2f(ms - M);
+    }
     if (a.out_f32) reinterpret_cast<float *>(a.out)[off + d] = o * inv;
     else reinterpret_cast<raw *>(a.out)[off + d] = E::st(o * inv);
   }
@@ -351,7 +358,7 @@ int decode_chunk_for(int Lmax, int num_splits) {
 }
 
 int launch_decode(const DecodeArgs &a, int dtype, hipStream_t stream) {
-  if (a.mfma_ok && decode_mfma_supported(dtype, a.D)) {
+  if (a.mfma_ok && decode_mfma_supported(dtype, a.D, a.B)) {
     const int rc = launch_decode_mfma_split(a, dtype, stream);
     if (rc != LMH_OK) return rc;
     return dtype == LMH_F16 ? launch_merge<F16>(a, stream) : launch_merge<BF16>(a, stream);

@@ -19,7 +19,16 @@
 //   O^T[d, head] += V^T P^T : A = V^T fragment via the transposing LDS read ds_read_b64_tr_b16,
 //   B = P^T = the softmax registers converted to 16 bit (never leaves the register file), as a
 //   head + remainder pair so that P keeps ~16 significant bits
-// Split-KV partials and the merge kernel are shared with decode.hip.
+//
+// Scheduling: a rectangular (split, kv head, batch) grid wastes a ragged batch twice — workgroups
+// whose split lies past kv_len[b] still have to be dispatched (≈40 % of the grid for lengths spread
+// over [Lmax/4, Lmax]), and every workgroup pays its own ramp-up. Instead the kernel is persistent:
+// the launch has as many workgroups as fit on the chip, every workgroup builds the prefix sum of
+// ceil(kv_len[b] / chunk) over the batch in LDS, and takes an equal, contiguous share of the
+// existing (b, kv head, chunk) units. Inside its share it streams through maximal runs of chunks of
+// one (b, kv head) with a single softmax state, so partials are written once per run, not once per
+// chunk (the other chunk slots of the run get an "empty" marker the merge kernel skips).
+// Split-KV partial layout and the merge kernel are shared with decode.hip.
 #include "common.hpp"
 #include "dtypes.hpp"
 
@@ -58,6 +67,8 @@ __device__ inline void wave_lds_fence() {
   __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 }
 
+constexpr int kMaxBatchPersistent = 1024;  // prefix sums live in LDS
+
 template <typename MT, int D>
 __global__ __launch_bounds__(kWaves * 64) void decode_mfma_kernel(DecodeArgs a, int g_chunks) {
   using vec8 = typename MT::vec8;
@@ -71,26 +82,63 @@ __global__ __launch_bounds__(kWaves * 64) void decode_mfma_kernel(DecodeArgs a, 
   constexpr int kMergeBytes = kWaves * 16 * (D + 2) * 4;
   constexpr int kSmemBytes = kWaves * kTileBytes > kMergeBytes ? kWaves * kTileBytes : kMergeBytes;
   __shared__ __attribute__((aligned(16))) unsigned char smem[kSmemBytes];
-
-  const int split = blockIdx.x;
-  const int kvh = blockIdx.y / g_chunks;
-  const int g0 = (blockIdx.y % g_chunks) * 16;  // first group member handled here
-  const int b = blockIdx.z;
-  const int group = a.Hq / a.Hkv;
-  const int n_heads = min(16, group - g0);
-
-  int L = a.kv_len ? a.kv_len[b] : a.Lmax;
-  L = min(max(L, 0), a.Lmax);
-  const int start = split * a.chunk;
-  if (start >= L) return;  // ragged tail: this split does not exist for sequence b
-  const int end = min(L, start + a.chunk);
+  __shared__ int s_pref[kMaxBatchPersistent + 1];  // s_pref[b] = chunks of sequences 0..b-1
 
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = tid >> 6;
   const int n = lane & 15, g = lane >> 4;
+  const int group = a.Hq / a.Hkv;
+  const int kv_slots = a.Hkv * g_chunks;  // (kv head, slice of <= 16 group members) pairs
+
+  // ---- this workgroup's share of the (b, kv slot, chunk) units ----
+  for (int i = tid; i < a.B; i += kWaves * 64) {
+    int L = a.kv_len ? a.kv_len[i] : a.Lmax;
+    L = min(max(L, 0), a.Lmax);
+    s_pref[i + 1] = (L + a.chunk - 1) / a.chunk;
+  }
+  __syncthreads();
+  if (tid == 0) {
+    int run = 0;
+    s_pref[0] = 0;
+    for (int i = 1; i <= a.B; i++) {
+      run += s_pref[i];
+      s_pref[i] = run;
+    }
+  }
+  __syncthreads();
+  const int64_t total_units = (int64_t)s_pref[a.B] * kv_slots;
+  int64_t u = total_units * blockIdx.x / gridDim.x;
+  const int64_t u_end = total_units * (blockIdx.x + 1) / gridDim.x;
 
   uint16_t *Ks = reinterpret_cast<uint16_t *>(smem + wave * kTileBytes);
   uint16_t *Vs = Ks + kBlk * LDK;
+  const float c = a.scale * kLog2e;
+  const int k_frag_off = n * LDK + 8 * g;                             // + 16*hb*LDK + 32*ks
+  const int v_frag_off = (4 * g + (n >> 2)) * LDV + 4 * (n & 3);      // + 16*hb*LDV + 16*db
+
+  while (u < u_end) {
+    // segment = the maximal run of units of one (b, kv slot) inside [u, u_end)
+    int lo = 0, hi = a.B;  // largest b with s_pref[b] * kv_slots <= u
+    while (hi - lo > 1) {
+      const int mid = (lo + hi) >> 1;
+      if ((int64_t)s_pref[mid] * kv_slots <= u) lo = mid; else hi = mid;
+    }
+    const int b = lo;
+    const int n_chunks = s_pref[b + 1] - s_pref[b];
+    const int64_t rem = u - (int64_t)s_pref[b] * kv_slots;
+    const int slot_id = (int)(rem / n_chunks);
+    const int c0 = (int)(rem % n_chunks);
+    const int c1 = (int)min((int64_t)n_chunks, c0 + (u_end - u));
+    u += c1 - c0;
+    const int kvh = slot_id / g_chunks;
+    const int g0 = (slot_id % g_chunks) * 16;  // first group member handled here
+    const int n_heads = min(16, group - g0);
+    int L = a.kv_len ? a.kv_len[b] : a.Lmax;
+    L = min(max(L, 0), a.Lmax);
+    const int start = c0 * a.chunk;
+    const int end = min(L, c1 * a.chunk);
+    const int split = c0;
+
 
   // Q^T fragments (B operand): lane (head n, g) holds q[head][32*ks + 8*g .. +7]; zero for padding heads
   vec8 qreg[KS];
@@ -114,7 +162,6 @@ __global__ __launch_bounds__(kWaves * 64) void decode_mfma_kernel(DecodeArgs a, 
   for (int db = 0; db < DB; db++) oacc[db] = floatx4_t{0.f, 0.f, 0.f, 0.f};
   float m_i = -INFINITY;  // running max of the raw scores of head n (same in the 4 lanes of a head)
   float l_i = 0.f;        // this lane's share of the running sum
-  const float c = a.scale * kLog2e;
 
   uint4 kreg[NL], vreg[NL];
   auto load_tile = [&](int key0) {
@@ -140,9 +187,6 @@ __global__ __launch_bounds__(kWaves * 64) void decode_mfma_kernel(DecodeArgs a, 
       *reinterpret_cast<uint4 *>(&Vs[row * LDV + col * 8]) = vreg[r];
     }
   };
-
-  const int k_frag_off = n * LDK + 8 * g;                             // + 16*hb*LDK + 32*ks
-  const int v_frag_off = (4 * g + (n >> 2)) * LDV + 4 * (n & 3);      // + 16*hb*LDV + 16*db
 
   const int n_blocks = (end - start + kBlk - 1) / kBlk;
   if (wave < n_blocks) load_tile(start + wave * kBlk);
@@ -256,14 +300,37 @@ __global__ __launch_bounds__(kWaves * 64) void decode_mfma_kernel(DecodeArgs a, 
       }
     }
   }
+  // the other chunk slots of this run hold nothing: mark them so the merge kernel skips them
+  if (a.num_splits > 1) {
+    for (int idx = tid; idx < n_heads * (c1 - c0 - 1); idx += kWaves * 64) {
+      const int h = idx / (c1 - c0 - 1), cs = c0 + 1 + idx % (c1 - c0 - 1);
+      const int hq = q_head_of(kvh, g0 + h, a.Hq, a.Hkv, a.head_map);
+      const int64_t row = ((int64_t)b * a.Hq + hq) * a.num_splits + cs;
+      a.ws_ml[row * 2 + 0] = -INFINITY;
+      a.ws_ml[row * 2 + 1] = 0.f;
+    }
+  }
+  __syncthreads();  // the merge buffers are tile memory again in the next segment
+  }  // while (u < u_end)
 }
 
 template <typename MT, int D>
 int launch_for_d(const DecodeArgs &a, hipStream_t stream) {
+  // Persistent launch: as many workgroups as the chip holds at once (never more than there are units).
+  static int wgs_per_device = 0;  // same for every device this library runs on (gfx950 only)
+  if (wgs_per_device == 0) {
+    int dev = 0, per_cu = 0;
+    hipDeviceProp_t prop;
+    LMH_HIP_TRY(hipGetDevice(&dev));
+    LMH_HIP_TRY(hipGetDeviceProperties(&prop, dev));
+    LMH_HIP_TRY(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, decode_mfma_kernel<MT, D>, kWaves * 64, 0));
+    wgs_per_device = (per_cu < 1 ? 1 : per_cu) * prop.multiProcessorCount;
+  }
   const int group = a.Hq / a.Hkv;
   const int g_chunks = (group + 15) / 16;
-  dim3 grid(a.num_splits, a.Hkv * g_chunks, a.B), block(kWaves * 64);
-  hipLaunchKernelGGL((decode_mfma_kernel<MT, D>), grid, block, 0, stream, a, g_chunks);
+  const int64_t max_units = (int64_t)a.B * a.Hkv * g_chunks * a.num_splits;
+  const int n_wgs = (int)(max_units < wgs_per_device ? max_units : wgs_per_device);
+  hipLaunchKernelGGL((decode_mfma_kernel<MT, D>), dim3(n_wgs), dim3(kWaves * 64), 0, stream, a, g_chunks);
   LMH_HIP_TRY(hipGetLastError());
   return LMH_OK;
 }
@@ -281,8 +348,9 @@ int launch_for_type(const DecodeArgs &a, hipStream_t stream) {
 
 }  // namespace
 
-bool decode_mfma_supported(int dtype, int D) {
-  return (dtype == LMH_F16 || dtype == LMH_BF16) && (D == 64 || D == 96 || D == 128 || D == 256);
+bool decode_mfma_supported(int dtype, int D, int B) {
+  return (dtype == LMH_F16 || dtype == LMH_BF16) && (D == 64 || D == 96 || D == 128 || D == 256) &&
+         B <= kMaxBatchPersistent;
 }
 
 // Enqueues only the split kernel; the caller adds the merge kernel when num_splits > 1.
