@@ -207,6 +207,8 @@ int lmh_flash_attn_fwd(const lmh_attn_params *p) {
   // The matrix-core kernel does 128-bit accesses and tracks the max on raw scores (needs scale>0).
   bool mfma_ok = prefill_mfma_supported(p->dtype, p->D) && p->scale > 0.f && aligned16(p->q) && aligned16(p->k) &&
                  aligned16(p->v) && aligned16(p->out);
+  // its K/V tiles are fetched with 32-bit buffer offsets inside one (b, kv head) slice
+  mfma_ok = mfma_ok && (int64_t)p->Sk * a.ks[2] * 2 < (int64_t(1) << 31) && (int64_t)p->Sk * a.vs[2] * 2 < (int64_t(1) << 31);
   for (int i = 0; i < 3 && mfma_ok; i++)
     mfma_ok = (a.qs[i] % 8 == 0) && (a.ks[i] % 8 == 0) && (a.vs[i] % 8 == 0) && (a.os[i] % 8 == 0);
   if (mfma_ok) return launch_prefill_mfma(a, p->dtype, (hipStream_t)p->stream);

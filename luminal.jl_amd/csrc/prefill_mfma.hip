@@ -29,27 +29,59 @@ namespace {
 
 constexpr int BM = 128;  // query rows per workgroup
 constexpr int BN = 64;   // keys per tile
-constexpr int kPad = 8;  // LDS row padding in elements (16 B): spreads rows over the banks
+#ifndef LMH_PREFILL_PAD
+#define LMH_PREFILL_PAD 8
+#endif
+constexpr int kPad = LMH_PREFILL_PAD;  // LDS row padding in elements: spreads rows over the banks
 constexpr float kLog2e = 1.4426950408889634f;
+// The running max is only raised (and the output rescaled) when a row's scores outgrow it by more
+// than this many powers of two; until then P is computed against the stale max and may reach
+// 2^kLazyRescale, which fp16/bf16/fp32 all hold. The quotient O / l does not depend on the reference
+// max, so the result is unchanged while most tiles skip the D-wide rescale.
+constexpr float kLazyRescale = 8.0f;
+typedef unsigned int u32x4_t __attribute__((ext_vector_type(4)));
 
 typedef short shortx8_t __attribute__((ext_vector_type(8)));
 typedef __attribute__((address_space(3))) shortx4_t lds_shortx4_t;
 
 struct MfmaF16 {
   using vec8 = half8_t;
+  static constexpr bool kSplitP = false;  // 11 significant bits in P are within the 2e-3 budget
   __device__ static floatx16_t mfma(vec8 a, vec8 b, floatx16_t c) {
     return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
   }
   __device__ static uint16_t cvt_bits(float x) { return __builtin_bit_cast(uint16_t, (_Float16)x); }
   __device__ static _Float16 cvt(float x) { return (_Float16)x; }
+  // acc + sum of the 8 (already rounded) elements: 4 x v_dot2_f32_f16 against (1, 1)
+  __device__ static float sum8(vec8 p, float acc) {
+    typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+    const h2 one = {(_Float16)1.f, (_Float16)1.f};
+    acc = __builtin_amdgcn_fdot2(__builtin_shufflevector(p, p, 0, 1), one, acc, false);
+    acc = __builtin_amdgcn_fdot2(__builtin_shufflevector(p, p, 2, 3), one, acc, false);
+    acc = __builtin_amdgcn_fdot2(__builtin_shufflevector(p, p, 4, 5), one, acc, false);
+    acc = __builtin_amdgcn_fdot2(__builtin_shufflevector(p, p, 6, 7), one, acc, false);
+    return acc;
+  }
 };
 struct MfmaBF16 {
   using vec8 = bf16x8_t;
+  // A bf16 P has 8 significant bits; on short or peaked rows that alone is ~2.5e-3 of the output
+  // range. P is therefore fed to the matrix cores as head + remainder (two MFMAs per V fragment).
+  static constexpr bool kSplitP = true;
   __device__ static floatx16_t mfma(vec8 a, vec8 b, floatx16_t c) {
     return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
   }
   __device__ static uint16_t cvt_bits(float x) { return f32_to_bf16_bits(x); }
   __device__ static __bf16 cvt(float x) { return (__bf16)x; }
+  __device__ static float sum8(vec8 p, float acc) {
+    typedef __bf16 b2 __attribute__((ext_vector_type(2)));
+    const b2 one = {(__bf16)1.f, (__bf16)1.f};
+    acc = __builtin_amdgcn_fdot2_f32_bf16(__builtin_shufflevector(p, p, 0, 1), one, acc, false);
+    acc = __builtin_amdgcn_fdot2_f32_bf16(__builtin_shufflevector(p, p, 2, 3), one, acc, false);
+    acc = __builtin_amdgcn_fdot2_f32_bf16(__builtin_shufflevector(p, p, 4, 5), one, acc, false);
+    acc = __builtin_amdgcn_fdot2_f32_bf16(__builtin_shufflevector(p, p, 6, 7), one, acc, false);
+    return acc;
+  }
 };
 
 template <typename MT, int D, bool CAUSAL>
@@ -61,8 +93,8 @@ __global__ __launch_bounds__(256, 2) void prefill_mfma_kernel(PrefillArgs a, int
   constexpr int CH = BN * CPR / 256;  // chunks per thread per tile
   constexpr int LDW = D + kPad;    // LDS row stride in elements
 
-  __shared__ __attribute__((aligned(16))) uint16_t Ks[BN * LDW];
-  __shared__ __attribute__((aligned(16))) uint16_t Vs[BN * LDW];
+  __shared__ __attribute__((aligned(16))) uint16_t Ks2[2][BN * LDW];  // double-buffered tiles
+  __shared__ __attribute__((aligned(16))) uint16_t Vs2[2][BN * LDW];
 
   // ---- which (b, hq, query tile) this workgroup owns ----
   const int bid = blockIdx.x;
@@ -111,30 +143,37 @@ __global__ __launch_bounds__(256, 2) void prefill_mfma_kernel(PrefillArgs a, int
   float l_i = 0.f;        // this lane's half of the running sum
   const float c = a.scale * kLog2e;
 
-  // ---- tile staging: global -> registers (prefetch) -> LDS ----
-  uint4 kreg[CH], vreg[CH];
+  // ---- tile staging: global -> registers (prefetched two tiles ahead) -> LDS ----
+  // Buffer loads: the descriptor's size is the end of the last valid key row, so rows past n_keys
+  // read as zero without a branch, and the per-lane byte offsets are loop invariants — a tile costs
+  // one scalar offset update instead of per-lane 64-bit address arithmetic.
+  const __amdgpu_buffer_rsrc_t k_rsrc =
+      __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t *>(kp), 0, (int)((int64_t)n_keys * a.ks[2] * 2), 0x00020000);
+  const __amdgpu_buffer_rsrc_t v_rsrc =
+      __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t *>(vp), 0, (int)((int64_t)n_keys * a.vs[2] * 2), 0x00020000);
+  int k_voff[CH], v_voff[CH], lds_off[CH];
+#pragma unroll
+  for (int r = 0; r < CH; r++) {
+    const int id = tid + 256 * r;
+    const int row = id / CPR, col = id % CPR;
+    k_voff[r] = (int)((row * a.ks[2] + col * 8) * 2);
+    v_voff[r] = (int)((row * a.vs[2] + col * 8) * 2);
+    lds_off[r] = row * LDW + col * 8;
+  }
+  const int k_tile_bytes = (int)(BN * a.ks[2] * 2), v_tile_bytes = (int)(BN * a.vs[2] * 2);
+  u32x4_t kreg[CH], vreg[CH];
   auto load_tile = [&](int kt) {
-    const int k0 = kt * BN;
 #pragma unroll
     for (int r = 0; r < CH; r++) {
-      const int id = tid + 256 * r;
-      const int row = id / CPR, col = id % CPR;
-      const int key = k0 + row;
-      kreg[r] = make_uint4(0, 0, 0, 0);
-      vreg[r] = make_uint4(0, 0, 0, 0);
-      if (key < n_keys) {
-        kreg[r] = *reinterpret_cast<const uint4 *>(kp + (int64_t)key * a.ks[2] + col * 8);
-        vreg[r] = *reinterpret_cast<const uint4 *>(vp + (int64_t)key * a.vs[2] + col * 8);
-      }
+      kreg[r] = __builtin_amdgcn_raw_buffer_load_b128(k_rsrc, k_voff[r], kt * k_tile_bytes, 0);
+      vreg[r] = __builtin_amdgcn_raw_buffer_load_b128(v_rsrc, v_voff[r], kt * v_tile_bytes, 0);
     }
   };
-  auto store_tile = [&]() {
+  auto store_tile = [&](int buf) {
 #pragma unroll
     for (int r = 0; r < CH; r++) {
-      const int id = tid + 256 * r;
-      const int row = id / CPR, col = id % CPR;
-      *reinterpret_cast<uint4 *>(&Ks[row * LDW + col * 8]) = kreg[r];
-      *reinterpret_cast<uint4 *>(&Vs[row * LDW + col * 8]) = vreg[r];
+      *reinterpret_cast<u32x4_t *>(&Ks2[buf][lds_off[r]]) = kreg[r];
+      *reinterpret_cast<u32x4_t *>(&Vs2[buf][lds_off[r]]) = vreg[r];
     }
   };
 
@@ -146,13 +185,20 @@ __global__ __launch_bounds__(256, 2) void prefill_mfma_kernel(PrefillArgs a, int
   const int v_frag_off = (4 * g + (i16 >> 2)) * LDW + 16 * ((lane >> 4) & 1) + 4 * (i16 & 3);
   // + (kb*32 + 16*t [+8]) * LDW + db*32
 
-  if (n_kv_tiles > 0) load_tile(0);
+  if (n_kv_tiles > 0) {
+    load_tile(0);
+    store_tile(0);
+  }
+  if (n_kv_tiles > 1) load_tile(1);
 
   for (int kt = 0; kt < n_kv_tiles; kt++) {
-    __syncthreads();  // every wave is done reading the previous tile
-    store_tile();
+    // One barrier per tile: tile kt (written one iteration ago) becomes visible, and every wave is
+    // done with tile kt-1, whose buffer now takes tile kt+1 from the registers.
     __syncthreads();
-    if (kt + 1 < n_kv_tiles) load_tile(kt + 1);  // in flight while this tile is computed
+    if (kt + 1 < n_kv_tiles) store_tile((kt + 1) & 1);
+    if (kt + 2 < n_kv_tiles) load_tile(kt + 2);  // in flight while tiles kt and kt+1 are computed
+    const uint16_t *Ks = Ks2[kt & 1];
+    const uint16_t *Vs = Vs2[kt & 1];
 
     const int k0 = kt * BN;
     if (CAUSAL && k0 > wave_q_hi) continue;  // whole tile above this wave's diagonal
@@ -192,24 +238,32 @@ __global__ __launch_bounds__(256, 2) void prefill_mfma_kernel(PrefillArgs a, int
 #pragma unroll
       for (int i = 0; i < 16; i++) mx = fmaxf(mx, sacc[kb][i]);
     mx = fmaxf(mx, __shfl_xor(mx, 32));
-    const float m_new = fmaxf(m_i, mx);  // finite: key 0 is visible to every query
-    const float alpha = __builtin_amdgcn_exp2f((m_i - m_new) * c);
-    const float mc = m_new * c;
-    m_i = m_new;
-    float psum = 0.f;
+    // m_i is finite after the first tile (key 0 is visible to every query); -inf before it.
+    if (__builtin_amdgcn_ballot_w64((mx - m_i) * c > kLazyRescale) != 0) {  // wave-uniform
+      const float m_new = fmaxf(m_i, mx);
+      const float alpha = __builtin_amdgcn_exp2f((m_i - m_new) * c);
+      m_i = m_new;
+      l_i *= alpha;
+#pragma unroll
+      for (int db = 0; db < DB; db++)
+#pragma unroll
+        for (int i = 0; i < 16; i++) oacc[db][i] *= alpha;
+    }
+    const float mc = m_i * c;
+    vec8 pf[2][2], pf_lo[2][2];
 #pragma unroll
     for (int kb = 0; kb < 2; kb++)
 #pragma unroll
-      for (int i = 0; i < 16; i++) {
-        const float p = __builtin_amdgcn_exp2f(sacc[kb][i] * c - mc);
-        sacc[kb][i] = p;
-        psum += p;
+      for (int t = 0; t < 2; t++) {
+#pragma unroll
+        for (int e = 0; e < 8; e++) {
+          const float p = __builtin_amdgcn_exp2f(sacc[kb][8 * t + e] * c - mc);
+          pf[kb][t][e] = MT::cvt(p);
+          if (MT::kSplitP) pf_lo[kb][t][e] = MT::cvt(p - (float)pf[kb][t][e]);
+        }
+        l_i = MT::sum8(pf[kb][t], l_i);
+        if (MT::kSplitP) l_i = MT::sum8(pf_lo[kb][t], l_i);
       }
-    l_i = l_i * alpha + psum;
-#pragma unroll
-    for (int db = 0; db < DB; db++)
-#pragma unroll
-      for (int i = 0; i < 16; i++) oacc[db][i] *= alpha;
 
     // ---- O^T += V^T P^T ----
 #pragma unroll
@@ -217,16 +271,14 @@ __global__ __launch_bounds__(256, 2) void prefill_mfma_kernel(PrefillArgs a, int
       if (kb == 1 && !blk1_active) continue;
 #pragma unroll
       for (int t = 0; t < 2; t++) {
-        vec8 pf;
-#pragma unroll
-        for (int e = 0; e < 8; e++) pf[e] = MT::cvt(sacc[kb][8 * t + e]);
 #pragma unroll
         for (int db = 0; db < DB; db++) {
           const uint16_t *vaddr = &Vs[v_frag_off + (kb * 32 + 16 * t) * LDW + db * 32];
           const shortx4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_shortx4_t *)(vaddr));
           const shortx4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_shortx4_t *)(vaddr + 8 * LDW));
           const shortx8_t v8 = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-          oacc[db] = MT::mfma(__builtin_bit_cast(vec8, v8), pf, oacc[db]);
+          oacc[db] = MT::mfma(__builtin_bit_cast(vec8, v8), pf[kb][t], oacc[db]);
+          if (MT::kSplitP) oacc[db] = MT::mfma(__builtin_bit_cast(vec8, v8), pf_lo[kb][t], oacc[db]);
         }
       }
     }
