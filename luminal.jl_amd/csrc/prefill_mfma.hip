@@ -17,8 +17,8 @@
 //   * K and V tiles (64 keys) are staged row-major in LDS; the K fragment is a plain 128-bit LDS
 //     read (contraction over the contiguous head dim), the V^T fragment uses the gfx950 transposing
 //     LDS read ds_read_b64_tr_b16, which hands each lane 4 consecutive keys of its head-dim column;
-//   * causal: key tiles beyond the workgroup's last query are never loaded, a wave skips tiles (and
-//     32-key blocks) that lie entirely above its diagonal, and only diagonal tiles pay for masking;
+//   * causal: key tiles beyond the workgroup's last query are never loaded, a wave skips tiles that
+//     lie entirely above its diagonal, and only diagonal tiles pay for masking;
 //   * blockIdx -> work mapping keeps all query tiles of a head on one XCD (private L2) and, for
 //     causal, issues the long rows first.
 #include "common.hpp"
@@ -29,10 +29,19 @@ namespace {
 
 constexpr int BM = 128;  // query rows per workgroup
 constexpr int BN = 64;   // keys per tile
-#ifndef LMH_PREFILL_PAD
-#define LMH_PREFILL_PAD 8
+#ifndef LMH_PREFILL_WAVES
+#define LMH_PREFILL_WAVES 2
 #endif
-constexpr int kPad = LMH_PREFILL_PAD;  // LDS row padding in elements: spreads rows over the banks
+#ifndef LMH_PREFILL_PADK
+#define LMH_PREFILL_PADK 8
+#endif
+#ifndef LMH_PREFILL_PADV
+#define LMH_PREFILL_PADV 0
+#endif
+// LDS row paddings in elements; K rows are read 16 bytes per lane (one row per lane), V rows through
+// the transposing read (4 rows x 32 bytes per 16 lanes), so the two tiles want different strides.
+constexpr int kPadK = LMH_PREFILL_PADK;
+constexpr int kPadV = LMH_PREFILL_PADV;
 constexpr float kLog2e = 1.4426950408889634f;
 // The running max is only raised (and the output rescaled) when a row's scores outgrow it by more
 // than this many powers of two; until then P is computed against the stale max and may reach
@@ -85,16 +94,17 @@ struct MfmaBF16 {
 };
 
 template <typename MT, int D, bool CAUSAL>
-__global__ __launch_bounds__(256, 2) void prefill_mfma_kernel(PrefillArgs a, int n_q_tiles, int n_bh_groups) {
+__global__ __launch_bounds__(256, LMH_PREFILL_WAVES) void prefill_mfma_kernel(PrefillArgs a, int n_q_tiles, int n_bh_groups) {
   using vec8 = typename MT::vec8;
   constexpr int KS = D / 16;       // k-steps of the S^T product
   constexpr int DB = D / 32;       // 32-row blocks of O^T
   constexpr int CPR = D / 8;       // 16-byte chunks per K/V row
   constexpr int CH = BN * CPR / 256;  // chunks per thread per tile
-  constexpr int LDW = D + kPad;    // LDS row stride in elements
+  constexpr int LDK = D + kPadK;   // LDS row strides in elements
+  constexpr int LDV = D + kPadV;
 
-  __shared__ __attribute__((aligned(16))) uint16_t Ks2[2][BN * LDW];  // double-buffered tiles
-  __shared__ __attribute__((aligned(16))) uint16_t Vs2[2][BN * LDW];
+  __shared__ __attribute__((aligned(16))) uint16_t Ks2[2][BN * LDK];  // double-buffered tiles
+  __shared__ __attribute__((aligned(16))) uint16_t Vs2[2][BN * LDV];
 
   // ---- which (b, hq, query tile) this workgroup owns ----
   const int bid = blockIdx.x;
@@ -151,14 +161,15 @@ __global__ __launch_bounds__(256, 2) void prefill_mfma_kernel(PrefillArgs a, int
       __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t *>(kp), 0, (int)((int64_t)n_keys * a.ks[2] * 2), 0x00020000);
   const __amdgpu_buffer_rsrc_t v_rsrc =
       __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t *>(vp), 0, (int)((int64_t)n_keys * a.vs[2] * 2), 0x00020000);
-  int k_voff[CH], v_voff[CH], lds_off[CH];
+  int k_voff[CH], v_voff[CH], k_lds_off[CH], v_lds_off[CH];
 #pragma unroll
   for (int r = 0; r < CH; r++) {
     const int id = tid + 256 * r;
     const int row = id / CPR, col = id % CPR;
     k_voff[r] = (int)((row * a.ks[2] + col * 8) * 2);
     v_voff[r] = (int)((row * a.vs[2] + col * 8) * 2);
-    lds_off[r] = row * LDW + col * 8;
+    k_lds_off[r] = row * LDK + col * 8;
+    v_lds_off[r] = row * LDV + col * 8;
   }
   const int k_tile_bytes = (int)(BN * a.ks[2] * 2), v_tile_bytes = (int)(BN * a.vs[2] * 2);
   u32x4_t kreg[CH], vreg[CH];
@@ -172,18 +183,18 @@ __global__ __launch_bounds__(256, 2) void prefill_mfma_kernel(PrefillArgs a, int
   auto store_tile = [&](int buf) {
 #pragma unroll
     for (int r = 0; r < CH; r++) {
-      *reinterpret_cast<u32x4_t *>(&Ks2[buf][lds_off[r]]) = kreg[r];
-      *reinterpret_cast<u32x4_t *>(&Vs2[buf][lds_off[r]]) = vreg[r];
+      *reinterpret_cast<u32x4_t *>(&Ks2[buf][k_lds_off[r]]) = kreg[r];
+      *reinterpret_cast<u32x4_t *>(&Vs2[buf][v_lds_off[r]]) = vreg[r];
     }
   };
 
   // lane-constant pieces of the LDS addresses
-  const int k_frag_off = n * LDW + 8 * g;  // + kb*32*LDW + 16*ks
+  const int k_frag_off = n * LDK + 8 * g;  // + kb*32*LDK + 16*ks
   // transposing V read: within each 16-lane block, lane i supplies row (i / 4) and 4-column group
   // (i % 4) of a 4-key x 16-column patch and receives the 4 keys of column i.
   const int i16 = lane & 15;
-  const int v_frag_off = (4 * g + (i16 >> 2)) * LDW + 16 * ((lane >> 4) & 1) + 4 * (i16 & 3);
-  // + (kb*32 + 16*t [+8]) * LDW + db*32
+  const int v_frag_off = (4 * g + (i16 >> 2)) * LDV + 16 * ((lane >> 4) & 1) + 4 * (i16 & 3);
+  // + (kb*32 + 16*t [+8]) * LDV + db*32
 
   if (n_kv_tiles > 0) {
     load_tile(0);
@@ -202,22 +213,24 @@ __global__ __launch_bounds__(256, 2) void prefill_mfma_kernel(PrefillArgs a, int
 
     const int k0 = kt * BN;
     if (CAUSAL && k0 > wave_q_hi) continue;  // whole tile above this wave's diagonal
-    const bool blk1_active = !(CAUSAL && k0 + 32 > wave_q_hi);
 
-    // ---- S^T = K Q^T for two 32-key blocks ----
+    // ---- S^T = K Q^T for two 32-key blocks: all fragments are fetched first, then the two
+    // accumulator chains alternate so that neither waits on LDS or on its own previous MFMA ----
+    vec8 kf[2][KS];
+#pragma unroll
+    for (int ks = 0; ks < KS; ks++)
+#pragma unroll
+      for (int kb = 0; kb < 2; kb++)
+        kf[kb][ks] = *reinterpret_cast<const vec8 *>(&Ks[k_frag_off + kb * 32 * LDK + 16 * ks]);
     floatx16_t sacc[2];
 #pragma unroll
-    for (int kb = 0; kb < 2; kb++) {
+    for (int kb = 0; kb < 2; kb++)
 #pragma unroll
       for (int i = 0; i < 16; i++) sacc[kb][i] = 0.f;
-      if (kb == 0 || blk1_active) {
 #pragma unroll
-        for (int ks = 0; ks < KS; ks++) {
-          const vec8 kf = *reinterpret_cast<const vec8 *>(&Ks[k_frag_off + kb * 32 * LDW + 16 * ks]);
-          sacc[kb] = MT::mfma(kf, qreg[ks], sacc[kb]);
-        }
-      }
-    }
+    for (int ks = 0; ks < KS; ks++)
+#pragma unroll
+      for (int kb = 0; kb < 2; kb++) sacc[kb] = MT::mfma(kf[kb][ks], qreg[ks], sacc[kb]);
 
     // ---- masking (diagonal tiles and the ragged last tile only) ----
     const bool need_mask = (k0 + BN > n_keys) || (CAUSAL && k0 + BN - 1 > wave_q_lo);
@@ -268,14 +281,13 @@ __global__ __launch_bounds__(256, 2) void prefill_mfma_kernel(PrefillArgs a, int
     // ---- O^T += V^T P^T ----
 #pragma unroll
     for (int kb = 0; kb < 2; kb++) {
-      if (kb == 1 && !blk1_active) continue;
 #pragma unroll
       for (int t = 0; t < 2; t++) {
 #pragma unroll
         for (int db = 0; db < DB; db++) {
-          const uint16_t *vaddr = &Vs[v_frag_off + (kb * 32 + 16 * t) * LDW + db * 32];
+          const uint16_t *vaddr = &Vs[v_frag_off + (kb * 32 + 16 * t) * LDV + db * 32];
           const shortx4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_shortx4_t *)(vaddr));
-          const shortx4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_shortx4_t *)(vaddr + 8 * LDW));
+          const shortx4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_shortx4_t *)(vaddr + 8 * LDV));
           const shortx8_t v8 = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
           oacc[db] = MT::mfma(__builtin_bit_cast(vec8, v8), pf[kb][t], oacc[db]);
           if (MT::kSplitP) oacc[db] = MT::mfma(__builtin_bit_cast(vec8, v8), pf_lo[kb][t], oacc[db]);
