@@ -32,6 +32,9 @@ constexpr int BN = 64;   // keys per tile
 #ifndef LMH_PREFILL_WAVES
 #define LMH_PREFILL_WAVES 2
 #endif
+#ifndef LMH_PREFILL_PAIR
+#define LMH_PREFILL_PAIR 0
+#endif
 #ifndef LMH_PREFILL_PADK
 #define LMH_PREFILL_PADK 8
 #endif
@@ -115,8 +118,14 @@ __global__ __launch_bounds__(256, LMH_PREFILL_WAVES) void prefill_mfma_kernel(Pr
   if (bh >= a.B * a.Hq) return;
   const int b = bh / a.Hq, hq = bh % a.Hq;
   const int kvh = kv_head_of(hq, a.Hq, a.Hkv, a.head_map);
-  const int q_tile = CAUSAL ? (n_q_tiles - 1 - tile_rank) : tile_rank;
+  // Causal rows grow with the query index, so a workgroup takes query tile (n - 1 - r) and then
+  // tile r: every workgroup of a head then does the same amount of work and the launch has no
+  // long tail of late, heavy tiles. Without a mask all tiles cost the same and r is the tile.
+  const int n_pass = (CAUSAL && LMH_PREFILL_PAIR && tile_rank != n_q_tiles - 1 - tile_rank) ? 2 : 1;
+  for (int pass = 0; pass < n_pass; pass++) {
+  const int q_tile = (CAUSAL && pass == 0) ? (n_q_tiles - 1 - tile_rank) : tile_rank;
   const int q0 = q_tile * BM;
+  if (pass > 0) __syncthreads();  // the tiles of the previous pass are no longer read
 
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = tid >> 6;
@@ -322,13 +331,15 @@ __global__ __launch_bounds__(256, LMH_PREFILL_WAVES) void prefill_mfma_kernel(Pr
         *reinterpret_cast<uint2 *>(op + d) = packed;
       }
   }
+  }  // pass
 }
 
 template <typename MT, int D>
 int launch_for_d(const PrefillArgs &a, hipStream_t stream) {
   const int n_q_tiles = (a.Sq + BM - 1) / BM;
   const int n_bh_groups = (a.B * a.Hq + 7) / 8;
-  dim3 grid(8 * n_bh_groups * n_q_tiles), block(256);
+  const int n_ranks = (a.causal && LMH_PREFILL_PAIR) ? (n_q_tiles + 1) / 2 : n_q_tiles;
+  dim3 grid(8 * n_bh_groups * n_ranks), block(256);
   if (a.causal)
     hipLaunchKernelGGL((prefill_mfma_kernel<MT, D, true>), grid, block, 0, stream, a, n_q_tiles, n_bh_groups);
   else
