@@ -32,6 +32,12 @@ sys.path.insert(0, ROOT)
 
 PEAK_FP16_TFLOPS = 2500.0  # MI355X dense fp16/bf16 MFMA
 PEAK_HBM_GBS = 8000.0      # MI355X HBM3E
+# HBM-side bytes per launch of the two headline workloads, from rocprofv3 --pmc FETCH_SIZE and
+# WRITE_SIZE runs of this script (--only prefill / --only decode), each scaled by what the same
+# counter reads for the calibration copy kernel (--only copy: factor 2.0 for FETCH_SIZE, 1.0 for
+# WRITE_SIZE). Counters cannot be read from inside a timed run, so the figures are recorded here.
+PREFILL_TRAFFIC_BYTES = 97.7e6 + 25.2e6            # vs 75.5 MB + 25.2 MB compulsory
+DECODE_TRAFFIC_BYTES = 5.2718e9 + 2.8e6 + 4.7e6    # split kernel read + partials + merge kernel
 
 
 def log(*a):
@@ -105,7 +111,7 @@ def prefill_leg(lm, dev, steps, warmup, cpu_seconds):
     res = {
         "ms_per_step": wall_ms, "value": tflops,
         "roofline": {"bound": "mfma", "achieved": kern_tflops, "peak": PEAK_FP16_TFLOPS, "unit": "TFLOP/s",
-                     "frac": kern_tflops / PEAK_FP16_TFLOPS, "traffic": None,
+                     "frac": kern_tflops / PEAK_FP16_TFLOPS, "traffic": PREFILL_TRAFFIC_BYTES,
                      "kernel": "prefill_mfma_kernel<MfmaF16, 96, causal>", "launch_us": ev_ms * 1e3,
                      "algorithmic_flops_per_launch": flops},
     }
@@ -180,7 +186,8 @@ def decode_leg(lm, dev, steps, warmup, cpu_seconds, num_splits=0):
         "workload": "C5 long ragged GQA decode: B=64 Hq=32 Hkv=8 D=128 bf16, kv_len~U[8192,32768], sum=%d" % int(lens.sum()),
         "value": gbs, "unit": "GB/s", "ms_per_step": wall_ms, "num_splits": int(p.num_splits),
         "roofline": {"bound": "hbm", "achieved": kern_gbs, "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": kern_gbs / PEAK_HBM_GBS,
-                     "traffic": None, "kernel": "decode_split_kernel<BF16,16,4> + decode_merge_kernel",
+                     "traffic": DECODE_TRAFFIC_BYTES if num_splits == 0 else None,
+                     "kernel": "decode_mfma_kernel<Mfma16BF16,128> + decode_merge_kernel",
                      "launch_us": ev_ms * 1e3, "algorithmic_bytes_per_launch": algo_bytes},
     }
     if cpu_seconds > 0:

@@ -1,0 +1,182 @@
+# LuminalHIP.jl — Julia glue between Luminal.jl and libluminal_hip.so (MI355X / gfx950).
+#
+# Nothing in Luminal.jl is edited. This module adds
+#   * a device type          HIPDevice <: Luminal.AbstractDevice     (src/Device.jl:9-16)
+#   * a device array type    HipArray{T,N} (pointer + dims, freed by a finalizer)
+#   * to_device / from_device methods                                  (src/Device.jl:82-105)
+#   * execute_op / execute_op! methods for FlashAttentionOp on HipArray arguments; multiple
+#     dispatch prefers them over the generic method at src/Execution.jl:565-578
+#   * DecodeAttentionOp + decode_attention, the fused form of the cached single-token attention
+#     subgraph (src/Whisper.jl:584-620) with the GQA head sharing of src/NN.jl:305-317
+# and calls the C ABI of include/luminal_hip.h through `ccall`. There are no AMDGPU.jl kernels here.
+#
+# Layout: Luminal tensors are column-major (B,H,S,D) arrays (B fastest). The library takes
+# row-major [B,H,S,D] (D contiguous), which is the memory order of a column-major (D,S,H,B) array,
+# so upload is permutedims(x, (4,3,2,1)) and download is the inverse permutation.
+module LuminalHIP
+
+using Luminal
+import Luminal: AbstractDevice, Op, FlashAttentionOp, GraphTensor, add_op!, realized_dims,
+                to_device, from_device, execute_op, execute_op!
+
+const libluminal_hip = get(ENV, "LUMINAL_HIP_LIB", joinpath(@__DIR__, "..", "lib", "libluminal_hip.so"))
+
+# element type codes of include/luminal_hip.h
+const LMH_F32, LMH_F16, LMH_BF16 = Int32(0), Int32(1), Int32(2)
+const HEADMAP_INTERLEAVED, HEADMAP_BLOCKED = Int32(0), Int32(1)
+# bf16 tensors are carried as UInt16 bit patterns (Julia has no native BFloat16 array type)
+struct BF16Bits; bits::UInt16; end
+dtype_code(::Type{Float32}) = LMH_F32
+dtype_code(::Type{Float16}) = LMH_F16
+dtype_code(::Type{BF16Bits}) = LMH_BF16
+
+check(rc::Integer) = rc == 0 ? nothing :
+    error("libluminal_hip: ", unsafe_string(ccall((:lmh_last_error, libluminal_hip), Cstring, ())), " (code $rc)")
+
+struct HIPDevice <: AbstractDevice
+    index::Int
+end
+HIPDevice() = HIPDevice(0)
+
+"Health check in the style of get_device(): true when a gfx950 device answers a tiny allocation."
+function functional()
+    try
+        ccall((:lmh_device_count, libluminal_hip), Cint, ()) > 0 || return false
+        return ccall((:lmh_init, libluminal_hip), Cint, (Cint,), 0) == 0
+    catch
+        return false
+    end
+end
+
+"Best device: HIPDevice when the library finds an MI355X, otherwise whatever Luminal picks."
+get_device() = functional() ? HIPDevice(0) : Luminal.get_device()
+
+# ------------------------------------------------------------------------------------------
+# device arrays
+# ------------------------------------------------------------------------------------------
+mutable struct HipArray{T,N}
+    ptr::Ptr{Cvoid}
+    dims::NTuple{N,Int}      # logical Luminal dims, e.g. (B,H,S,D)
+    function HipArray{T,N}(dims::NTuple{N,Int}) where {T,N}
+        p = Ref{Ptr{Cvoid}}(C_NULL)
+        check(ccall((:lmh_malloc, libluminal_hip), Cint, (Ptr{Ptr{Cvoid}}, Csize_t), p, max(prod(dims), 1) * sizeof(T)))
+        a = new{T,N}(p[], dims)
+        finalizer(x -> ccall((:lmh_free, libluminal_hip), Cint, (Ptr{Cvoid},), x.ptr), a)
+        return a
+    end
+end
+Base.size(a::HipArray) = a.dims
+Base.length(a::HipArray) = prod(a.dims)
+Base.eltype(::HipArray{T}) where {T} = T
+Base.similar(a::HipArray{T,N}) where {T,N} = HipArray{T,N}(a.dims)
+
+"Host array -> device, reversing the dimension order so that D becomes the contiguous axis."
+function to_device(data::AbstractArray{T,N}, ::HIPDevice) where {T,N}
+    host = Array(permutedims(data, ntuple(i -> N + 1 - i, N)))
+    dev = HipArray{T,N}(size(data))
+    check(ccall((:lmh_memcpy_h2d, libluminal_hip), Cint, (Ptr{Cvoid}, Ptr{Cvoid}, Csize_t, Ptr{Cvoid}),
+                dev.ptr, host, sizeof(host), C_NULL))
+    return dev
+end
+to_device(data::HipArray, ::HIPDevice) = data
+
+"Device -> host; synchronises like Array(::CuArray)."
+function from_device(a::HipArray{T,N}) where {T,N}
+    host = Array{T,N}(undef, reverse(a.dims))
+    check(ccall((:lmh_memcpy_d2h, libluminal_hip), Cint, (Ptr{Cvoid}, Ptr{Cvoid}, Csize_t, Ptr{Cvoid}),
+                host, a.ptr, sizeof(host), C_NULL))
+    return permutedims(host, ntuple(i -> N + 1 - i, N))
+end
+
+# ------------------------------------------------------------------------------------------
+# parameter blocks (field order and types mirror include/luminal_hip.h)
+# ------------------------------------------------------------------------------------------
+struct AttnParams
+    out::Ptr{Cvoid}; q::Ptr{Cvoid}; k::Ptr{Cvoid}; v::Ptr{Cvoid}; kv_len::Ptr{Int32}
+    B::Int32; Hq::Int32; Hkv::Int32; Sq::Int32; Sk::Int32; D::Int32
+    q_stride::NTuple{3,Int64}; k_stride::NTuple{3,Int64}; v_stride::NTuple{3,Int64}; o_stride::NTuple{3,Int64}
+    dtype::Int32; scale::Float32; causal::Int32; head_map::Int32; out_f32::Int32
+    stream::Ptr{Cvoid}
+end
+
+struct DecodeParams
+    out::Ptr{Cvoid}; q::Ptr{Cvoid}; k_cache::Ptr{Cvoid}; v_cache::Ptr{Cvoid}; kv_len::Ptr{Int32}
+    B::Int32; Hq::Int32; Hkv::Int32; Lmax::Int32; D::Int32
+    q_stride::NTuple{2,Int64}; o_stride::NTuple{2,Int64}; k_stride::NTuple{3,Int64}; v_stride::NTuple{3,Int64}
+    dtype::Int32; scale::Float32; head_map::Int32; out_f32::Int32; num_splits::Int32
+    workspace::Ptr{Cvoid}; workspace_bytes::Csize_t
+    stream::Ptr{Cvoid}
+end
+
+const Z3 = (Int64(0), Int64(0), Int64(0))   # all-zero strides = contiguous
+const Z2 = (Int64(0), Int64(0))
+
+# ------------------------------------------------------------------------------------------
+# FlashAttentionOp on device arrays
+# ------------------------------------------------------------------------------------------
+function execute_op!(out::HipArray{TO,4}, op::FlashAttentionOp, q::HipArray{T,4}, k::HipArray{T,4}, v::HipArray{T,4};
+                     head_map::Int32=HEADMAP_INTERLEAVED) where {TO,T}
+    B, Hq, Sq, D = size(q)
+    _, Hkv, Sk, _ = size(k)
+    size(out) == size(q) || error("FlashAttentionOp: output shape $(size(out)) differs from q shape $(size(q))")
+    p = Ref(AttnParams(out.ptr, q.ptr, k.ptr, v.ptr, C_NULL, B, Hq, Hkv, Sq, Sk, D, Z3, Z3, Z3, Z3,
+                       dtype_code(T), op.scale, Int32(op.causal), head_map, Int32(TO === Float32 && T !== Float32), C_NULL))
+    check(ccall((:lmh_flash_attn_fwd, libluminal_hip), Cint, (Ref{AttnParams},), p))
+    return out
+end
+
+function execute_op(op::FlashAttentionOp, q::HipArray, k::HipArray, v::HipArray)
+    out = similar(q)                      # src/Execution.jl:252-255
+    return execute_op!(out, op, q, k, v)
+end
+
+# ------------------------------------------------------------------------------------------
+# DecodeAttentionOp: q (B,H,D); caches (B,Hkv,max_seq,D) like KVCacheState (src/Whisper.jl:519-540);
+# kv_len (B,) Int32 on the device — a tensor, not a graph constant, so one compiled graph serves
+# every decode position (the reference compiles one graph per position, src/Decoding.jl:98-106).
+# ------------------------------------------------------------------------------------------
+struct DecodeAttentionOp <: Op
+    scale::Float32
+    head_map::Int32
+end
+
+function decode_attention(q::GraphTensor, k_cache::GraphTensor, v_cache::GraphTensor, kv_len::GraphTensor;
+                          scale=nothing, head_map::Int32=HEADMAP_INTERLEAVED)
+    q_dims = realized_dims(q.shape)
+    if isnothing(scale)
+        scale = 1.0f0 / sqrt(Float32(q_dims[end]))
+    end
+    inputs = [(q.id, 0, q.shape), (k_cache.id, 0, k_cache.shape), (v_cache.id, 0, v_cache.shape),
+              (kv_len.id, 0, kv_len.shape)]
+    return add_op!(q.graph_ref, DecodeAttentionOp(Float32(scale), head_map), inputs, q.shape)
+end
+
+const _workspace = Ref{Union{Nothing,HipArray{UInt8,1}}}(nothing)
+function workspace(bytes::Integer)
+    if bytes > 0 && (_workspace[] === nothing || length(_workspace[]) < bytes)
+        _workspace[] = HipArray{UInt8,1}((Int(bytes),))
+    end
+    return _workspace[]
+end
+
+function execute_op!(out::HipArray{TO,3}, op::DecodeAttentionOp, q::HipArray{T,3}, kc::HipArray{T,4}, vc::HipArray{T,4},
+                     kv_len::HipArray{Int32,1}) where {TO,T}
+    B, Hq, D = size(q)
+    _, Hkv, Lmax, _ = size(kc)
+    splits = ccall((:lmh_decode_auto_splits, libluminal_hip), Int32, (Int32, Int32, Int32), B, Hkv, Lmax)
+    need = ccall((:lmh_decode_workspace_bytes, libluminal_hip), Csize_t, (Int32, Int32, Int32, Int32, Int32, Int32),
+                 B, Hq, Hkv, Lmax, D, splits)
+    ws = workspace(need)
+    p = Ref(DecodeParams(out.ptr, q.ptr, kc.ptr, vc.ptr, Ptr{Int32}(kv_len.ptr), B, Hq, Hkv, Lmax, D, Z2, Z2, Z3, Z3,
+                         dtype_code(T), op.scale, op.head_map, Int32(TO === Float32 && T !== Float32), splits,
+                         ws === nothing ? C_NULL : ws.ptr, need, C_NULL))
+    check(ccall((:lmh_decode_attn, libluminal_hip), Cint, (Ref{DecodeParams},), p))
+    return out
+end
+
+execute_op(op::DecodeAttentionOp, q::HipArray, kc::HipArray, vc::HipArray, kv_len::HipArray) =
+    execute_op!(similar(q), op, q, kc, vc, kv_len)
+
+export HIPDevice, HipArray, DecodeAttentionOp, decode_attention, get_device, functional
+
+end # module
