@@ -145,6 +145,53 @@ size_t lmh_decode_workspace_bytes(int32_t B, int32_t Hq, int32_t Hkv, int32_t Lm
 int32_t lmh_decode_auto_splits(int32_t B, int32_t Hkv, int32_t Lmax);
 int lmh_decode_attn(const lmh_decode_params *p);
 
+/* ---- rotary position embedding: replaces the ~25-node subgraph of
+ *   apply_rotary_embeddings(input, prev_seq; base)    reference src/NN.jl:253-303
+ * out[b,h,s,:] = rotate(x[b,h,s,:], position = (pos0 ? pos0[b] : prev_seq) + s); out may alias x.
+ * pairing LMH_ROPE_HALF_SPLIT rotates (j, j + D/2), which is what the reference's column-major
+ * reshape to (D/2, 2) produces; LMH_ROPE_INTERLEAVED rotates (2j, 2j+1). D must be even. ---- */
+#define LMH_ROPE_HALF_SPLIT 0
+#define LMH_ROPE_INTERLEAVED 1
+typedef struct lmh_rope_params {
+  void *out;           /* [B,H,S,D] device */
+  const void *x;       /* [B,H,S,D] device */
+  const int32_t *pos0; /* optional device int32[B]; null = prev_seq for every sequence */
+  int32_t prev_seq;
+  int32_t B, H, S, D;
+  int64_t x_stride[3]; /* (b, h, s); all-zero = contiguous */
+  int64_t o_stride[3];
+  int32_t dtype;
+  float base;          /* 10000 in the reference */
+  int32_t pairing;     /* LMH_ROPE_* */
+  void *stream;
+} lmh_rope_params;
+int lmh_rope(const lmh_rope_params *p);
+
+/* ---- in-place KV-cache append: replaces
+ *   _kv_scatter(past, new_slot, step_pos)              reference src/Whisper.jl:552-570
+ * (a slice + concat rebuild of the whole (B,H,max_seq,D) cache) and the per-step host round trip of
+ * decode_step!, reference src/Whisper.jl:775-797.
+ * cache[b,h,pos+t,:] = new[b,h,t,:] for t < T, pos = pos ? pos[b] : pos_all; rows that would fall
+ * outside 0..Lmax-1 are dropped. With rope_k != 0, K is rotated by its row position while it is
+ * written (V never is). ---- */
+typedef struct lmh_kv_append_params {
+  void *k_cache;        /* [B,Hkv,Lmax,D] device, updated in place */
+  void *v_cache;
+  const void *k_new;    /* [B,Hkv,T,D] device, contiguous */
+  const void *v_new;
+  const int32_t *pos;   /* optional device int32[B]: first row to write per sequence */
+  int32_t pos_all;      /* used when pos is null */
+  int32_t B, Hkv, T, D, Lmax;
+  int64_t k_stride[3];  /* cache strides (b, h, s); all-zero = contiguous */
+  int64_t v_stride[3];
+  int32_t dtype;
+  int32_t rope_k;       /* 0 / 1 */
+  int32_t pairing;      /* LMH_ROPE_*, used when rope_k != 0 */
+  float base;
+  void *stream;
+} lmh_kv_append_params;
+int lmh_kv_append(const lmh_kv_append_params *p);
+
 #ifdef __cplusplus
 }
 #endif

@@ -23,7 +23,8 @@ EXPORTS = [
     "lmh_version", "lmh_last_error", "lmh_device_count", "lmh_init", "lmh_device_name", "lmh_malloc", "lmh_free",
     "lmh_memset", "lmh_memcpy_h2d", "lmh_memcpy_d2h", "lmh_memcpy_d2d", "lmh_sync", "lmh_event_create",
     "lmh_event_destroy", "lmh_event_record", "lmh_event_elapsed_ms", "lmh_flash_attn_fwd",
-    "lmh_decode_workspace_bytes", "lmh_decode_auto_splits", "lmh_decode_attn", "lmh_calib_copy",
+    "lmh_decode_workspace_bytes", "lmh_decode_auto_splits", "lmh_decode_attn", "lmh_calib_copy", "lmh_rope",
+    "lmh_kv_append",
 ]
 
 
@@ -59,6 +60,29 @@ class DecodeParams(ctypes.Structure):
         ("stream", ctypes.c_void_p),
     ]
 
+
+class RopeParams(ctypes.Structure):
+    _fields_ = [
+        ("out", ctypes.c_void_p), ("x", ctypes.c_void_p), ("pos0", ctypes.c_void_p), ("prev_seq", ctypes.c_int32),
+        ("B", ctypes.c_int32), ("H", ctypes.c_int32), ("S", ctypes.c_int32), ("D", ctypes.c_int32),
+        ("x_stride", ctypes.c_int64 * 3), ("o_stride", ctypes.c_int64 * 3),
+        ("dtype", ctypes.c_int32), ("base", ctypes.c_float), ("pairing", ctypes.c_int32), ("stream", ctypes.c_void_p),
+    ]
+
+
+class KvAppendParams(ctypes.Structure):
+    _fields_ = [
+        ("k_cache", ctypes.c_void_p), ("v_cache", ctypes.c_void_p), ("k_new", ctypes.c_void_p),
+        ("v_new", ctypes.c_void_p), ("pos", ctypes.c_void_p), ("pos_all", ctypes.c_int32),
+        ("B", ctypes.c_int32), ("Hkv", ctypes.c_int32), ("T", ctypes.c_int32), ("D", ctypes.c_int32),
+        ("Lmax", ctypes.c_int32),
+        ("k_stride", ctypes.c_int64 * 3), ("v_stride", ctypes.c_int64 * 3),
+        ("dtype", ctypes.c_int32), ("rope_k", ctypes.c_int32), ("pairing", ctypes.c_int32), ("base", ctypes.c_float),
+        ("stream", ctypes.c_void_p),
+    ]
+
+
+ROPE_HALF_SPLIT, ROPE_INTERLEAVED = 0, 1
 
 _lib = None
 
@@ -97,7 +121,9 @@ def load():
     L.lmh_decode_auto_splits.restype = ctypes.c_int32
     L.lmh_decode_auto_splits.argtypes = [ctypes.c_int32] * 3
     L.lmh_calib_copy.argtypes = [vp, vp, ctypes.c_size_t, vp]
-    for name in ("lmh_calib_copy", "lmh_init", "lmh_device_name", "lmh_malloc", "lmh_free", "lmh_memset", "lmh_memcpy_h2d",
+    L.lmh_rope.argtypes = [ctypes.POINTER(RopeParams)]
+    L.lmh_kv_append.argtypes = [ctypes.POINTER(KvAppendParams)]
+    for name in ("lmh_rope", "lmh_kv_append", "lmh_calib_copy", "lmh_init", "lmh_device_name", "lmh_malloc", "lmh_free", "lmh_memset", "lmh_memcpy_h2d",
                  "lmh_memcpy_d2h", "lmh_memcpy_d2d", "lmh_sync", "lmh_event_create", "lmh_event_destroy",
                  "lmh_event_record", "lmh_event_elapsed_ms", "lmh_flash_attn_fwd", "lmh_decode_attn"):
         getattr(L, name).restype = ctypes.c_int
@@ -182,6 +208,14 @@ def flash_attn_fwd(params):
 
 def decode_attn(params):
     check(load().lmh_decode_attn(ctypes.byref(params)))
+
+
+def rope(params):
+    check(load().lmh_rope(ctypes.byref(params)))
+
+
+def kv_append(params):
+    check(load().lmh_kv_append(ctypes.byref(params)))
 
 
 def calib_copy(dst, src, nbytes, stream=None):

@@ -1,6 +1,7 @@
 // C-ABI layer of libluminal_hip.so: argument validation, dispatch to the kernel launchers, and
 // the small device-runtime surface (allocation, copies, sync, events) that stands in for the
 // CuArray()/Array() calls of the reference's device layer (reference src/Device.jl:82-105).
+#include <math.h>
 #include <stdarg.h>
 #include <stdio.h>
 #include <string.h>
@@ -300,6 +301,69 @@ int lmh_decode_attn(const lmh_decode_params *p) {
     a.ws_ml = a.ws_o + (size_t)p->B * p->Hq * a.num_splits * p->D;
   }
   return launch_decode(a, p->dtype, (hipStream_t)p->stream);
+}
+
+// --------------------------------------------------------------------------------------------
+// rotary embedding and KV-cache append
+// --------------------------------------------------------------------------------------------
+int lmh_rope(const lmh_rope_params *p) {
+  if (!p) return fail(LMH_E_NULL, "lmh_rope: null params");
+  if (!p->out || !p->x) return fail(LMH_E_NULL, "lmh_rope: null tensor pointer");
+  if (p->B <= 0 || p->H <= 0 || p->S <= 0 || p->D <= 0)
+    return fail(LMH_E_SHAPE, "lmh_rope: non-positive dimension (B=%d H=%d S=%d D=%d)", p->B, p->H, p->S, p->D);
+  if (p->D % 2 != 0) return fail(LMH_E_SHAPE, "lmh_rope: head dim %d must be even", p->D);
+  if (p->dtype != LMH_F32 && p->dtype != LMH_F16 && p->dtype != LMH_BF16)
+    return fail(LMH_E_UNSUPPORTED, "lmh_rope: unknown dtype %d", p->dtype);
+  if (p->pairing != LMH_ROPE_HALF_SPLIT && p->pairing != LMH_ROPE_INTERLEAVED)
+    return fail(LMH_E_UNSUPPORTED, "lmh_rope: unknown pairing %d", p->pairing);
+  if (!(p->base > 0.f)) return fail(LMH_E_SHAPE, "lmh_rope: base must be positive");
+  RopeArgs a;
+  a.out = p->out; a.x = p->x; a.pos0 = p->pos0; a.prev_seq = p->prev_seq;
+  a.B = p->B; a.H = p->H; a.S = p->S; a.D = p->D;
+  auto fill = [&](int64_t *dst, const int64_t *src) {
+    if (all_zero(src, 3)) { dst[0] = (int64_t)p->H * p->S * p->D; dst[1] = (int64_t)p->S * p->D; dst[2] = p->D; }
+    else { dst[0] = src[0]; dst[1] = src[1]; dst[2] = src[2]; }
+  };
+  fill(a.xs, p->x_stride);
+  fill(a.os, p->o_stride);
+  for (int i = 0; i < 3; i++)
+    if (a.xs[i] < 0 || a.os[i] < 0) return fail(LMH_E_SHAPE, "lmh_rope: negative stride");
+  a.log2_base = log2f(p->base);
+  a.interleaved = p->pairing == LMH_ROPE_INTERLEAVED;
+  return launch_rope(a, p->dtype, (hipStream_t)p->stream);
+}
+
+int lmh_kv_append(const lmh_kv_append_params *p) {
+  if (!p) return fail(LMH_E_NULL, "lmh_kv_append: null params");
+  if (!p->k_cache || !p->v_cache || !p->k_new || !p->v_new) return fail(LMH_E_NULL, "lmh_kv_append: null tensor pointer");
+  if (p->B <= 0 || p->Hkv <= 0 || p->T <= 0 || p->D <= 0 || p->Lmax <= 0)
+    return fail(LMH_E_SHAPE, "lmh_kv_append: non-positive dimension (B=%d Hkv=%d T=%d D=%d Lmax=%d)", p->B, p->Hkv, p->T,
+                p->D, p->Lmax);
+  if (p->dtype != LMH_F32 && p->dtype != LMH_F16 && p->dtype != LMH_BF16)
+    return fail(LMH_E_UNSUPPORTED, "lmh_kv_append: unknown dtype %d", p->dtype);
+  if (p->rope_k) {
+    if (p->D % 2 != 0) return fail(LMH_E_SHAPE, "lmh_kv_append: head dim %d must be even for the rotary embedding", p->D);
+    if (p->pairing != LMH_ROPE_HALF_SPLIT && p->pairing != LMH_ROPE_INTERLEAVED)
+      return fail(LMH_E_UNSUPPORTED, "lmh_kv_append: unknown pairing %d", p->pairing);
+    if (!(p->base > 0.f)) return fail(LMH_E_SHAPE, "lmh_kv_append: base must be positive");
+  }
+  KvAppendArgs a;
+  a.k_cache = p->k_cache; a.v_cache = p->v_cache; a.k_new = p->k_new; a.v_new = p->v_new;
+  a.pos = p->pos; a.pos_all = p->pos_all;
+  a.B = p->B; a.Hkv = p->Hkv; a.T = p->T; a.D = p->D; a.Lmax = p->Lmax;
+  auto fill = [&](int64_t *dst, const int64_t *src) {
+    if (all_zero(src, 3)) { dst[0] = (int64_t)p->Hkv * p->Lmax * p->D; dst[1] = (int64_t)p->Lmax * p->D; dst[2] = p->D; }
+    else { dst[0] = src[0]; dst[1] = src[1]; dst[2] = src[2]; }
+  };
+  fill(a.ks, p->k_stride);
+  fill(a.vs, p->v_stride);
+  for (int i = 0; i < 3; i++)
+    if (a.ks[i] < 0 || a.vs[i] < 0) return fail(LMH_E_SHAPE, "lmh_kv_append: negative stride");
+  if (a.ks[2] < p->D || a.vs[2] < p->D) return fail(LMH_E_SHAPE, "lmh_kv_append: cache row stride smaller than head dim");
+  a.rope_k = p->rope_k ? 1 : 0;
+  a.interleaved = p->pairing == LMH_ROPE_INTERLEAVED;
+  a.log2_base = p->rope_k ? log2f(p->base) : 0.f;
+  return launch_kv_append(a, p->dtype, (hipStream_t)p->stream);
 }
 
 }  // extern "C"

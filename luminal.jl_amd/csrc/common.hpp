@@ -50,6 +50,31 @@ struct DecodeArgs {
   float *ws_ml;   // [B][Hq][num_splits][2] (running max in log2 units, partial sum)
 };
 
+// Rotary embedding launch arguments.
+struct RopeArgs {
+  void *out;
+  const void *x;
+  const int32_t *pos0;  // per-sequence position of row 0 (device), or null -> prev_seq
+  int32_t prev_seq;
+  int32_t B, H, S, D;
+  int64_t xs[3], os[3];
+  float log2_base;
+  int32_t interleaved;  // 0: pairs (j, j + D/2) as the reference; 1: pairs (2j, 2j+1)
+};
+
+// KV-cache append launch arguments; k_new / v_new are contiguous [B, Hkv, T, D].
+struct KvAppendArgs {
+  void *k_cache, *v_cache;
+  const void *k_new, *v_new;
+  const int32_t *pos;  // per-sequence first row (device), or null -> pos_all
+  int32_t pos_all;
+  int32_t B, Hkv, T, D, Lmax;
+  int64_t ks[3], vs[3];
+  int32_t rope_k;  // rotate K by its row position while writing it
+  int32_t interleaved;
+  float log2_base;
+};
+
 __host__ __device__ inline int kv_head_of(int hq, int Hq, int Hkv, int head_map) {
   if (Hq == Hkv) return hq;
   return head_map == LMH_HEADMAP_BLOCKED ? hq / (Hq / Hkv) : hq % Hkv;
@@ -67,6 +92,8 @@ bool prefill_mfma_supported(int dtype, int D);
 int launch_prefill_mfma(const PrefillArgs &a, int dtype, hipStream_t stream);
 int launch_prefill_valu(const PrefillArgs &a, int dtype, hipStream_t stream);
 int launch_decode(const DecodeArgs &a, int dtype, hipStream_t stream);
+int launch_rope(const RopeArgs &a, int dtype, hipStream_t stream);
+int launch_kv_append(const KvAppendArgs &a, int dtype, hipStream_t stream);
 bool decode_mfma_supported(int dtype, int D, int B);
 int launch_decode_mfma_split(const DecodeArgs &a, int dtype, hipStream_t stream);
 

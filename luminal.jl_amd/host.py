@@ -435,6 +435,88 @@ def compile(graph, device=None):
     return CompiledGraph(steps, results)
 
 
+# ---------------------------------------------------------------------------------------------
+# the operators directly in front of decode attention
+# ---------------------------------------------------------------------------------------------
+def apply_rotary_embeddings(x, prev_seq=0, base=10000.0, pos0=None, out=None, interleaved=False, stream=None):
+    """Rotary embedding of a (B,H,S,D) HipArray with the reference's pairing (j, j + D/2)
+    (apply_rotary_embeddings(input, prev_seq; base), reference src/NN.jl:253-303). `pos0` (HipArray
+    int32[B]) gives per-sequence start positions instead of the scalar prev_seq; `out` may be x."""
+    _require_hip(x)
+    if len(x.shape) != 4:
+        raise ValueError("rotary embedding expects (B,H,S,D); got %s" % (x.shape,))
+    out = out if out is not None else HipArray(x.shape, x.dtype, x.device)
+    if out.shape != x.shape or out.dtype != x.dtype:
+        raise ValueError("rotary embedding: out must match x in shape and element type")
+    p = binding.RopeParams()
+    p.out, p.x = out.ptr, x.ptr
+    p.pos0 = pos0.ptr if pos0 is not None else None
+    p.prev_seq = int(prev_seq)
+    p.B, p.H, p.S, p.D = x.shape
+    p.dtype = binding.DTYPE_CODES[x.dtype]
+    p.base = float(base)
+    p.pairing = binding.ROPE_INTERLEAVED if interleaved else binding.ROPE_HALF_SPLIT
+    p.stream = stream
+    binding.rope(p)
+    return out
+
+
+def kv_append(k_cache, v_cache, k_new, v_new, pos, rope_k=False, base=10000.0, interleaved=False, stream=None):
+    """In-place cache update cache[b,h,pos[b]+t,:] = new[b,h,t,:] (the reference rebuilds the whole cache
+    with _kv_scatter, reference src/Whisper.jl:552-570). `pos` is a HipArray int32[B] or an int."""
+    _require_hip(k_cache, v_cache, k_new, v_new)
+    if k_cache.shape != v_cache.shape or k_new.shape != v_new.shape or len(k_cache.shape) != 4:
+        raise ValueError("kv_append expects caches (B,Hkv,Lmax,D) and new rows (B,Hkv,T,D)")
+    B, Hkv, Lmax, D = k_cache.shape
+    if k_new.shape[:2] != (B, Hkv) or k_new.shape[3] != D:
+        raise ValueError("kv_append: new rows %s do not match the cache %s" % (k_new.shape, k_cache.shape))
+    if not (k_cache.dtype == v_cache.dtype == k_new.dtype == v_new.dtype):
+        raise ValueError("kv_append: caches and new rows must share one element type")
+    p = binding.KvAppendParams()
+    p.k_cache, p.v_cache, p.k_new, p.v_new = k_cache.ptr, v_cache.ptr, k_new.ptr, v_new.ptr
+    if isinstance(pos, HipArray):
+        p.pos = pos.ptr
+    else:
+        p.pos, p.pos_all = None, int(pos)
+    p.B, p.Hkv, p.T, p.D, p.Lmax = B, Hkv, k_new.shape[2], D, Lmax
+    p.dtype = binding.DTYPE_CODES[k_cache.dtype]
+    p.rope_k = int(bool(rope_k))
+    p.pairing = binding.ROPE_INTERLEAVED if interleaved else binding.ROPE_HALF_SPLIT
+    p.base = float(base)
+    p.stream = stream
+    binding.kv_append(p)
+
+
+class KVCacheState:
+    """Device-resident decode cache: the mirror of KVCacheState (reference src/Whisper.jl:519-540) with
+    per-sequence lengths. `append` writes the new rows in place and advances kv_len; `attend` is the
+    fused cached attention (reference src/Whisper.jl:584-620) over rows 0 .. kv_len[b]-1."""
+
+    def __init__(self, batch, n_kv_heads, head_dim, max_seq, dtype="f32", device=None):
+        self.device = device or get_device()
+        self.max_seq = max_seq
+        self.k = HipArray((batch, n_kv_heads, max_seq, head_dim), dtype, self.device).fill_bytes(0)
+        self.v = HipArray((batch, n_kv_heads, max_seq, head_dim), dtype, self.device).fill_bytes(0)
+        self.kv_len_host = np.zeros(batch, np.int32)
+        self.kv_len = HipArray((batch,), "i32", self.device).copy_from_host(self.kv_len_host)
+
+    @property
+    def step_pos(self):
+        return int(self.kv_len_host.max())
+
+    def append(self, k_new, v_new, rope_k=False, base=10000.0):
+        T = k_new.shape[2]
+        if int(self.kv_len_host.max()) + T > self.max_seq:
+            raise ValueError("KV cache is full (max_seq=%d)" % self.max_seq)
+        kv_append(self.k, self.v, k_new, v_new, self.kv_len, rope_k=rope_k, base=base)
+        self.kv_len_host += T
+        self.kv_len.copy_from_host(self.kv_len_host)
+
+    def attend(self, q, scale=None, head_map=HEADMAP_INTERLEAVED, out_dtype=None):
+        op = DecodeAttentionOp(default_scale(q.shape[-1]) if scale is None else scale, head_map, 0, out_dtype)
+        return execute_op(op, q, self.k, self.v, self.kv_len)
+
+
 def default_scale(D):
     return float(np.float32(1.0) / np.sqrt(np.float32(D)))
 
@@ -443,5 +525,5 @@ __all__ = [
     "AbstractDevice", "CPUDevice", "HIPDevice", "HipArray", "get_device", "to_device", "from_device", "Graph",
     "GraphTensor", "tensor", "add_op", "FlashAttentionOp", "DecodeAttentionOp", "flash_attention", "decode_attention",
     "execute_op", "execute_op_inplace", "execute", "compile", "CompiledGraph", "HEADMAP_INTERLEAVED",
-    "HEADMAP_BLOCKED", "LuminalHipError", "encode", "decode", "f32_to_bf16_bits", "bf16_bits_to_f32", "default_scale",
+    "HEADMAP_BLOCKED", "LuminalHipError", "apply_rotary_embeddings", "kv_append", "KVCacheState", "encode", "decode", "f32_to_bf16_bits", "bf16_bits_to_f32", "default_scale",
 ]

@@ -66,6 +66,7 @@ mutable struct HipArray{T,N}
     end
 end
 Base.size(a::HipArray) = a.dims
+Base.size(a::HipArray, i::Integer) = a.dims[i]
 Base.length(a::HipArray) = prod(a.dims)
 Base.eltype(::HipArray{T}) where {T} = T
 Base.similar(a::HipArray{T,N}) where {T,N} = HipArray{T,N}(a.dims)
@@ -177,6 +178,43 @@ end
 execute_op(op::DecodeAttentionOp, q::HipArray, kc::HipArray, vc::HipArray, kv_len::HipArray) =
     execute_op!(similar(q), op, q, kc, vc, kv_len)
 
-export HIPDevice, HipArray, DecodeAttentionOp, decode_attention, get_device, functional
+# ------------------------------------------------------------------------------------------
+# the operators in front of decode attention
+# ------------------------------------------------------------------------------------------
+struct RopeParams
+    out::Ptr{Cvoid}; x::Ptr{Cvoid}; pos0::Ptr{Int32}; prev_seq::Int32
+    B::Int32; H::Int32; S::Int32; D::Int32
+    x_stride::NTuple{3,Int64}; o_stride::NTuple{3,Int64}
+    dtype::Int32; base::Float32; pairing::Int32
+    stream::Ptr{Cvoid}
+end
+
+"In-place rotary embedding of a (B,H,S,D) device array; same pairing as apply_rotary_embeddings (src/NN.jl:253-303)."
+function rope!(x::HipArray{T,4}; prev_seq::Integer=0, base::Real=10000.0f0) where {T}
+    B, H, S, D = size(x)
+    p = Ref(RopeParams(x.ptr, x.ptr, C_NULL, prev_seq, B, H, S, D, Z3, Z3, dtype_code(T), Float32(base), Int32(0), C_NULL))
+    check(ccall((:lmh_rope, libluminal_hip), Cint, (Ref{RopeParams},), p))
+    return x
+end
+
+struct KvAppendParams
+    k_cache::Ptr{Cvoid}; v_cache::Ptr{Cvoid}; k_new::Ptr{Cvoid}; v_new::Ptr{Cvoid}; pos::Ptr{Int32}; pos_all::Int32
+    B::Int32; Hkv::Int32; T::Int32; D::Int32; Lmax::Int32
+    k_stride::NTuple{3,Int64}; v_stride::NTuple{3,Int64}
+    dtype::Int32; rope_k::Int32; pairing::Int32; base::Float32
+    stream::Ptr{Cvoid}
+end
+
+"cache[b,h,pos[b]+t,:] = new[b,h,t,:] in place (the reference rebuilds the cache with _kv_scatter, src/Whisper.jl:552-570)."
+function kv_append!(kc::HipArray{T,4}, vc::HipArray{T,4}, k_new::HipArray{T,4}, v_new::HipArray{T,4},
+                    pos::HipArray{Int32,1}; rope_k::Bool=false, base::Real=10000.0f0) where {T}
+    B, Hkv, Lmax, D = size(kc)
+    p = Ref(KvAppendParams(kc.ptr, vc.ptr, k_new.ptr, v_new.ptr, Ptr{Int32}(pos.ptr), 0, B, Hkv, size(k_new, 3), D, Lmax,
+                           Z3, Z3, dtype_code(T), Int32(rope_k), Int32(0), Float32(base), C_NULL))
+    check(ccall((:lmh_kv_append, libluminal_hip), Cint, (Ref{KvAppendParams},), p))
+    return kc, vc
+end
+
+export HIPDevice, HipArray, DecodeAttentionOp, decode_attention, get_device, functional, rope!, kv_append!
 
 end # module

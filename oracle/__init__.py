@@ -61,6 +61,10 @@ def lib():
         L.lmo_round_f16.restype = None
         L.lmo_round_f16.argtypes = [f32p, ctypes.c_uint64]
         L.lmo_max_threads.restype = ctypes.c_int
+        L.lmo_rope.restype = ctypes.c_int
+        L.lmo_rope.argtypes = [f32p, f32p, i32p, ctypes.c_int] + [ctypes.c_int] * 4 + [ctypes.c_float, ctypes.c_int]
+        L.lmo_kv_append.restype = ctypes.c_int
+        L.lmo_kv_append.argtypes = [f32p, f32p, i32p] + [ctypes.c_int] * 5
         _lib = L
     return _lib
 
@@ -153,9 +157,67 @@ def naive_attention_f64(q, k, v, scale=None, causal=False, head_map=HEADMAP_INTE
     return out
 
 
+def rope(x, prev_seq=0, base=10000.0, pos0=None, interleaved=False):
+    """Restated apply_rotary_embeddings on row-major [B,H,S,D] (fp32)."""
+    x, xp = _f32(x)
+    B, H, S, D = x.shape
+    out = np.empty_like(x)
+    p0, p0p = _i32_or_null(pos0)
+    rc = lib().lmo_rope(out.ctypes.data_as(ctypes.POINTER(ctypes.c_float)), xp, p0p, int(prev_seq), B, H, S, D,
+                        float(base), int(bool(interleaved)))
+    if rc != 0:
+        raise ValueError("oracle rejected the arguments")
+    return out
+
+
+def kv_append(cache, new_rows, pos):
+    """cache [B,H,Lmax,D] with new_rows [B,H,T,D] written at rows pos[b]..pos[b]+T-1 (returns a copy)."""
+    cache = np.array(cache, dtype=np.float32, order="C", copy=True)
+    new_rows, nrp = _f32(new_rows)
+    B, H, Lmax, D = cache.shape
+    T = new_rows.shape[2]
+    pos, posp = _i32_or_null(pos)
+    rc = lib().lmo_kv_append(cache.ctypes.data_as(ctypes.POINTER(ctypes.c_float)), nrp, posp, B, H, T, D, Lmax)
+    if rc != 0:
+        raise ValueError("oracle rejected the arguments")
+    return cache
+
+
 # ---------------------------------------------------------------------------------------------
 # numpy twins (independent of the C code)
 # ---------------------------------------------------------------------------------------------
+def rope_column_major_replay(x, prev_seq=0, base=10000.0):
+    """Literal replay of the reference's apply_rotary_embeddings graph (reference src/NN.jl:253-303):
+    every reshape is done in column-major element order, as Base.reshape does on Julia arrays
+    (reference src/Execution.jl:228), in float64."""
+    x = np.asarray(x, dtype=np.float64)
+    B, H, S, D = x.shape
+    half = D // 2
+    freqs = np.arange(half, dtype=np.float64) * 2.0 / D
+    inv_freqs = 1.0 / np.exp2(freqs * np.log2(base))
+    pos = np.arange(S, dtype=np.float64) + prev_seq
+    emb = pos[:, None] @ inv_freqs[None, :]                               # (S, half)
+    split = np.asfortranarray(x).reshape((B, H, S, half, 2), order="F")  # :274
+    x0 = split[..., 0]                                                    # slice_along(split, 5, 0, 1)
+    x1 = split[..., 1]
+    sin_e, cos_e = np.sin(emb)[None, None], np.cos(emb)[None, None]
+    x0_out = x0 * cos_e - x1 * sin_e
+    x1_out = x0 * sin_e + x1 * cos_e
+    res = np.asfortranarray(np.stack([x0_out, x1_out], axis=4))           # concat along dim 5
+    return np.ascontiguousarray(res.reshape((B, H, S, D), order="F"))
+
+
+def kv_scatter_replay(past, new_slot, step_pos):
+    """Literal replay of _kv_scatter (reference src/Whisper.jl:552-570): slices of `past` around
+    step_pos concatenated with the one-row new_slot along the sequence axis."""
+    max_seq = past.shape[2]
+    suffix_len = max_seq - step_pos - 1
+    if step_pos == 0:
+        return np.concatenate([new_slot, past[:, :, 1:max_seq]], axis=2)
+    if suffix_len == 0:
+        return np.concatenate([past[:, :, 0:step_pos], new_slot], axis=2)
+    return np.concatenate([past[:, :, 0:step_pos], new_slot, past[:, :, step_pos + 1:max_seq]], axis=2)
+
 def repeat_kv_column_major(x, groups):
     """Literal replay of the reference's repeat_kv on a column-major array.
 

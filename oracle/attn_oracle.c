@@ -26,13 +26,20 @@
  *                          src/HighLevelOps.jl:313-319. It shares no code with lmo_flash_attn, so
  *                          an error in either shows up as a disagreement.
  *
+ *   lmo_rope            <- apply_rotary_embeddings, src/NN.jl:253-303 (pairs (j, j+D/2) under the
+ *                          reference's column-major reshape)
+ *   lmo_kv_append       <- _kv_scatter, src/Whisper.jl:552-570, as an in-place row write
+ *
  * Pinned by (tests/test_oracle.py): flash == naive-f64 to 1e-5 on the reference's test shape
  * (B=H=1,S=8,D=16; the reference's own criterion is rtol 1e-4,
  * tests/test_flash_attention_verification.jl:48); closed forms (row 0 == V[0], Q=0 -> running
  * mean of V, V=1 -> 1, single key -> that V row, logit-shift invariance); the GQA map against a
  * literal column-major replay of Expand+Reshape; decode == last row of causal prefill; and the
  * committed golden vectors under tests/golden/, which were produced by an independent numpy
- * float64 implementation.
+ * float64 implementation. lmo_rope is pinned by a literal numpy replay of the reference's graph
+ * on column-major arrays (reshape to (D/2,2), slice, rotate, concat, reshape back), by norm
+ * preservation, the position-0 identity, additivity of positions and the relative-position
+ * property of q.k; lmo_kv_append by a literal replay of the slice + concat of _kv_scatter.
  *
  * Layout: row-major [B, H, S, D] (D contiguous), all tensors fp32. Half-precision configs are
  * evaluated on inputs already rounded to fp16 / bf16 (lmo_round_f16 / lmo_round_bf16).
@@ -191,6 +198,56 @@ int lmo_attn_naive_f64(double *out, const float *q, const float *k, const float 
     }
     free(w);
   }
+  return 0;
+}
+
+/*
+ * Rotary embedding, restating apply_rotary_embeddings (src/NN.jl:253-303) on row-major [B,H,S,D]:
+ *   freqs = arange(D/2) * 2 / D; inv_freqs = 1 / exp2(freqs * log2(base))     (:261-263)
+ *   pos = arange(S) + prev_seq; emb[s][j] = pos[s] * inv_freqs[j]              (:265-270)
+ *   the input is reshaped to (B,H,S,D/2,2) in COLUMN-major order and split on the last axis
+ *   (:274-276), so x0 = x[.., j] and x1 = x[.., j + D/2];
+ *   x0' = x0 cos - x1 sin, x1' = x0 sin + x1 cos                                (:292-293)
+ * interleaved != 0 pairs (2j, 2j+1) instead. pos0 (int32[B]) overrides prev_seq per sequence.
+ */
+int lmo_rope(float *out, const float *x, const int32_t *pos0, int prev_seq, int B, int H, int S, int D,
+             float base, int interleaved) {
+  if (!out || !x || B <= 0 || H <= 0 || S <= 0 || D <= 0 || D % 2 != 0) return -1;
+  const int half = D / 2;
+  const float log2_base = log2f(base);
+  for (int b = 0; b < B; b++)
+    for (int h = 0; h < H; h++)
+      for (int s = 0; s < S; s++) {
+        const float *xr = x + (((int64_t)b * H + h) * S + s) * D;
+        float *orow = out + (((int64_t)b * H + h) * S + s) * D;
+        const float pos = (float)((pos0 ? pos0[b] : prev_seq) + s);
+        for (int j = 0; j < half; j++) {
+          const float freq = (float)j * 2.0f / (float)D;
+          const float inv_freq = 1.0f / exp2f(freq * log2_base);
+          const float ang = pos * inv_freq;
+          const int d0 = interleaved ? 2 * j : j, d1 = interleaved ? 2 * j + 1 : j + half;
+          const float x0 = xr[d0], x1 = xr[d1];
+          orow[d0] = x0 * cosf(ang) - x1 * sinf(ang);
+          orow[d1] = x0 * sinf(ang) + x1 * cosf(ang);
+        }
+      }
+  return 0;
+}
+
+/*
+ * KV-cache append, the in-place equivalent of _kv_scatter (src/Whisper.jl:552-570):
+ * cache[b,h,pos[b]+t,:] = new[b,h,t,:]; every other row unchanged. cache [B,H,Lmax,D], new [B,H,T,D].
+ */
+int lmo_kv_append(float *cache, const float *new_rows, const int32_t *pos, int B, int H, int T, int D, int Lmax) {
+  if (!cache || !new_rows || !pos || B <= 0 || H <= 0 || T <= 0 || D <= 0 || Lmax <= 0) return -1;
+  for (int b = 0; b < B; b++)
+    for (int h = 0; h < H; h++)
+      for (int t = 0; t < T; t++) {
+        const int row = pos[b] + t;
+        if (row < 0 || row >= Lmax) continue;
+        memcpy(cache + (((int64_t)b * H + h) * Lmax + row) * D, new_rows + (((int64_t)b * H + h) * T + t) * D,
+               sizeof(float) * (size_t)D);
+      }
   return 0;
 }
 

@@ -117,3 +117,28 @@ def test_null_and_zero_size_plumbing(lm):
     assert b.load().lmh_memcpy_h2d(None, None, 0, None) == 0
     with pytest.raises(lm.LuminalHipError):
         b.check(b.load().lmh_memcpy_h2d(None, None, 8, None))
+
+
+def test_rope_and_kv_append_argument_errors(lm):
+    b = lm.binding
+    r = b.RopeParams()
+    r.out, r.x = 0x1000, 0x2000
+    r.B, r.H, r.S, r.D = 1, 2, 4, 7  # odd head dim
+    r.dtype, r.base, r.pairing = 0, 10000.0, 0
+    with pytest.raises(lm.LuminalHipError) as e:
+        b.rope(r)
+    assert e.value.code == b.LMH_E_SHAPE and "lmh_rope" in str(e.value)
+    r.D, r.pairing = 8, 5
+    with pytest.raises(lm.LuminalHipError) as e:
+        b.rope(r)
+    assert e.value.code == b.LMH_E_UNSUPPORTED
+    a = b.KvAppendParams()
+    a.k_cache, a.v_cache, a.k_new = 0x1000, 0x2000, 0x3000  # v_new missing
+    a.B, a.Hkv, a.T, a.D, a.Lmax = 1, 1, 1, 8, 16
+    with pytest.raises(lm.LuminalHipError) as e:
+        b.kv_append(a)
+    assert e.value.code == b.LMH_E_NULL and "lmh_kv_append" in str(e.value)
+    a.v_new, a.Lmax = 0x4000, 0
+    with pytest.raises(lm.LuminalHipError) as e:
+        b.kv_append(a)
+    assert e.value.code == b.LMH_E_SHAPE

@@ -162,3 +162,65 @@ def test_generator_twins_and_rounding(oracle):
     assert np.all(np.abs(r - x) <= np.abs(x) * 2.0 ** -8)
     lens = oracle.gen_uniform_int(1000, 3, 8192, 32768)
     assert lens.min() >= 8192 and lens.max() <= 32768 and len(set(lens.tolist())) > 900
+
+
+# ---------------------------------------------------------------------------------------------
+# rotary embedding and KV-cache append (the operators in front of decode attention)
+# ---------------------------------------------------------------------------------------------
+def test_rope_matches_column_major_replay_of_the_reference_graph(oracle):
+    for (shape, prev) in [((1, 2, 5, 8), 0), ((2, 3, 9, 64), 17), ((1, 1, 1, 128), 4095)]:
+        x = oracle.gen_normal(shape, 60 + prev)
+        want = oracle.rope_column_major_replay(x, prev_seq=prev)
+        # the oracle works in fp32 like the reference; the angle pos * inv_freq then carries a rounding
+        # error of ~pos * 2^-24 rad, which is what separates it from the float64 replay
+        assert rel_err(oracle.rope(x, prev_seq=prev), want) <= 1e-5 + prev * 4e-8
+    # the pairing is (j, j + D/2): rotating a tensor that is non-zero only at d = 0 moves weight to d = D/2
+    x = np.zeros((1, 1, 2, 8), np.float32)
+    x[..., 0] = 1.0
+    y = oracle.rope(x, prev_seq=1)
+    assert abs(y[0, 0, 0, 4] - np.sin(1.0)) < 1e-6 and abs(y[0, 0, 0, 0] - np.cos(1.0)) < 1e-6
+    assert np.all(y[0, 0, 0, [1, 2, 3, 5, 6, 7]] == 0)
+    # the interleaved variant pairs (2j, 2j+1) instead
+    yi = oracle.rope(x, prev_seq=1, interleaved=True)
+    assert abs(yi[0, 0, 0, 1] - np.sin(1.0)) < 1e-6 and yi[0, 0, 0, 4] == 0
+
+
+def test_rope_properties(oracle):
+    B, H, S, D = 2, 2, 6, 32
+    x = oracle.gen_normal((B, H, S, D), 70)
+    y = oracle.rope(x, prev_seq=3)
+    # rotations preserve the norm of every pair, hence of every row
+    np.testing.assert_allclose(np.linalg.norm(y, axis=-1), np.linalg.norm(x, axis=-1), rtol=1e-5)
+    # position 0 is the identity
+    np.testing.assert_allclose(oracle.rope(x[:, :, :1], prev_seq=0), x[:, :, :1], rtol=0, atol=1e-7)
+    # rotating by a then by b is rotating by a + b (single-row tensors so that every row sits at s = 0)
+    row = x[:, :, :1]
+    np.testing.assert_allclose(oracle.rope(oracle.rope(row, prev_seq=5), prev_seq=9), oracle.rope(row, prev_seq=14),
+                               rtol=0, atol=2e-5)
+    # q.k after the embedding depends on the position difference only
+    q, k = oracle.gen_normal((1, 1, 1, D), 71), oracle.gen_normal((1, 1, 1, D), 72)
+    d1 = float(np.sum(oracle.rope(q, prev_seq=10) * oracle.rope(k, prev_seq=4)))
+    d2 = float(np.sum(oracle.rope(q, prev_seq=106) * oracle.rope(k, prev_seq=100)))
+    assert abs(d1 - d2) < 1e-3
+    # per-sequence start positions equal separate calls with scalar prev_seq
+    pos0 = np.array([4, 9], np.int32)
+    yp = oracle.rope(x, pos0=pos0)
+    for b in range(B):
+        np.testing.assert_array_equal(yp[b:b + 1], oracle.rope(x[b:b + 1], prev_seq=int(pos0[b])))
+
+
+def test_kv_append_equals_slice_and_concat_scatter(oracle):
+    B, H, Lmax, D = 1, 2, 6, 4
+    past = oracle.gen_normal((B, H, Lmax, D), 80)
+    new = oracle.gen_normal((B, H, 1, D), 81)
+    for step_pos in range(Lmax):  # includes the two special cases of the reference (first and last row)
+        got = oracle.kv_append(past, new, np.array([step_pos], np.int32))
+        np.testing.assert_array_equal(got, oracle.kv_scatter_replay(past, new, step_pos))
+    # several tokens, per-sequence positions, rows past the end are dropped
+    past = oracle.gen_normal((2, 2, 5, 4), 82)
+    new = oracle.gen_normal((2, 2, 3, 4), 83)
+    got = oracle.kv_append(past, new, np.array([1, 3], np.int32))
+    want = past.copy()
+    want[0, :, 1:4] = new[0]
+    want[1, :, 3:5] = new[1, :, :2]
+    np.testing.assert_array_equal(got, want)

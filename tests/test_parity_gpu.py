@@ -315,3 +315,66 @@ def test_rerun_is_bitwise_deterministic(lm, hip, oracle):
     np.testing.assert_array_equal(a, b)
     qd, kd, vd = inputs(oracle, (4, 8, 128), (4, 2, 3000, 128), "bf16", 8400)
     np.testing.assert_array_equal(run_decode(lm, hip, qd, kd, vd, "bf16"), run_decode(lm, hip, qd, kd, vd, "bf16"))
+
+
+# ---------------------------------------------------------------------------------------------
+# rotary embedding and KV-cache append
+# ---------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("dtype", ["f32", "f16", "bf16"])
+@pytest.mark.parametrize("interleaved", [False, True])
+def test_rope(lm, hip, oracle, dtype, interleaved):
+    B, H, S, D = 2, 3, 37, 64
+    x = oracle.round_to(oracle.gen_normal((B, H, S, D), 9000), dtype)
+    dx = lm.to_device(x, hip, dtype)
+    got = lm.apply_rotary_embeddings(dx, prev_seq=100, interleaved=interleaved).to_host()
+    want = oracle.round_to(oracle.rope(x, prev_seq=100, interleaved=interleaved), dtype)
+    # fp32: 1e-5 of the output range plus the spread of sin/cos at ~100 rad between libm and the GPU
+    tol = {"f32": 2e-5, "f16": 2e-3, "bf16": 8e-3}[dtype]  # bf16 output rounding alone is up to 2^-8
+    assert rel_err(got, want) <= tol
+    # per-sequence positions, in place
+    pos0 = np.array([5, 2000], np.int32)
+    lm.apply_rotary_embeddings(dx, pos0=lm.to_device(pos0, hip), out=dx, interleaved=interleaved)
+    want = oracle.round_to(oracle.rope(x, pos0=pos0, interleaved=interleaved), dtype)
+    assert rel_err(dx.to_host(), want) <= tol * (10 if dtype == "f32" else 1)  # 2000 rad: fp32 angle rounding
+
+
+def test_rope_reference_graph_replay_fp32(lm, hip, oracle):
+    x = oracle.gen_normal((1, 8, 128, 64), 9100)
+    got = lm.apply_rotary_embeddings(lm.to_device(x, hip), prev_seq=0).to_host()
+    assert rel_err(got, oracle.rope_column_major_replay(x, prev_seq=0)) <= 2e-5
+
+
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+def test_kv_append_in_place(lm, hip, oracle, dtype):
+    B, Hkv, Lmax, D, T = 3, 2, 50, 128, 2
+    kc = oracle.round_to(oracle.gen_normal((B, Hkv, Lmax, D), 9200), dtype)
+    vc = oracle.round_to(oracle.gen_normal((B, Hkv, Lmax, D), 9201), dtype)
+    kn = oracle.round_to(oracle.gen_normal((B, Hkv, T, D), 9202), dtype)
+    vn = oracle.round_to(oracle.gen_normal((B, Hkv, T, D), 9203), dtype)
+    pos = np.array([0, 17, 49], np.int32)  # the last sequence has room for one of its two rows
+    dk, dv, dkn, dvn = (lm.to_device(a, hip, dtype) for a in (kc, vc, kn, vn))
+    lm.kv_append(dk, dv, dkn, dvn, lm.to_device(pos, hip))
+    np.testing.assert_array_equal(dk.to_host(), oracle.kv_append(kc, kn, pos))
+    np.testing.assert_array_equal(dv.to_host(), oracle.kv_append(vc, vn, pos))
+    # fused rotary embedding of K: equals rope at the row position, then append; V untouched
+    dk2, dv2 = lm.to_device(kc, hip, dtype), lm.to_device(vc, hip, dtype)
+    lm.kv_append(dk2, dv2, dkn, dvn, lm.to_device(pos, hip), rope_k=True)
+    kn_rot = oracle.round_to(oracle.rope(kn, pos0=pos), dtype)
+    tol = 2e-5 if dtype == "f32" else 8e-3
+    assert rel_err(dk2.to_host(), oracle.kv_append(kc, kn_rot, pos)) <= tol
+    np.testing.assert_array_equal(dv2.to_host(), oracle.kv_append(vc, vn, pos))
+
+
+def test_incremental_decode_equals_causal_prefill(lm, hip, oracle):
+    """Token-by-token decode through KVCacheState (append + fused cached attention) reproduces causal
+    prefill row by row — the end-to-end property the reference's cached path is built on
+    (reference src/Whisper.jl:584-620 with the cache update of :552-570)."""
+    B, Hq, Hkv, S, D = 2, 8, 2, 40, 64
+    q, k, v = inputs(oracle, (B, Hq, S, D), (B, Hkv, S, D), "f32", 9300)
+    want = oracle.flash_attn(q, k, v, causal=True)
+    cache = lm.KVCacheState(B, Hkv, D, max_seq=64, dtype="f32", device=hip)
+    for t in range(S):
+        cache.append(lm.to_device(np.ascontiguousarray(k[:, :, t:t + 1]), hip), lm.to_device(np.ascontiguousarray(v[:, :, t:t + 1]), hip))
+        out = cache.attend(lm.to_device(np.ascontiguousarray(q[:, :, t]), hip)).to_host()
+        assert rel_err(out, want[:, :, t]) <= 1e-5, t
+    assert cache.step_pos == S
