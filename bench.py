@@ -159,8 +159,6 @@ def decode_leg(lm, dev, steps, warmup, cpu_seconds, num_splits=0):
     B, Hq, Hkv, Lmax, D = 64, 32, 8, 32768, 128
     rng = np.random.default_rng(5)
     lens = rng.integers(8192, 32768, size=B, endpoint=True).astype(np.int32)
-    if os.environ.get("LMH_EXP_FULL_LENS"):
-        lens[:] = int(os.environ["LMH_EXP_FULL_LENS"])
     pool_rows = 1 << 18  # 256 Ki rows of 128 bf16 = 64 MiB per pool
     pools_host = [lm.f32_to_bf16_bits(rng.standard_normal((pool_rows, D), dtype=np.float32)) for _ in range(2)]
     kpool, vpool = (lm.HipArray((pool_rows, D), "bf16", dev).copy_from_host(x) for x in pools_host)

@@ -19,7 +19,9 @@ HIPCC_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fno-gpu-rdc",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wno-unused-command-line-argument",
-] + os.environ.get("LMH_EXTRA_FLAGS", "").split()
+]
+# extra -D switches for one-off kernel experiments (never set by the tests, the bench or the driver)
+HIPCC_FLAGS += os.environ.get("LMH_EXTRA_FLAGS", "").split()
 
 
 def hipcc_path():

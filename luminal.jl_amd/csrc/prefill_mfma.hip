@@ -29,22 +29,13 @@ namespace {
 
 constexpr int BM = 128;  // query rows per workgroup
 constexpr int BN = 64;   // keys per tile
-#ifndef LMH_PREFILL_WAVES
-#define LMH_PREFILL_WAVES 2
-#endif
-#ifndef LMH_PREFILL_PAIR
-#define LMH_PREFILL_PAIR 0
-#endif
-#ifndef LMH_PREFILL_PADK
-#define LMH_PREFILL_PADK 8
-#endif
-#ifndef LMH_PREFILL_PADV
-#define LMH_PREFILL_PADV 0
-#endif
-// LDS row paddings in elements; K rows are read 16 bytes per lane (one row per lane), V rows through
-// the transposing read (4 rows x 32 bytes per 16 lanes), so the two tiles want different strides.
-constexpr int kPadK = LMH_PREFILL_PADK;
-constexpr int kPadV = LMH_PREFILL_PADV;
+// LDS row paddings in elements. K rows are read 16 bytes per lane, one row per lane: a stride of
+// D + 8 elements spreads 16 consecutive rows over all banks (5 cycles per 1 KB fragment per CU,
+// against 16 unpadded). V rows go through the transposing read (4 rows x 32 bytes per 16 lanes),
+// which is conflict-free when the stride is 96 elements modulo 128 (5.6 cycles per fragment, against
+// 8 at D + 8 and 16 at a multiple of 128 bytes): no padding for D = 96, +32 for D = 64 and 128.
+constexpr int kPadK = 8;
+template <int D> constexpr int pad_v() { return D == 96 ? 0 : 32; }
 constexpr float kLog2e = 1.4426950408889634f;
 // The running max is only raised (and the output rescaled) when a row's scores outgrow it by more
 // than this many powers of two; until then P is computed against the stale max and may reach
@@ -97,14 +88,14 @@ struct MfmaBF16 {
 };
 
 template <typename MT, int D, bool CAUSAL>
-__global__ __launch_bounds__(256, LMH_PREFILL_WAVES) void prefill_mfma_kernel(PrefillArgs a, int n_q_tiles, int n_bh_groups) {
+__global__ __launch_bounds__(256, (D <= 96 ? 3 : 2)) void prefill_mfma_kernel(PrefillArgs a, int n_q_tiles, int n_bh_groups) {
   using vec8 = typename MT::vec8;
   constexpr int KS = D / 16;       // k-steps of the S^T product
   constexpr int DB = D / 32;       // 32-row blocks of O^T
   constexpr int CPR = D / 8;       // 16-byte chunks per K/V row
   constexpr int CH = BN * CPR / 256;  // chunks per thread per tile
   constexpr int LDK = D + kPadK;   // LDS row strides in elements
-  constexpr int LDV = D + kPadV;
+  constexpr int LDV = D + pad_v<D>();
 
   __shared__ __attribute__((aligned(16))) uint16_t Ks2[2][BN * LDK];  // double-buffered tiles
   __shared__ __attribute__((aligned(16))) uint16_t Vs2[2][BN * LDV];
@@ -118,14 +109,11 @@ __global__ __launch_bounds__(256, LMH_PREFILL_WAVES) void prefill_mfma_kernel(Pr
   if (bh >= a.B * a.Hq) return;
   const int b = bh / a.Hq, hq = bh % a.Hq;
   const int kvh = kv_head_of(hq, a.Hq, a.Hkv, a.head_map);
-  // Causal rows grow with the query index, so a workgroup takes query tile (n - 1 - r) and then
-  // tile r: every workgroup of a head then does the same amount of work and the launch has no
-  // long tail of late, heavy tiles. Without a mask all tiles cost the same and r is the tile.
-  const int n_pass = (CAUSAL && LMH_PREFILL_PAIR && tile_rank != n_q_tiles - 1 - tile_rank) ? 2 : 1;
-  for (int pass = 0; pass < n_pass; pass++) {
-  const int q_tile = (CAUSAL && pass == 0) ? (n_q_tiles - 1 - tile_rank) : tile_rank;
+  // Causal rows grow with the query index: long rows are issued first so that the short ones fill
+  // the tail of the launch. (Pairing tile r with tile n-1-r in one workgroup equalises the work but
+  // halves the number of workgroups; measured 15 % slower on the S = 4096 workload.)
+  const int q_tile = CAUSAL ? (n_q_tiles - 1 - tile_rank) : tile_rank;
   const int q0 = q_tile * BM;
-  if (pass > 0) __syncthreads();  // the tiles of the previous pass are no longer read
 
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = tid >> 6;
@@ -331,15 +319,13 @@ __global__ __launch_bounds__(256, LMH_PREFILL_WAVES) void prefill_mfma_kernel(Pr
         *reinterpret_cast<uint2 *>(op + d) = packed;
       }
   }
-  }  // pass
 }
 
 template <typename MT, int D>
 int launch_for_d(const PrefillArgs &a, hipStream_t stream) {
   const int n_q_tiles = (a.Sq + BM - 1) / BM;
   const int n_bh_groups = (a.B * a.Hq + 7) / 8;
-  const int n_ranks = (a.causal && LMH_PREFILL_PAIR) ? (n_q_tiles + 1) / 2 : n_q_tiles;
-  dim3 grid(8 * n_bh_groups * n_ranks), block(256);
+  dim3 grid(8 * n_bh_groups * n_q_tiles), block(256);
   if (a.causal)
     hipLaunchKernelGGL((prefill_mfma_kernel<MT, D, true>), grid, block, 0, stream, a, n_q_tiles, n_bh_groups);
   else
