@@ -139,6 +139,13 @@ def prefill_leg(lm, dev, steps, warmup, cpu_seconds):
         res["parity"] = {"max_rel_err": worst, "tolerance": 2e-3, "checked": "heads 0..%d vs CPU oracle" % (heads - 1)}
         if worst > 2e-3:
             raise SystemExit("prefill parity check failed: rel err %.3g > 2e-3" % worst)
+        # the reference's own execution model is one scalar thread: same oracle, one thread, one head
+        t0 = time.perf_counter()
+        oracle.flash_attn(q32[:, :1], k32[:, :1], v32[:, :1], scale=scale, causal=True, nthreads=1)
+        t1 = time.perf_counter() - t0
+        res["cpu_baseline_single_thread"] = {"value": flops / H / t1 / 1e12, "unit": "TFLOP/s", "cores": 1, "kind": "port",
+                                             "sample": "head 0 of %d, all %d query rows, %.1f s" % (H, S, t1)}
+        log("[prefill] CPU oracle, 1 thread: head 0 in %.1f s = %.5f TFLOP/s" % (t1, flops / H / t1 / 1e12))
     return res
 
 
@@ -310,6 +317,7 @@ def main():
         line["roofline"] = r["roofline"]
         if "cpu_baseline" in r:
             line["cpu_baseline"], line["parity"] = r["cpu_baseline"], r["parity"]
+            line["cpu_baseline_single_thread"] = r["cpu_baseline_single_thread"]
     if args.only in ("all", "decode"):
         line["decode"] = decode_leg(lm, dev, args.steps, args.warmup, args.cpu_seconds, args.decode_splits)
     if args.only == "all":
