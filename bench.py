@@ -108,12 +108,17 @@ def prefill_leg(lm, dev, steps, warmup, cpu_seconds):
     kern_tflops = flops / (ev_ms * 1e-3) / 1e12
     log("[prefill] C2 causal fp16 B=1 H=32 S=4096 D=96: %.1f us/step wall, %.1f us/launch events, %.1f TFLOP/s (%.1f%% of %g)"
         % (wall_ms * 1e3, ev_ms * 1e3, kern_tflops, 100 * kern_tflops / PEAK_FP16_TFLOPS, PEAK_FP16_TFLOPS))
+    sustained = mfma_sustained(lm, dev, dq)
     res = {
         "ms_per_step": wall_ms, "value": tflops,
         "roofline": {"bound": "mfma", "achieved": kern_tflops, "peak": PEAK_FP16_TFLOPS, "unit": "TFLOP/s",
                      "frac": kern_tflops / PEAK_FP16_TFLOPS, "traffic": PREFILL_TRAFFIC_BYTES,
                      "kernel": "prefill_mfma_kernel<MfmaF16, 96, causal>", "launch_us": ev_ms * 1e3,
-                     "algorithmic_flops_per_launch": flops},
+                     "algorithmic_flops_per_launch": flops,
+                     # what a bare MFMA loop sustains on this GPU right now (clock management under load):
+                     # on all-zero operands and on the Q tensor of this workload
+                     "mfma_sustained_tflops": sustained,
+                     "frac_of_sustained": kern_tflops / sustained["workload_operands"]},
     }
     if cpu_seconds > 0:
         # CPU baseline = the oracle on a head subset of the same workload, all host threads; the same
@@ -147,6 +152,22 @@ def prefill_leg(lm, dev, steps, warmup, cpu_seconds):
                                              "sample": "head 0 of %d, all %d query rows, %.1f s" % (H, S, t1)}
         log("[prefill] CPU oracle, 1 thread: head 0 in %.1f s = %.5f TFLOP/s" % (t1, flops / H / t1 / 1e12))
     return res
+
+
+def mfma_sustained(lm, dev, operands):
+    """TFLOP/s of lmh_calib_mfma (a bare v_mfma_f32_32x32x16_f16 loop on the whole chip) on zeros and on `operands`."""
+    sink = lm.HipArray((512 * 256,), "f32", dev)
+    zeros = lm.HipArray((1 << 16,), "f16", dev).fill_bytes(0)
+    out = {}
+    for name, buf, nbytes in (("zero_operands", zeros, 1 << 17), ("workload_operands", operands, 1 << 17)):
+        flops = [0.0]
+        def fn():
+            flops[0] = lm.binding.calib_mfma(sink.ptr, buf.ptr, nbytes, 40000)
+        _, ev = time_steps(fn, 3, 1, lm.binding)
+        out[name] = flops[0] / (ev * 1e-3) / 1e12
+    log("[prefill] bare MFMA loop sustains %.0f TFLOP/s on zero operands, %.0f TFLOP/s on the workload's Q values (published peak %g)"
+        % (out["zero_operands"], out["workload_operands"], PEAK_FP16_TFLOPS))
+    return out
 
 
 def fill_cache_from_pool(lm, cache, pool, lens, Hkv, Lmax, D, rng):

@@ -80,6 +80,13 @@ int lmh_event_elapsed_ms(float *ms, void *start, void *stop);
  * counters against a known transfer. */
 int lmh_calib_copy(void *dst_dev, const void *src_dev, size_t bytes, void *stream);
 
+/* Measurement aid with no counterpart in the reference: a bare loop of fp16 MFMAs (512 workgroups, 4
+ * waves each, 8 v_mfma_f32_32x32x16_f16 per iteration) on operands read from `operands_dev`
+ * (`operand_bytes` >= 32, a multiple of 16). The sustained matrix-core rate depends on the operand
+ * values (clock management under load), so time it on data like the attention inputs. `sink_dev`
+ * receives 512*256 floats; `*flops` (host, optional) the flops of one launch. */
+int lmh_calib_mfma(void *sink_dev, const void *operands_dev, size_t operand_bytes, int iters, double *flops, void *stream);
+
 /* ---- flash attention forward: replaces
  *   execute_op!(out, op::FlashAttentionOp, q, k, v)   reference src/Execution.jl:565-578
  *   flash_attn_cpu(q, k, v, scale, causal)            reference src/Execution.jl:453-479

@@ -23,7 +23,7 @@ EXPORTS = [
     "lmh_version", "lmh_last_error", "lmh_device_count", "lmh_init", "lmh_device_name", "lmh_malloc", "lmh_free",
     "lmh_memset", "lmh_memcpy_h2d", "lmh_memcpy_d2h", "lmh_memcpy_d2d", "lmh_sync", "lmh_event_create",
     "lmh_event_destroy", "lmh_event_record", "lmh_event_elapsed_ms", "lmh_flash_attn_fwd",
-    "lmh_decode_workspace_bytes", "lmh_decode_auto_splits", "lmh_decode_attn", "lmh_calib_copy", "lmh_rope",
+    "lmh_decode_workspace_bytes", "lmh_decode_auto_splits", "lmh_decode_attn", "lmh_calib_copy", "lmh_calib_mfma", "lmh_rope",
     "lmh_kv_append",
 ]
 
@@ -121,9 +121,10 @@ def load():
     L.lmh_decode_auto_splits.restype = ctypes.c_int32
     L.lmh_decode_auto_splits.argtypes = [ctypes.c_int32] * 3
     L.lmh_calib_copy.argtypes = [vp, vp, ctypes.c_size_t, vp]
+    L.lmh_calib_mfma.argtypes = [vp, vp, ctypes.c_size_t, ctypes.c_int, ctypes.POINTER(ctypes.c_double), vp]
     L.lmh_rope.argtypes = [ctypes.POINTER(RopeParams)]
     L.lmh_kv_append.argtypes = [ctypes.POINTER(KvAppendParams)]
-    for name in ("lmh_rope", "lmh_kv_append", "lmh_calib_copy", "lmh_init", "lmh_device_name", "lmh_malloc", "lmh_free", "lmh_memset", "lmh_memcpy_h2d",
+    for name in ("lmh_rope", "lmh_kv_append", "lmh_calib_copy", "lmh_calib_mfma", "lmh_init", "lmh_device_name", "lmh_malloc", "lmh_free", "lmh_memset", "lmh_memcpy_h2d",
                  "lmh_memcpy_d2h", "lmh_memcpy_d2d", "lmh_sync", "lmh_event_create", "lmh_event_destroy",
                  "lmh_event_record", "lmh_event_elapsed_ms", "lmh_flash_attn_fwd", "lmh_decode_attn"):
         getattr(L, name).restype = ctypes.c_int
@@ -220,6 +221,13 @@ def kv_append(params):
 
 def calib_copy(dst, src, nbytes, stream=None):
     check(load().lmh_calib_copy(dst, src, nbytes, stream))
+
+
+def calib_mfma(sink, operands, operand_bytes, iters, stream=None):
+    """Launch the bare MFMA loop; returns the flops of the launch."""
+    flops = ctypes.c_double(0.0)
+    check(load().lmh_calib_mfma(sink, operands, operand_bytes, iters, ctypes.byref(flops), stream))
+    return flops.value
 
 
 def decode_workspace_bytes(B, Hq, Hkv, Lmax, D, num_splits=0):

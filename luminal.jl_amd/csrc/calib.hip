@@ -1,10 +1,47 @@
 // A plain device-to-device copy kernel of known size. It exists so that hardware traffic counters
 // (FETCH_SIZE / WRITE_SIZE) can be scaled: profile this kernel on N bytes, read what the counter
 // reports, and apply the same factor to the attention kernels' readings.
+//
+// A bare MFMA loop on caller-supplied operands. The published matrix-core peak assumes the boost clock;
+// under a full-chip MFMA load the clock is power-managed and depends on how many operand bits toggle
+// (all-zero operands sustain a much higher rate than random ones). Timing this kernel on the same
+// kind of data as the attention inputs gives the rate the matrix cores can actually sustain, the
+// ceiling an attention kernel is measured against besides the published figure.
 #include "common.hpp"
 
 namespace lmh {
 namespace {
+typedef _Float16 calib_half8_t __attribute__((ext_vector_type(8)));
+typedef float calib_floatx16_t __attribute__((ext_vector_type(16)));
+constexpr int kCalibMfmaGrid = 512;    // two workgroups per CU
+constexpr int kCalibMfmaPerIter = 8;   // MFMAs per wave per loop iteration
+
+__global__ __launch_bounds__(256, 2) void calib_mfma_kernel(float *__restrict__ sink, const calib_half8_t *__restrict__ operands,
+                                                            int n_operands, int iters) {
+  calib_half8_t a[4], b[4];
+#pragma unroll
+  for (int i = 0; i < 4; i++) {
+    a[i] = operands[(threadIdx.x * 4 + i) % n_operands];
+    b[i] = operands[(threadIdx.x * 4 + i + n_operands / 2) % n_operands];
+  }
+  calib_floatx16_t acc[4];
+#pragma unroll
+  for (int c = 0; c < 4; c++)
+#pragma unroll
+    for (int i = 0; i < 16; i++) acc[c][i] = 0.f;
+  for (int it = 0; it < iters; it++) {
+#pragma unroll
+    for (int m = 0; m < kCalibMfmaPerIter; m++)
+      acc[m & 3] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[m & 3], b[(m >> 1) & 3], acc[m & 3], 0, 0, 0);
+  }
+  float s = 0.f;
+#pragma unroll
+  for (int c = 0; c < 4; c++)
+#pragma unroll
+    for (int i = 0; i < 16; i++) s += acc[c][i];
+  sink[blockIdx.x * 256 + threadIdx.x] = s;
+}
+
 __global__ __launch_bounds__(256) void calib_copy_kernel(uint4 *__restrict__ dst, const uint4 *__restrict__ src, size_t n) {
   size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
   const size_t stride = (size_t)gridDim.x * blockDim.x;
@@ -22,5 +59,17 @@ extern "C" int lmh_calib_copy(void *dst, const void *src, size_t bytes, void *st
   hipLaunchKernelGGL(calib_copy_kernel, dim3(8192), dim3(256), 0, (hipStream_t)stream, reinterpret_cast<uint4 *>(dst),
                      reinterpret_cast<const uint4 *>(src), bytes / 16);
   LMH_HIP_TRY(hipGetLastError());
+  return LMH_OK;
+}
+
+extern "C" int lmh_calib_mfma(void *sink, const void *operands, size_t operand_bytes, int iters, double *flops, void *stream) {
+  using namespace lmh;
+  if (!sink || !operands) return fail(LMH_E_NULL, "lmh_calib_mfma: null pointer");
+  if (operand_bytes < 32 || operand_bytes % 16 != 0 || (reinterpret_cast<uintptr_t>(operands) & 15u) || iters < 1)
+    return fail(LMH_E_SHAPE, "lmh_calib_mfma: operands must be >= 32 bytes, a multiple of 16, 16-byte aligned; iters >= 1");
+  hipLaunchKernelGGL(calib_mfma_kernel, dim3(kCalibMfmaGrid), dim3(256), 0, (hipStream_t)stream, reinterpret_cast<float *>(sink),
+                     reinterpret_cast<const calib_half8_t *>(operands), (int)(operand_bytes / 16), iters);
+  LMH_HIP_TRY(hipGetLastError());
+  if (flops) *flops = (double)kCalibMfmaGrid * 4.0 * iters * kCalibMfmaPerIter * (2.0 * 32 * 32 * 16);
   return LMH_OK;
 }
