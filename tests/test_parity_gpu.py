@@ -378,3 +378,21 @@ def test_incremental_decode_equals_causal_prefill(lm, hip, oracle):
         out = cache.attend(lm.to_device(np.ascontiguousarray(q[:, :, t]), hip)).to_host()
         assert rel_err(out, want[:, :, t]) <= 1e-5, t
     assert cache.step_pos == S
+
+
+def test_calibration_kernels(lm, hip):
+    # measurement aids: the copy kernel copies, the bare MFMA loop reports its flops and checks its arguments
+    n = 1 << 16
+    src = lm.HipArray((n,), "f32", hip).copy_from_host(np.arange(n, dtype=np.float32))
+    dst = lm.HipArray((n,), "f32", hip).fill_bytes(0)
+    lm.binding.calib_copy(dst.ptr, src.ptr, n * 4)
+    assert np.array_equal(dst.to_host(), np.arange(n, dtype=np.float32))
+    sink = lm.HipArray((512 * 256,), "f32", hip).fill_bytes(0xFF)
+    ones = lm.HipArray((1 << 12,), "f16", hip).copy_from_host(np.ones(1 << 12, np.float16))
+    flops = lm.binding.calib_mfma(sink.ptr, ones.ptr, 1 << 13, 3)
+    assert flops == 512 * 4 * 3 * 8 * 2 * 32 * 32 * 16
+    got = sink.to_host()
+    # every accumulator element is a sum of 16 products 1*1 per MFMA: 6 MFMAs per accumulator, 64 elements per lane
+    assert np.all(got == 64 * 16 * 6)
+    with pytest.raises(lm.LuminalHipError):
+        lm.binding.calib_mfma(sink.ptr, ones.ptr, 24, 1)
