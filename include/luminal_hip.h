@@ -30,7 +30,7 @@ extern "C" {
 #define LMH_E_NULL (-1)        /* a required pointer is null */
 #define LMH_E_SHAPE (-2)       /* non-positive or inconsistent dimension / stride */
 #define LMH_E_UNSUPPORTED (-3) /* head dim / dtype / head map not implemented */
-#define LMH_E_WORKSPACE (-4)   /* decode workspace missing or too small */
+#define LMH_E_WORKSPACE (-4)   /* decode workspace missing, too small or not 16-byte aligned */
 #define LMH_E_HIP (-5)         /* a HIP runtime call failed */
 #define LMH_E_NODEVICE (-6)    /* no usable gfx950 device */
 
@@ -140,7 +140,7 @@ typedef struct lmh_decode_params {
   int32_t head_map;
   int32_t out_f32;       /* 0: out has element type `dtype`; 1: out is fp32 */
   int32_t num_splits;    /* KV splits per (b, kv head); 0 = choose */
-  void *workspace;       /* device, >= lmh_decode_workspace_bytes(...) */
+  void *workspace;       /* device, 16-byte aligned, >= lmh_decode_workspace_bytes(...) */
   size_t workspace_bytes;
   void *stream;
 } lmh_decode_params;

@@ -297,6 +297,7 @@ int lmh_decode_attn(const lmh_decode_params *p) {
     if (!p->workspace || p->workspace_bytes < need)
       return fail(LMH_E_WORKSPACE, "lmh_decode_attn: workspace of %zu bytes needed for %d splits, got %zu", need,
                   a.num_splits, p->workspace ? p->workspace_bytes : (size_t)0);
+    if (!aligned16(p->workspace)) return fail(LMH_E_WORKSPACE, "lmh_decode_attn: workspace must be 16-byte aligned");
     a.ws_o = reinterpret_cast<float *>(p->workspace);
     a.ws_ml = a.ws_o + (size_t)p->B * p->Hq * a.num_splits * p->D;
   }

@@ -280,30 +280,74 @@ __global__ __launch_bounds__(kWaves * 64) void decode_split_kernel(DecodeArgs a,
 }
 
 // out[b,hq,:] = sum_s o_s 2^(m_s - M) / sum_s l_s 2^(m_s - M) over the splits that exist.
+// One workgroup per (b, hq). The slot statistics are fetched in parallel (one slot per thread), reduced
+// across the workgroup, and the per-slot weights go through LDS, so the loop over slots that follows
+// issues independent loads of the partial outputs instead of a chain of dependent ones.
+constexpr int kMergeThreads = 128;
+constexpr int kMergeMaxSlots = 1024;  // weights kept in LDS; more slots than this take the strided path below
 template <typename E>
-__global__ __launch_bounds__(128) void decode_merge_kernel(DecodeArgs a) {
+__global__ __launch_bounds__(kMergeThreads) void decode_merge_kernel(DecodeArgs a) {
   using raw = typename E::raw;
+  __shared__ float w_s[kMergeMaxSlots];
+  __shared__ float red_m[kMergeThreads / 64], red_l[kMergeThreads / 64];
   const int hq = blockIdx.x, b = blockIdx.y;
+  const int tid = threadIdx.x;
   int L = a.kv_len ? a.kv_len[b] : a.Lmax;
   L = min(max(L, 0), a.Lmax);
   const int n = (L + a.chunk - 1) / a.chunk;
   const int64_t off = b * a.os[0] + hq * a.os[1];
   const int64_t row0 = ((int64_t)b * a.Hq + hq) * a.num_splits;
+  const float2 *ml = reinterpret_cast<const float2 *>(a.ws_ml) + row0;
+
+  // running max over the slots
   float M = -INFINITY;
-  for (int s = 0; s < n; s++) M = fmaxf(M, a.ws_ml[(row0 + s) * 2]);
+  for (int s = tid; s < n; s += kMergeThreads) M = fmaxf(M, ml[s].x);
+#pragma unroll
+  for (int o = 32; o >= 1; o >>= 1) M = fmaxf(M, __shfl_xor(M, o));
+  if ((tid & 63) == 0) red_m[tid >> 6] = M;
+  __syncthreads();
+  M = red_m[0];
+#pragma unroll
+  for (int w = 1; w < kMergeThreads / 64; w++) M = fmaxf(M, red_m[w]);
+
+  // weights 2^(m_s - M) (0 for a slot marked (-inf, 0): it was folded into an earlier slot of the same
+  // run and its output row is unset) and the normaliser
   float lsum = 0.f;
-  for (int s = 0; s < n; s++) {
-    const float ms = a.ws_ml[(row0 + s) * 2];
-    if (ms != -INFINITY) lsum += a.ws_ml[(row0 + s) * 2 + 1] * __builtin_amdgcn_exp2f(ms - M);
+  for (int s = tid; s < n; s += kMergeThreads) {
+    const float2 v = ml[s];
+    const float w = v.x == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(v.x - M);
+    if (s < kMergeMaxSlots) w_s[s] = w;
+    lsum += v.y * w;
   }
+#pragma unroll
+  for (int o = 32; o >= 1; o >>= 1) lsum += __shfl_xor(lsum, o);
+  if ((tid & 63) == 0) red_l[tid >> 6] = lsum;
+  __syncthreads();
+  lsum = 0.f;
+#pragma unroll
+  for (int w = 0; w < kMergeThreads / 64; w++) lsum += red_l[w];
   const float inv = 1.f / lsum;
-  for (int d = threadIdx.x; d < a.D; d += blockDim.x) {
-    float o = 0.f;
-    for (int s = 0; s < n; s++) {
-      const float ms = a.ws_ml[(row0 + s) * 2];
-      // a slot marked (-inf, 0) was folded into an earlier slot of the same run: its output row is unset
-      if (ms != -INFINITY) o += a.ws_o[(row0 + s) * a.D + d] * __builtin_amdgcn_exp2f(ms - M);
+
+  const float *po = a.ws_o + row0 * a.D;
+  for (int d = tid; d < a.D; d += kMergeThreads) {
+    float acc[4] = {0.f, 0.f, 0.f, 0.f};
+    int s = 0;
+    const int n_lds = min(n, kMergeMaxSlots);
+    for (; s + 4 <= n_lds; s += 4) {
+#pragma unroll
+      for (int u = 0; u < 4; u++) {
+        const float w = w_s[s + u];
+        // the row of a zero-weight slot is unset memory: select, do not multiply
+        const float x = po[(int64_t)(s + u) * a.D + d];
+        acc[u] += w != 0.f ? x * w : 0.f;
+      }
     }
+    for (; s < n; s++) {
+      const float w = s < kMergeMaxSlots ? w_s[s] : (ml[s].x == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(ml[s].x - M));
+      const float x = po[(int64_t)s * a.D + d];
+      acc[0] += w != 0.f ? x * w : 0.f;
+    }
+    const float o = (acc[0] + acc[1]) + (acc[2] + acc[3]);
     if (a.out_f32) reinterpret_cast<float *>(a.out)[off + d] = o * inv;
     else reinterpret_cast<raw *>(a.out)[off + d] = E::st(o * inv);
   }
@@ -312,7 +356,7 @@ __global__ __launch_bounds__(128) void decode_merge_kernel(DecodeArgs a) {
 template <typename E>
 int launch_merge(const DecodeArgs &a, hipStream_t stream) {
   if (a.num_splits > 1) {
-    hipLaunchKernelGGL((decode_merge_kernel<E>), dim3(a.Hq, a.B), dim3(128), 0, stream, a);
+    hipLaunchKernelGGL((decode_merge_kernel<E>), dim3(a.Hq, a.B), dim3(kMergeThreads), 0, stream, a);
     LMH_HIP_TRY(hipGetLastError());
   }
   return LMH_OK;

@@ -157,7 +157,22 @@ class HipArray:
         binding.memset(self.ptr, value, self.nbytes)
         return self
 
+    def view(self, shape):
+        """Same memory under another shape of equal size (Base.reshape); the view keeps this array alive and
+        frees nothing."""
+        shape = tuple(int(x) for x in shape)
+        if int(np.prod(shape, dtype=np.int64)) != self.size:
+            raise ValueError("reshape: %s has %d elements, %s needs %d" % (self.shape, self.size, shape,
+                                                                          int(np.prod(shape, dtype=np.int64))))
+        v = HipArray.__new__(HipArray)
+        v.shape, v.dtype, v.device, v.nbytes, v.ptr = shape, self.dtype, self.device, self.nbytes, self.ptr
+        v._base = self
+        return v
+
     def free(self):
+        if getattr(self, "_base", None) is not None:
+            self.ptr = 0
+            return
         if getattr(self, "ptr", 0):
             binding.free(self.ptr)
             self.ptr = 0
@@ -221,6 +236,26 @@ class DecodeAttentionOp(Op):
         self.out_dtype = out_dtype
 
 
+class RotaryEmbeddingOp(Op):
+    """apply_rotary_embeddings(input, prev_seq; base) (reference src/NN.jl:253-303) as one node; inputs (x,) or
+    (x, pos0) with pos0 an int32[B] tensor of per-sequence start positions."""
+
+    def __init__(self, prev_seq=0, base=10000.0, interleaved=False):
+        self.prev_seq = int(prev_seq)
+        self.base = float(base)
+        self.interleaved = bool(interleaved)
+
+
+class KVAppendOp(Op):
+    """In-place cache update (the reference rebuilds the cache with _kv_scatter, src/Whisper.jl:552-570); inputs
+    (k_cache, v_cache, k_new, v_new, pos); outputs 0 and 1 are the two caches themselves (same buffers)."""
+
+    def __init__(self, rope_k=False, base=10000.0, interleaved=False):
+        self.rope_k = bool(rope_k)
+        self.base = float(base)
+        self.interleaved = bool(interleaved)
+
+
 class Node:
     def __init__(self, op, inputs):
         self.op = op
@@ -228,8 +263,9 @@ class Node:
 
 
 class GraphTensor:
-    def __init__(self, id, shape, graph_ref):
+    def __init__(self, id, shape, graph_ref, index=0):
         self.id = id
+        self.index = index  # which output of node `id` (reference src/Graph.jl input triples carry the same index)
         self.shape = tuple(shape)
         self.graph_ref = graph_ref
 
@@ -261,7 +297,7 @@ def flash_attention(q, k, v, scale=None, causal=False, head_map=HEADMAP_INTERLEA
     computed in fp32 (reference src/HighLevelOps.jl:377-388)."""
     if scale is None:
         scale = np.float32(1.0) / np.sqrt(np.float32(q.shape[-1]))
-    inputs = [(q.id, 0, q.shape), (k.id, 0, k.shape), (v.id, 0, v.shape)]
+    inputs = [(q.id, q.index, q.shape), (k.id, k.index, k.shape), (v.id, v.index, v.shape)]
     return add_op(q.graph_ref, FlashAttentionOp(np.float32(scale), causal, head_map, out_dtype), inputs, q.shape,
                   out_dtype or q.graph_ref.dtypes[q.id])
 
@@ -271,10 +307,63 @@ def decode_attention(q, k_cache, v_cache, kv_len, scale=None, head_map=HEADMAP_I
     """q: (Batch, Head, HeadDim); caches: (Batch, KVHead, MaxSeq, HeadDim); kv_len: (Batch,) int32."""
     if scale is None:
         scale = np.float32(1.0) / np.sqrt(np.float32(q.shape[-1]))
-    inputs = [(q.id, 0, q.shape), (k_cache.id, 0, k_cache.shape), (v_cache.id, 0, v_cache.shape),
-              (kv_len.id, 0, kv_len.shape)]
+    inputs = [(q.id, q.index, q.shape), (k_cache.id, k_cache.index, k_cache.shape),
+              (v_cache.id, v_cache.index, v_cache.shape), (kv_len.id, kv_len.index, kv_len.shape)]
     return add_op(q.graph_ref, DecodeAttentionOp(np.float32(scale), head_map, num_splits, out_dtype), inputs, q.shape,
                   out_dtype or q.graph_ref.dtypes[q.id])
+
+
+def rotary_embedding(x, prev_seq=0, base=10000.0, pos0=None, interleaved=False):
+    """Graph form of apply_rotary_embeddings (reference src/NN.jl:253-303): x (B,H,S,D); row s of sequence b is
+    rotated by position prev_seq + s, or pos0[b] + s when the int32[B] tensor pos0 is given."""
+    g = x.graph_ref
+    inputs = [(x.id, x.index, x.shape)]
+    if pos0 is not None:
+        inputs.append((pos0.id, pos0.index, pos0.shape))
+    return add_op(g, RotaryEmbeddingOp(prev_seq, base, interleaved), inputs, x.shape, g.dtypes[x.id])
+
+
+def kv_cache_append(k_cache, v_cache, k_new, v_new, pos, rope_k=False, base=10000.0, interleaved=False):
+    """Graph form of the cache update: returns the (k, v) cache tensors after rows pos[b] .. pos[b]+T-1 of sequence
+    b were overwritten by k_new / v_new (K optionally rotated by its position on the way in)."""
+    g = k_cache.graph_ref
+    inputs = [(t.id, t.index, t.shape) for t in (k_cache, v_cache, k_new, v_new, pos)]
+    k_out = add_op(g, KVAppendOp(rope_k, base, interleaved), inputs, k_cache.shape, g.dtypes[k_cache.id])
+    return k_out, GraphTensor(k_out.id, v_cache.shape, g, index=1)
+
+
+def self_attention_core(q, k, v, causal=True, prev_seq=0, rope_base=None, scale=None, head_map=HEADMAP_INTERLEAVED,
+                        out_dtype=None):
+    """What SelfAttention does between its projections (reference src/NN.jl:352-382: rotary embedding of Q and K,
+    repeat_kv, scaled causal softmax attention), emitted as fused nodes: two rotary nodes and one flash attention
+    node that reads the Hkv key/value heads directly (`head_map` INTERLEAVED is the head order repeat_kv produces,
+    src/NN.jl:305-317) instead of materialising G copies. rope_base=None skips the rotary embedding (Whisper's
+    attention layers, reference src/Whisper.jl:263-272 and :310-312, with causal=False for cross attention)."""
+    if rope_base is not None:
+        q = rotary_embedding(q, prev_seq, rope_base)
+        k = rotary_embedding(k, prev_seq, rope_base)
+    return flash_attention(q, k, v, scale=scale, causal=causal, head_map=head_map, out_dtype=out_dtype)
+
+
+def cached_self_attention_core(q, k_new, v_new, k_cache, v_cache, pos, kv_len, rope_base=None, scale=None,
+                               head_map=HEADMAP_INTERLEAVED, num_splits=0, out_dtype=None):
+    """One decode step of a cached attention layer (reference src/Whisper.jl:584-620) as three fused nodes:
+    q (B,Hq,1,D), k_new / v_new (B,Hkv,1,D) are this step's projections, pos int32[B] the row each sequence
+    writes, kv_len = pos + 1 the rows it then attends over. Positions are tensors, so one compiled graph serves
+    every step (the reference compiles one graph per position, src/Decoding.jl:98-106). Returns (out (B,Hq,D),
+    k_cache, v_cache)."""
+    g = q.graph_ref
+    if rope_base is not None:
+        q = rotary_embedding(q, 0, rope_base, pos0=pos)
+    k_cache, v_cache = kv_cache_append(k_cache, v_cache, k_new, v_new, pos, rope_k=rope_base is not None,
+                                       base=rope_base or 10000.0)
+    B, Hq, one, D = q.shape
+    if one != 1:
+        raise ValueError("cached attention takes one query token per sequence; got q %s" % (q.shape,))
+    q3 = GraphTensor(q.id, (B, Hq, D), g, q.index)  # (B,Hq,1,D) and (B,Hq,D) are the same buffer
+    out = decode_attention(q3, k_cache, v_cache, kv_len, scale=scale, head_map=head_map, num_splits=num_splits,
+                           out_dtype=out_dtype)
+    return out, k_cache, v_cache
 
 
 # ---------------------------------------------------------------------------------------------
@@ -358,6 +447,17 @@ def execute_op_inplace(out, op, *inputs, stream=None):
         p.stream = stream
         binding.decode_attn(p)
         return out
+    if isinstance(op, RotaryEmbeddingOp):
+        x = inputs[0]
+        pos0 = inputs[1] if len(inputs) > 1 else None
+        return apply_rotary_embeddings(x, op.prev_seq, op.base, pos0=pos0, out=out, interleaved=op.interleaved,
+                                       stream=stream)
+    if isinstance(op, KVAppendOp):
+        kc, vc, k_new, v_new, pos = inputs
+        if out is not None and not (isinstance(out, tuple) and out[0] is kc and out[1] is vc):
+            raise ValueError("KVAppendOp works in place: its outputs are its cache inputs")
+        kv_append(kc, vc, k_new, v_new, pos, rope_k=op.rope_k, base=op.base, interleaved=op.interleaved, stream=stream)
+        return (kc, vc)
     raise TypeError("no HIP kernel for op %s" % type(op).__name__)
 
 
@@ -365,8 +465,19 @@ def execute_op(op, *inputs):
     """Allocating form: out = similar(q); execute_op!(out, ...) (reference src/Execution.jl:252-255)."""
     q = inputs[0]
     _require_hip(q)
+    if isinstance(op, KVAppendOp):
+        return execute_op_inplace(None, op, *inputs)
     out = HipArray(q.shape, getattr(op, "out_dtype", None) or q.dtype, q.device)
     return execute_op_inplace(out, op, *inputs)
+
+
+def _pick(results, ref):
+    """Value of input triple (node_id, output_index, shape): multi-output nodes store a tuple."""
+    r = results[ref[0]]
+    r = r[ref[1]] if isinstance(r, tuple) else r
+    if isinstance(r, HipArray) and tuple(ref[2]) != r.shape:
+        r = r.view(ref[2])
+    return r
 
 
 def execute(graph, output_ids, initial_inputs, device=None, dtype=None):
@@ -386,8 +497,8 @@ def execute(graph, output_ids, initial_inputs, device=None, dtype=None):
             continue
         if isinstance(node.op, InputTensor):
             raise KeyError("no value given for input tensor %d" % node_id)
-        results[node_id] = execute_op(node.op, *[results[i] for (i, _, _) in node.inputs])
-    final = {i: from_device(results[i]) for i in ids}
+        results[node_id] = execute_op(node.op, *[_pick(results, ref) for ref in node.inputs])
+    final = {i: from_device(results[i][0] if isinstance(results[i], tuple) else results[i]) for i in ids}
     return final[ids[0]] if single else final
 
 
@@ -424,13 +535,15 @@ def compile(graph, device=None):
         raise RuntimeError("compile: no HIP device available and this backend has no CPU path")
     results = []
     for node_id, node in enumerate(graph.nodes):
-        dt = "i32" if graph.dtypes[node_id] == "i32" else graph.dtypes[node_id]
-        results.append(HipArray(graph.shapes[node_id], dt, device).fill_bytes(0))
+        if isinstance(node.op, KVAppendOp):  # in place: the node's outputs are its cache inputs
+            results.append((_pick(results, node.inputs[0]), _pick(results, node.inputs[1])))
+            continue
+        results.append(HipArray(graph.shapes[node_id], graph.dtypes[node_id], device).fill_bytes(0))
     steps = []
     for node_id, node in enumerate(graph.nodes):
         if isinstance(node.op, InputTensor):
             continue
-        args = [results[i] for (i, _, _) in node.inputs]
+        args = [_pick(results, ref) for ref in node.inputs]
         steps.append(lambda out=results[node_id], op=node.op, args=args: execute_op_inplace(out, op, *args))
     return CompiledGraph(steps, results)
 
@@ -524,6 +637,7 @@ def default_scale(D):
 __all__ = [
     "AbstractDevice", "CPUDevice", "HIPDevice", "HipArray", "get_device", "to_device", "from_device", "Graph",
     "GraphTensor", "tensor", "add_op", "FlashAttentionOp", "DecodeAttentionOp", "flash_attention", "decode_attention",
-    "execute_op", "execute_op_inplace", "execute", "compile", "CompiledGraph", "HEADMAP_INTERLEAVED",
+    "RotaryEmbeddingOp", "KVAppendOp", "rotary_embedding", "kv_cache_append", "self_attention_core",
+    "cached_self_attention_core", "execute_op", "execute_op_inplace", "execute", "compile", "CompiledGraph", "HEADMAP_INTERLEAVED",
     "HEADMAP_BLOCKED", "LuminalHipError", "apply_rotary_embeddings", "kv_append", "KVCacheState", "encode", "decode", "f32_to_bf16_bits", "bf16_bits_to_f32", "default_scale",
 ]

@@ -57,13 +57,16 @@ get_device() = functional() ? HIPDevice(0) : Luminal.get_device()
 mutable struct HipArray{T,N}
     ptr::Ptr{Cvoid}
     dims::NTuple{N,Int}      # logical Luminal dims, e.g. (B,H,S,D)
+    parent::Any              # nothing for an owning array; the owner for a reshaped view
     function HipArray{T,N}(dims::NTuple{N,Int}) where {T,N}
         p = Ref{Ptr{Cvoid}}(C_NULL)
         check(ccall((:lmh_malloc, libluminal_hip), Cint, (Ptr{Ptr{Cvoid}}, Csize_t), p, max(prod(dims), 1) * sizeof(T)))
-        a = new{T,N}(p[], dims)
+        a = new{T,N}(p[], dims, nothing)
         finalizer(x -> ccall((:lmh_free, libluminal_hip), Cint, (Ptr{Cvoid},), x.ptr), a)
         return a
     end
+    # same memory under other dims (Base.reshape); frees nothing and keeps the owner reachable
+    HipArray{T,N}(ptr::Ptr{Cvoid}, dims::NTuple{N,Int}, owner) where {T,N} = new{T,N}(ptr, dims, owner)
 end
 Base.size(a::HipArray) = a.dims
 Base.size(a::HipArray, i::Integer) = a.dims[i]
@@ -190,9 +193,11 @@ struct RopeParams
 end
 
 "In-place rotary embedding of a (B,H,S,D) device array; same pairing as apply_rotary_embeddings (src/NN.jl:253-303)."
-function rope!(x::HipArray{T,4}; prev_seq::Integer=0, base::Real=10000.0f0) where {T}
+function rope!(x::HipArray{T,4}; prev_seq::Integer=0, base::Real=10000.0f0,
+               pos0::Union{Nothing,HipArray{Int32,1}}=nothing) where {T}
     B, H, S, D = size(x)
-    p = Ref(RopeParams(x.ptr, x.ptr, C_NULL, prev_seq, B, H, S, D, Z3, Z3, dtype_code(T), Float32(base), Int32(0), C_NULL))
+    p = Ref(RopeParams(x.ptr, x.ptr, pos0 === nothing ? Ptr{Int32}(C_NULL) : Ptr{Int32}(pos0.ptr), prev_seq, B, H, S, D,
+                       Z3, Z3, dtype_code(T), Float32(base), Int32(0), C_NULL))
     check(ccall((:lmh_rope, libluminal_hip), Cint, (Ref{RopeParams},), p))
     return x
 end
@@ -215,6 +220,43 @@ function kv_append!(kc::HipArray{T,4}, vc::HipArray{T,4}, k_new::HipArray{T,4}, 
     return kc, vc
 end
 
-export HIPDevice, HipArray, DecodeAttentionOp, decode_attention, get_device, functional, rope!, kv_append!
+# ------------------------------------------------------------------------------------------
+# What the attention layers do between their projections, as fused calls on device arrays.
+# SelfAttention (src/NN.jl:352-382) = rotary embedding of Q and K, repeat_kv, scaled causal softmax
+# attention; the fused op reads the Hkv key/value heads directly in the head order repeat_kv produces
+# (src/NN.jl:305-317). Whisper's layers (src/Whisper.jl:263-272, :310-312) are the same call without
+# rotary embedding, cross attention with causal=false.
+# ------------------------------------------------------------------------------------------
+function self_attention_core!(out::HipArray, q::HipArray{T,4}, k::HipArray{T,4}, v::HipArray{T,4}; causal::Bool=true,
+                              prev_seq::Integer=0, rope_base=nothing, scale=nothing,
+                              head_map::Int32=HEADMAP_INTERLEAVED) where {T}
+    if rope_base !== nothing
+        rope!(q; prev_seq=prev_seq, base=rope_base)
+        rope!(k; prev_seq=prev_seq, base=rope_base)
+    end
+    s = isnothing(scale) ? 1.0f0 / sqrt(Float32(size(q, 4))) : Float32(scale)
+    return execute_op!(out, FlashAttentionOp(s, causal), q, k, v; head_map=head_map)
+end
+
+"""
+One decode step of a cached attention layer (src/Whisper.jl:584-620): q (B,Hq,1,D) and k_new, v_new
+(B,Hkv,1,D) are this step's projections, `pos` (B,) the cache row each sequence writes, `kv_len` = pos .+ 1
+the rows it then attends over. Both are device arrays, so nothing is recompiled per position
+(the reference builds one graph per position, src/Decoding.jl:98-106).
+"""
+function cached_self_attention_core!(out::HipArray{TO,3}, q::HipArray{T,4}, k_new::HipArray{T,4}, v_new::HipArray{T,4},
+                                     kc::HipArray{T,4}, vc::HipArray{T,4}, pos::HipArray{Int32,1},
+                                     kv_len::HipArray{Int32,1}; rope_base=nothing, scale=nothing,
+                                     head_map::Int32=HEADMAP_INTERLEAVED) where {TO,T}
+    size(q, 3) == 1 || error("cached attention takes one query token per sequence")
+    rope_base !== nothing && rope!(q; pos0=pos, base=rope_base)
+    kv_append!(kc, vc, k_new, v_new, pos; rope_k=(rope_base !== nothing), base=something(rope_base, 10000.0f0))
+    s = isnothing(scale) ? 1.0f0 / sqrt(Float32(size(q, 4))) : Float32(scale)
+    q3 = HipArray{T,3}(q.ptr, (size(q, 1), size(q, 2), size(q, 4)), q)   # same memory, (B,Hq,D); keeps q alive
+    return execute_op!(out, DecodeAttentionOp(s, head_map), q3, kc, vc, kv_len)
+end
+
+export HIPDevice, HipArray, DecodeAttentionOp, decode_attention, get_device, functional, rope!, kv_append!,
+       self_attention_core!, cached_self_attention_core!
 
 end # module

@@ -67,3 +67,39 @@ def test_execute_needs_values_for_inputs(lm):
     out = lm.flash_attention(q, q, q)
     with pytest.raises(KeyError):
         lm.execute(g, out.id, {}, lm.CPUDevice())
+
+
+def test_cached_attention_core_emits_three_fused_nodes(lm):
+    # rotary on q, in-place append (K rotated on the way in), fused cached attention; positions are tensors
+    B, Hq, Hkv, D, Lmax = 2, 8, 2, 64, 32
+    g = lm.Graph()
+    q, kn, vn = lm.tensor(g, (B, Hq, 1, D)), lm.tensor(g, (B, Hkv, 1, D)), lm.tensor(g, (B, Hkv, 1, D))
+    kc, vc = lm.tensor(g, (B, Hkv, Lmax, D)), lm.tensor(g, (B, Hkv, Lmax, D))
+    pos, kv_len = lm.tensor(g, (B,), "i32"), lm.tensor(g, (B,), "i32")
+    n_inputs = len(g.nodes)
+    out, kc2, vc2 = lm.cached_self_attention_core(q, kn, vn, kc, vc, pos, kv_len, rope_base=10000.0)
+    ops = [type(n.op).__name__ for n in g.nodes[n_inputs:]]
+    assert ops == ["RotaryEmbeddingOp", "KVAppendOp", "DecodeAttentionOp"]
+    rot, app, att = g.nodes[n_inputs:]
+    assert [i[0] for i in rot.inputs] == [q.id, pos.id]
+    assert app.op.rope_k is True and [i[0] for i in app.inputs] == [kc.id, vc.id, kn.id, vn.id, pos.id]
+    # attention reads outputs 0 and 1 of the append node (the caches after the update) and q as (B, Hq, D)
+    assert [(i[0], i[1]) for i in att.inputs] == [(n_inputs, 0), (kc2.id, 0), (vc2.id, 1), (kv_len.id, 0)]
+    assert att.inputs[0][2] == (B, Hq, D) and out.shape == (B, Hq, D)
+    assert kc2.id == vc2.id and (kc2.index, vc2.index) == (0, 1)
+    with pytest.raises(ValueError):
+        lm.cached_self_attention_core(lm.tensor(g, (B, Hq, 2, D)), kn, vn, kc, vc, pos, kv_len)
+
+
+def test_self_attention_core_without_rope_is_one_flash_node(lm):
+    # Whisper's layers: no rotary embedding; cross attention is the same node with causal=False
+    g = lm.Graph()
+    q, k, v = lm.tensor(g, (4, 20, 448, 64), "f16"), lm.tensor(g, (4, 20, 1500, 64), "f16"), lm.tensor(g, (4, 20, 1500, 64), "f16")
+    n = len(g.nodes)
+    out = lm.self_attention_core(q, k, v, causal=False)
+    assert len(g.nodes) == n + 1 and isinstance(g.nodes[out.id].op, lm.FlashAttentionOp)
+    assert g.nodes[out.id].op.causal is False and out.shape == q.shape
+    out2 = lm.self_attention_core(q, k, v, causal=True, prev_seq=3, rope_base=10000.0)
+    kinds = [type(x.op).__name__ for x in g.nodes[n + 1:]]
+    assert kinds == ["RotaryEmbeddingOp", "RotaryEmbeddingOp", "FlashAttentionOp"]
+    assert g.nodes[n + 1].op.prev_seq == 3 and g.nodes[out2.id].op.causal is True

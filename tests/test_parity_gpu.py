@@ -396,3 +396,45 @@ def test_calibration_kernels(lm, hip):
     assert np.all(got == 64 * 16 * 6)
     with pytest.raises(lm.LuminalHipError):
         lm.binding.calib_mfma(sink.ptr, ones.ptr, 24, 1)
+
+
+def test_compiled_decode_step_graph_serves_every_position(lm, hip, oracle):
+    """One compiled graph — rotary embedding of q, in-place cache append with K rotated on the way in, fused
+    cached attention — is built once and stepped through all positions with `pos` / `kv_len` as device tensors
+    (the reference compiles one graph per position, src/Decoding.jl:98-106). Every step must equal the matching
+    row of causal attention over the rotated sequence (reference src/NN.jl:352-382 as a whole)."""
+    B, Hq, Hkv, S, D, Lmax = 2, 8, 2, 24, 64, 32
+    q, k, v = inputs(oracle, (B, Hq, S, D), (B, Hkv, S, D), "f32", 9400)
+    want = oracle.flash_attn(oracle.rope(q), oracle.rope(k), v, causal=True)
+    g = lm.Graph()
+    tq, tkn, tvn = lm.tensor(g, (B, Hq, 1, D)), lm.tensor(g, (B, Hkv, 1, D)), lm.tensor(g, (B, Hkv, 1, D))
+    tkc, tvc = lm.tensor(g, (B, Hkv, Lmax, D)), lm.tensor(g, (B, Hkv, Lmax, D))
+    tpos, tlen = lm.tensor(g, (B,), "i32"), lm.tensor(g, (B,), "i32")
+    out, kc2, vc2 = lm.cached_self_attention_core(tq, tkn, tvn, tkc, tvc, tpos, tlen, rope_base=10000.0)
+    cg = lm.compile(g, hip)
+    n_steps_built = len(cg.steps)
+    for t in range(S):
+        res = cg({tq.id: np.ascontiguousarray(q[:, :, t:t + 1]), tkn.id: np.ascontiguousarray(k[:, :, t:t + 1]),
+                  tvn.id: np.ascontiguousarray(v[:, :, t:t + 1]), tpos.id: np.full(B, t, np.int32),
+                  tlen.id: np.full(B, t + 1, np.int32)})
+        got = res[out.id].to_host()
+        assert rel_err(got, want[:, :, t]) <= 2e-5, t
+    assert len(cg.steps) == n_steps_built == 3  # rotary, append, attention: nothing was rebuilt per position
+    # the cache the graph holds is the rotated K and the raw V of all steps
+    kc_host = res[kc2.id][0].to_host()
+    assert rel_err(kc_host[:, :, :S], oracle.rope(k)) <= 2e-5
+    assert np.array_equal(res[kc2.id][1].to_host()[:, :, :S], v)
+
+
+@pytest.mark.parametrize("dtype", ["f32", "f16"])
+def test_self_attention_core_is_rope_plus_gqa_flash(lm, hip, oracle, dtype):
+    """Prefill form of the attention layer core: rotary nodes on Q and K, then one flash node reading the Hkv heads
+    directly; equals the oracle's rope followed by GQA attention in the head order repeat_kv produces."""
+    B, Hq, Hkv, S, D = 1, 8, 2, 96, 64
+    q, k, v = inputs(oracle, (B, Hq, S, D), (B, Hkv, S, D), dtype, 9500)
+    want = oracle.flash_attn(oracle.round_to(oracle.rope(q, prev_seq=5), dtype), oracle.round_to(oracle.rope(k, prev_seq=5), dtype), v, causal=True)
+    g = lm.Graph()
+    tq, tk, tv = lm.tensor(g, q.shape, dtype), lm.tensor(g, k.shape, dtype), lm.tensor(g, v.shape, dtype)
+    out = lm.self_attention_core(tq, tk, tv, causal=True, prev_seq=5, rope_base=10000.0, out_dtype=out_type(dtype, None))
+    got = lm.execute(g, out.id, {tq.id: q, tk.id: k, tv.id: v}, hip)
+    assert rel_err(got, want) <= (2e-5 if dtype == "f32" else 3e-3)
