@@ -30,6 +30,7 @@ import numpy as np
 ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
+PEAK_FP32_TFLOPS = 157.3  # dense fp32 MFMA
 PEAK_FP16_TFLOPS = 2500.0  # MI355X dense fp16/bf16 MFMA
 PEAK_HBM_GBS = 8000.0      # MI355X HBM3E
 # HBM-side bytes per launch of the two headline workloads, from rocprofv3 --pmc FETCH_SIZE and
@@ -262,6 +263,10 @@ def other_configs(lm, dev):
         log("[other] %s: %.1f us, %.2f TFLOP/s" % (name, ev * 1e3, res[name]["TFLOP/s"]))
 
     flash("C1 causal fp32 B=1 H=8 S=128 D=64", 1, 8, 8, 128, 128, 64, "f32", True, 4.0 * 8 * 64 * 128 * 129 / 2)
+    # the reference's element type on the C2 shape (not a BASELINE config): fp32 matrix-core kernel
+    flash("C2 shape in fp32 (causal B=1 H=32 S=4096 D=96)", 1, 32, 32, 4096, 4096, 96, "f32", True, 4.0 * 32 * 96 * 4096 * 4097 / 2)
+    res["C2 shape in fp32 (causal B=1 H=32 S=4096 D=96)"]["frac_of_fp32_mfma_peak"] = \
+        res["C2 shape in fp32 (causal B=1 H=32 S=4096 D=96)"]["TFLOP/s"] / PEAK_FP32_TFLOPS
     flash("C3 cross fp16 B=4 H=20 Sq=448 Sk=1500 D=64", 4, 20, 20, 448, 1500, 64, "f16", False, 4.0 * 4 * 20 * 448 * 1500 * 64)
 
     # C4: B=16 L=4096 decode; 268 MB would sit in the 256 MB last-level cache, so rotate over 4 caches
@@ -305,7 +310,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--only", choices=["all", "prefill", "decode", "copy"], default="all")
+    ap.add_argument("--only", choices=["all", "prefill", "decode", "other", "copy"], default="all")
     ap.add_argument("--decode-splits", type=int, default=0, help="KV splits for the decode leg (0 = library heuristic)")
     ap.add_argument("--cpu-seconds", type=float, default=15.0, help="CPU-baseline budget per leg; 0 disables it")
     args = ap.parse_args()
@@ -341,7 +346,7 @@ def main():
             line["cpu_baseline_single_thread"] = r["cpu_baseline_single_thread"]
     if args.only in ("all", "decode"):
         line["decode"] = decode_leg(lm, dev, args.steps, args.warmup, args.cpu_seconds, args.decode_splits)
-    if args.only == "all":
+    if args.only in ("all", "other"):
         line["other_configs"] = other_configs(lm, dev)
     print(json.dumps(line))
 

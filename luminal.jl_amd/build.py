@@ -12,7 +12,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIBDIR = os.path.join(HERE, "lib")
 LIBNAME = "libluminal_hip.so"
-SOURCES = ["api.hip", "prefill_valu.hip", "prefill_mfma.hip", "decode.hip", "decode_mfma.hip", "cache_ops.hip", "calib.hip"]
+SOURCES = ["api.hip", "prefill_valu.hip", "prefill_mfma.hip", "prefill_f32.hip", "decode.hip", "decode_mfma.hip", "cache_ops.hip", "calib.hip"]
 
 # -packed-fp32-ops: keep the compiler from forming v_pk_{add,mul,fma}_f32 out of scalar fp32 code.
 HIPCC_FLAGS = [

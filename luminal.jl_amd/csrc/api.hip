@@ -205,13 +205,15 @@ int lmh_flash_attn_fwd(const lmh_attn_params *p) {
   if (a.qs[2] < p->D || a.os[2] < p->D || a.ks[2] < p->D || a.vs[2] < p->D)
     return fail(LMH_E_SHAPE, "lmh_flash_attn_fwd: row stride smaller than head dim (rows overlap)");
 
-  // The matrix-core kernel does 128-bit accesses and tracks the max on raw scores (needs scale>0).
-  bool mfma_ok = prefill_mfma_supported(p->dtype, p->D) && p->scale > 0.f && aligned16(p->q) && aligned16(p->k) &&
-                 aligned16(p->v) && aligned16(p->out);
-  // its K/V tiles are fetched with 32-bit buffer offsets inside one (b, kv head) slice
-  mfma_ok = mfma_ok && (int64_t)p->Sk * a.ks[2] * 2 < (int64_t(1) << 31) && (int64_t)p->Sk * a.vs[2] * 2 < (int64_t(1) << 31);
+  // The matrix-core kernels do 128-bit accesses, track the max on raw scores (needs scale > 0) and fetch
+  // K/V tiles with 32-bit buffer offsets inside one (b, kv head) slice.
+  const int64_t esz = (int64_t)elem_bytes(p->dtype), vec = 16 / esz;
+  bool mfma_ok = (prefill_mfma_supported(p->dtype, p->D) || prefill_f32_mfma_supported(p->dtype, p->D)) && p->scale > 0.f &&
+                 aligned16(p->q) && aligned16(p->k) && aligned16(p->v) && aligned16(p->out);
+  mfma_ok = mfma_ok && (int64_t)p->Sk * a.ks[2] * esz < (int64_t(1) << 31) && (int64_t)p->Sk * a.vs[2] * esz < (int64_t(1) << 31);
   for (int i = 0; i < 3 && mfma_ok; i++)
-    mfma_ok = (a.qs[i] % 8 == 0) && (a.ks[i] % 8 == 0) && (a.vs[i] % 8 == 0) && (a.os[i] % 8 == 0);
+    mfma_ok = (a.qs[i] % vec == 0) && (a.ks[i] % vec == 0) && (a.vs[i] % vec == 0) && (a.os[i] % vec == 0);
+  if (mfma_ok && p->dtype == LMH_F32) return launch_prefill_f32_mfma(a, (hipStream_t)p->stream);
   if (mfma_ok) return launch_prefill_mfma(a, p->dtype, (hipStream_t)p->stream);
   return launch_prefill_valu(a, p->dtype, (hipStream_t)p->stream);
 }

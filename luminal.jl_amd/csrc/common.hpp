@@ -90,6 +90,8 @@ __host__ __device__ inline int q_head_of(int kvh, int g, int Hq, int Hkv, int he
 // Return LMH_OK or LMH_E_UNSUPPORTED / LMH_E_HIP.
 bool prefill_mfma_supported(int dtype, int D);
 int launch_prefill_mfma(const PrefillArgs &a, int dtype, hipStream_t stream);
+bool prefill_f32_mfma_supported(int dtype, int D);
+int launch_prefill_f32_mfma(const PrefillArgs &a, hipStream_t stream);
 int launch_prefill_valu(const PrefillArgs &a, int dtype, hipStream_t stream);
 int launch_decode(const DecodeArgs &a, int dtype, hipStream_t stream);
 int launch_rope(const RopeArgs &a, int dtype, hipStream_t stream);

@@ -1,0 +1,247 @@
+// Flash attention forward in fp32 on the gfx950 matrix cores (v_mfma_f32_32x32x2_f32).
+//
+// fp32 is the reference's only element type (flash_attn_cpu, reference src/Execution.jl:453-479), and its
+// parity budget (1e-5 of the output range) rules out half-precision operands, so this kernel keeps Q, K,
+// V and P in fp32 end to end; only the order of the fp32 additions differs from the reference's loop.
+//
+// Same structure as prefill_mfma.hip: a workgroup of 4 waves owns 128 query rows of one (b, hq), a wave
+// 32 of them with its Q fragments in registers; scores are computed transposed, S^T = K Q^T, so a lane
+// holds one query column and the softmax statistics are per-lane scalars; the accumulator registers that
+// hold P are directly the B operands of O^T = V^T P^T (no conversion, no LDS round trip). Differences:
+//   * the MFMA contracts 2 elements at a time (lane half g supplies one of them), so a 128-bit K fragment
+//     read feeds four MFMAs: the head dim is contracted in the order d = 8j + 4g + e, the same in Q and K;
+//   * the contraction over keys in the second product follows the accumulator layout: MFMA i of a 32-key
+//     tile pairs key 8(i/4) + (i%4) from lanes 0-31 with key 8(i/4) + 4 + (i%4) from lanes 32-63, and the
+//     V^T fragment is one 32-bit LDS read of those two rows;
+//   * tiles are 32 keys (fp32 tiles are twice as large in LDS) and exp2 runs on v_exp_f32 with the scale
+//     folded into the argument, as in the half-precision kernel.
+// The matrix pipe does 64 flops per cycle per SIMD in fp32 (157 TFLOP/s peak), 16 times less than in
+// fp16, so the ~70 vector instructions and ~80 LDS reads per tile hide behind 64-128 MFMAs of 64 cycles.
+#include "common.hpp"
+#include "dtypes.hpp"
+
+namespace lmh {
+namespace {
+
+constexpr int BM = 128;  // query rows per workgroup
+constexpr int BN = 32;   // keys per tile
+constexpr int kPadK = 4;  // floats: a row stride of D + 4 puts 16 consecutive rows' 16-byte reads on distinct banks
+constexpr int kPadV = 8;  // floats: rows key and key + 4 (the two halves of a wave) land 32 banks apart
+constexpr float kLog2e = 1.4426950408889634f;
+constexpr float kLazyRescale = 8.0f;  // see prefill_mfma.hip: the running max is raised only when outgrown by 2^8
+typedef float floatx4_t __attribute__((ext_vector_type(4)));
+
+template <int D, bool CAUSAL>
+__global__ __launch_bounds__(256, 2) void prefill_f32_kernel(PrefillArgs a, int n_q_tiles, int n_bh_groups) {
+  constexpr int KJ = D / 8;         // 128-bit K fragments per tile (4 MFMAs each)
+  constexpr int DB = D / 32;        // 32-row blocks of O^T
+  constexpr int CPR = D / 4;        // 16-byte chunks per K/V row
+  constexpr int CH = BN * CPR / 256;  // chunks per thread per tile
+  constexpr int LDK = D + kPadK;    // LDS row strides in floats
+  constexpr int LDV = D + kPadV;
+
+  __shared__ __attribute__((aligned(16))) float Ks2[2][BN * LDK];  // double-buffered tiles
+  __shared__ __attribute__((aligned(16))) float Vs2[2][BN * LDV];
+
+  // ---- which (b, hq, query tile) this workgroup owns: see prefill_mfma.hip ----
+  const int bid = blockIdx.x;
+  const int xcd = bid & 7;
+  const int idx = bid >> 3;
+  const int tile_rank = idx / n_bh_groups;
+  const int bh = (idx % n_bh_groups) * 8 + xcd;
+  if (bh >= a.B * a.Hq) return;
+  const int b = bh / a.Hq, hq = bh % a.Hq;
+  const int kvh = kv_head_of(hq, a.Hq, a.Hkv, a.head_map);
+  const int q_tile = CAUSAL ? (n_q_tiles - 1 - tile_rank) : tile_rank;
+  const int q0 = q_tile * BM;
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63, wave = tid >> 6;
+  const int n = lane & 31, g = lane >> 5;
+  const int wave_q_lo = q0 + wave * 32;
+  const int wave_q_hi = wave_q_lo + 31;
+  const int qi = wave_q_lo + n;
+
+  int n_keys = a.kv_len ? a.kv_len[b] : a.Sk;
+  n_keys = min(max(n_keys, 0), a.Sk);
+  int k_end = n_keys;
+  if (CAUSAL) k_end = min(k_end, q0 + BM);
+  const int n_kv_tiles = (k_end + BN - 1) / BN;
+
+  const float *qp = reinterpret_cast<const float *>(a.q) + b * a.qs[0] + hq * a.qs[1];
+  const float *kp = reinterpret_cast<const float *>(a.k) + b * a.ks[0] + kvh * a.ks[1];
+  const float *vp = reinterpret_cast<const float *>(a.v) + b * a.vs[0] + kvh * a.vs[1];
+
+  // ---- Q fragments: lane (n, g) holds q[qi][8j + 4g .. + 3] for every j ----
+  floatx4_t qf[KJ];
+#pragma unroll
+  for (int j = 0; j < KJ; j++) {
+    float4 raw = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (qi < a.Sq) raw = *reinterpret_cast<const float4 *>(qp + (int64_t)qi * a.qs[2] + 8 * j + 4 * g);
+    qf[j] = (floatx4_t){raw.x, raw.y, raw.z, raw.w};
+  }
+
+  floatx16_t oacc[DB];
+#pragma unroll
+  for (int db = 0; db < DB; db++)
+#pragma unroll
+    for (int i = 0; i < 16; i++) oacc[db][i] = 0.f;
+  float m_i = -INFINITY;  // running max of the raw (unscaled) scores of query qi
+  float l_i = 0.f;        // this lane's half of the running sum
+  const float c = a.scale * kLog2e;
+
+  // ---- tile staging: global -> registers (prefetched two tiles ahead) -> LDS; rows past n_keys read as
+  // zero through the buffer descriptor's bounds ----
+  const __amdgpu_buffer_rsrc_t k_rsrc =
+      __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(kp), 0, (int)((int64_t)n_keys * a.ks[2] * 4), 0x00020000);
+  const __amdgpu_buffer_rsrc_t v_rsrc =
+      __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(vp), 0, (int)((int64_t)n_keys * a.vs[2] * 4), 0x00020000);
+  int k_voff[CH], v_voff[CH], k_lds_off[CH], v_lds_off[CH];
+#pragma unroll
+  for (int r = 0; r < CH; r++) {
+    const int id = tid + 256 * r;
+    const int row = id / CPR, col = id % CPR;
+    k_voff[r] = (int)((row * a.ks[2] + col * 4) * 4);
+    v_voff[r] = (int)((row * a.vs[2] + col * 4) * 4);
+    k_lds_off[r] = row * LDK + col * 4;
+    v_lds_off[r] = row * LDV + col * 4;
+  }
+  const int k_tile_bytes = (int)(BN * a.ks[2] * 4), v_tile_bytes = (int)(BN * a.vs[2] * 4);
+  typedef unsigned int u32x4_t __attribute__((ext_vector_type(4)));
+  u32x4_t kreg[CH], vreg[CH];
+  auto load_tile = [&](int kt) {
+#pragma unroll
+    for (int r = 0; r < CH; r++) {
+      kreg[r] = __builtin_amdgcn_raw_buffer_load_b128(k_rsrc, k_voff[r], kt * k_tile_bytes, 0);
+      vreg[r] = __builtin_amdgcn_raw_buffer_load_b128(v_rsrc, v_voff[r], kt * v_tile_bytes, 0);
+    }
+  };
+  auto store_tile = [&](int buf) {
+#pragma unroll
+    for (int r = 0; r < CH; r++) {
+      *reinterpret_cast<u32x4_t *>(&Ks2[buf][k_lds_off[r]]) = kreg[r];
+      *reinterpret_cast<u32x4_t *>(&Vs2[buf][v_lds_off[r]]) = vreg[r];
+    }
+  };
+
+  const int k_frag_off = n * LDK + 4 * g;  // + 8 * j
+  const int v_frag_off = 4 * g * LDV + n;  // + (8 * (i / 4) + i % 4) * LDV + 32 * db
+
+  if (n_kv_tiles > 0) {
+    load_tile(0);
+    store_tile(0);
+  }
+  if (n_kv_tiles > 1) load_tile(1);
+
+  for (int kt = 0; kt < n_kv_tiles; kt++) {
+    // One barrier per tile: tile kt (written one iteration ago) becomes visible, and every wave is
+    // done with tile kt-1, whose buffer now takes tile kt+1 from the registers.
+    __syncthreads();
+    if (kt + 1 < n_kv_tiles) store_tile((kt + 1) & 1);
+    if (kt + 2 < n_kv_tiles) load_tile(kt + 2);
+    const float *Ks = Ks2[kt & 1];
+    const float *Vs = Vs2[kt & 1];
+
+    const int k0 = kt * BN;
+    if (CAUSAL && k0 > wave_q_hi) continue;  // whole tile above this wave's diagonal
+
+    // ---- S^T = K Q^T: 32 keys x 32 queries, contraction over the head dim two elements per MFMA ----
+    floatx16_t sacc;
+#pragma unroll
+    for (int i = 0; i < 16; i++) sacc[i] = 0.f;
+#pragma unroll
+    for (int j = 0; j < KJ; j++) {
+      const floatx4_t kf = *reinterpret_cast<const floatx4_t *>(&Ks[k_frag_off + 8 * j]);
+#pragma unroll
+      for (int e = 0; e < 4; e++) sacc = __builtin_amdgcn_mfma_f32_32x32x2f32(kf[e], qf[j][e], sacc, 0, 0, 0);
+    }
+
+    // ---- masking (diagonal tiles and the ragged last tile only) ----
+    const bool need_mask = (k0 + BN > n_keys) || (CAUSAL && k0 + BN - 1 > wave_q_lo);
+    if (need_mask) {
+#pragma unroll
+      for (int i = 0; i < 16; i++) {
+        const int key = k0 + 8 * (i >> 2) + 4 * g + (i & 3);
+        if (key >= n_keys || (CAUSAL && key > qi)) sacc[i] = -INFINITY;
+      }
+    }
+
+    // ---- online softmax; all statistics are per lane (one query column) ----
+    float mx = sacc[0];
+#pragma unroll
+    for (int i = 1; i < 16; i++) mx = fmaxf(mx, sacc[i]);
+    mx = fmaxf(mx, __shfl_xor(mx, 32));
+    // m_i is finite after the first tile (key 0 is visible to every query); -inf before it.
+    if (__builtin_amdgcn_ballot_w64((mx - m_i) * c > kLazyRescale) != 0) {  // wave-uniform
+      const float m_new = fmaxf(m_i, mx);
+      const float alpha = __builtin_amdgcn_exp2f((m_i - m_new) * c);
+      m_i = m_new;
+      l_i *= alpha;
+#pragma unroll
+      for (int db = 0; db < DB; db++)
+#pragma unroll
+        for (int i = 0; i < 16; i++) oacc[db][i] *= alpha;
+    }
+    const float mc = m_i * c;
+    float l0 = 0.f, l1 = 0.f;
+#pragma unroll
+    for (int i = 0; i < 16; i += 2) {
+      sacc[i] = __builtin_amdgcn_exp2f(sacc[i] * c - mc);
+      sacc[i + 1] = __builtin_amdgcn_exp2f(sacc[i + 1] * c - mc);
+      l0 += sacc[i];
+      l1 += sacc[i + 1];
+    }
+    l_i += l0 + l1;
+
+    // ---- O^T += V^T P^T: MFMA i contracts the two keys lanes (., 0) and (., 1) hold in register i ----
+#pragma unroll
+    for (int i = 0; i < 16; i++) {
+      const float *vrow = &Vs[v_frag_off + (8 * (i >> 2) + (i & 3)) * LDV];
+#pragma unroll
+      for (int db = 0; db < DB; db++) oacc[db] = __builtin_amdgcn_mfma_f32_32x32x2f32(vrow[32 * db], sacc[i], oacc[db], 0, 0, 0);
+    }
+  }
+
+  // ---- epilogue: out[qi][d] = O^T[d][qi] / l ----
+  const float l_tot = l_i + __shfl_xor(l_i, 32);
+  const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
+  if (qi < a.Sq) {
+    float *op = reinterpret_cast<float *>(a.out) + b * a.os[0] + hq * a.os[1] + (int64_t)qi * a.os[2];
+#pragma unroll
+    for (int db = 0; db < DB; db++)
+#pragma unroll
+      for (int i4 = 0; i4 < 4; i4++) {
+        const int d = db * 32 + 8 * i4 + 4 * g;
+        *reinterpret_cast<float4 *>(op + d) = make_float4(oacc[db][4 * i4 + 0] * inv, oacc[db][4 * i4 + 1] * inv,
+                                                          oacc[db][4 * i4 + 2] * inv, oacc[db][4 * i4 + 3] * inv);
+      }
+  }
+}
+
+template <int D>
+int launch_for_d(const PrefillArgs &a, hipStream_t stream) {
+  const int n_q_tiles = (a.Sq + BM - 1) / BM;
+  const int n_bh_groups = (a.B * a.Hq + 7) / 8;
+  dim3 grid(8 * n_bh_groups * n_q_tiles), block(256);
+  if (a.causal)
+    hipLaunchKernelGGL((prefill_f32_kernel<D, true>), grid, block, 0, stream, a, n_q_tiles, n_bh_groups);
+  else
+    hipLaunchKernelGGL((prefill_f32_kernel<D, false>), grid, block, 0, stream, a, n_q_tiles, n_bh_groups);
+  LMH_HIP_TRY(hipGetLastError());
+  return LMH_OK;
+}
+
+}  // namespace
+
+bool prefill_f32_mfma_supported(int dtype, int D) { return dtype == LMH_F32 && (D == 64 || D == 96 || D == 128); }
+
+int launch_prefill_f32_mfma(const PrefillArgs &a, hipStream_t stream) {
+  switch (a.D) {
+    case 64: return launch_for_d<64>(a, stream);
+    case 96: return launch_for_d<96>(a, stream);
+    case 128: return launch_for_d<128>(a, stream);
+  }
+  return fail(LMH_E_UNSUPPORTED, "fp32 MFMA flash attention: head dim %d not tiled", a.D);
+}
+
+}  // namespace lmh

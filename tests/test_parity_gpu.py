@@ -177,6 +177,27 @@ def test_mfma_shapes(lm, hip, oracle, dtype, D, causal, Sq, Sk):
     assert rel_err(got, oracle.flash_attn(q, k, v, causal=causal, nthreads=NT)) <= 2e-3
 
 
+@pytest.mark.parametrize("D", [64, 96, 128])
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("Sq,Sk", [(1, 1), (1, 200), (31, 33), (64, 64), (127, 127), (128, 128), (129, 129), (300, 1000), (1000, 300), (513, 513)])
+def test_fp32_mfma_shapes(lm, hip, oracle, D, causal, Sq, Sk):
+    # the fp32 matrix-core kernel (head dims 64 / 96 / 128) at the fp32 budget
+    q, k, v = inputs(oracle, (2, 3, Sq, D), (2, 3, Sk, D), "f32", 7300 + Sq + D)
+    got = run_flash(lm, hip, q, k, v, "f32", causal)
+    assert rel_err(got, oracle.flash_attn(q, k, v, causal=causal, nthreads=NT)) <= 1e-5
+
+
+def test_fp32_large_logits_and_late_maximum(lm, hip, oracle):
+    # scores far apart (scale 1, |q.k| up to ~60) and a maximum that arrives in the last tile exercise the
+    # lazily raised running max of the fp32 kernel; the oracle follows the reference's exact recurrence
+    B, H, S, D = 1, 2, 200, 64
+    q, k, v = inputs(oracle, (B, H, S, D), (B, H, S, D), "f32", 7400)
+    k[:, :, -1] *= 6.0
+    for causal in (False, True):
+        got = run_flash(lm, hip, q, k, v, "f32", causal, scale=1.0)
+        assert rel_err(got, oracle.flash_attn(q, k, v, scale=1.0, causal=causal)) <= 1e-5
+
+
 @pytest.mark.parametrize("dtype", ["f32", "f16", "bf16"])
 @pytest.mark.parametrize("head_map", [0, 1])
 def test_gqa_prefill_both_head_maps(lm, hip, oracle, dtype, head_map):
