@@ -101,7 +101,7 @@ typedef struct lmh_attn_params {
   const void *q;      /* [B,Hq,Sq,D] device */
   const void *k;      /* [B,Hkv,Sk,D] device */
   const void *v;      /* [B,Hkv,Sk,D] device */
-  const int32_t *kv_len; /* optional device int32[B]: valid keys per sequence (1..Sk); null = Sk */
+  const int32_t *kv_len; /* optional device int32[B]: valid keys per sequence (0..Sk; 0 writes zeros); null = Sk */
   int32_t B, Hq, Hkv, Sq, Sk, D;
   int64_t q_stride[3]; /* element strides for (b, h, s); all-zero = contiguous */
   int64_t k_stride[3];

@@ -326,7 +326,7 @@ __global__ __launch_bounds__(kMergeThreads) void decode_merge_kernel(DecodeArgs 
   lsum = 0.f;
 #pragma unroll
   for (int w = 0; w < kMergeThreads / 64; w++) lsum += red_l[w];
-  const float inv = 1.f / lsum;
+  const float inv = lsum > 0.f ? 1.f / lsum : 0.f;
 
   const float *po = a.ws_o + row0 * a.D;
   for (int d = tid; d < a.D; d += kMergeThreads) {

@@ -117,7 +117,7 @@ __global__ __launch_bounds__(256) void prefill_valu_kernel(PrefillArgs a) {
     const int64_t off = b * a.os[0] + hq * a.os[1] + (int64_t)qi * a.os[2];
     raw *op = reinterpret_cast<raw *>(a.out) + off;
     float *op32 = reinterpret_cast<float *>(a.out) + off;
-    float inv = 1.f / l_i;
+    float inv = l_i > 0.f ? 1.f / l_i : 0.f;  // a row with no visible key (kv_len[b] == 0) is written as zeros
 #pragma unroll
     for (int c = 0; c < NCH; c++) {
       float tmp[4] = {of[c].x, of[c].y, of[c].z, of[c].w};

@@ -220,6 +220,19 @@ def test_prefill_ragged_kv_len_with_poisoned_tail(lm, hip, oracle, dtype):
     assert rel_err(got, oracle.flash_attn(q, k, v, kv_len=lens)) <= TOL[dtype]
 
 
+@pytest.mark.parametrize("dtype,D", [("f32", 64), ("f16", 64), ("bf16", 96), ("f16", 80), ("f32", 40)])
+def test_prefill_sequence_without_keys_is_written_as_zeros(lm, hip, oracle, dtype, D):
+    # kv_len[b] == 0 does not occur in the reference (its 0/0 would be NaN); every kernel writes zeros for it
+    B, H, Sq, Sk = 3, 2, 70, 130
+    q, k, v = inputs(oracle, (B, H, Sq, D), (B, H, Sk, D), dtype, 7450)
+    lens = np.array([130, 0, 5], np.int32)
+    got = run_flash(lm, hip, q, k, v, dtype, False, kv_len=lens)
+    want = oracle.flash_attn(q, k, v, kv_len=np.array([130, 1, 5], np.int32))
+    assert np.all(got[1] == 0)
+    keep = [0, 2]
+    assert rel_err(got[keep], want[keep]) <= TOL[dtype]
+
+
 @pytest.mark.parametrize("dtype", ["f16", "bf16"])
 def test_unusual_head_dim_and_scale_take_the_vector_path(lm, hip, oracle, dtype):
     q, k, v = inputs(oracle, (1, 2, 90, 80), (1, 2, 90, 80), dtype, 7500)
