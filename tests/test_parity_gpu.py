@@ -472,3 +472,16 @@ def test_self_attention_core_is_rope_plus_gqa_flash(lm, hip, oracle, dtype):
     out = lm.self_attention_core(tq, tk, tv, causal=True, prev_seq=5, rope_base=10000.0, out_dtype=out_type(dtype, None))
     got = lm.execute(g, out.id, {tq.id: q, tk.id: k, tv.id: v}, hip)
     assert rel_err(got, want) <= (2e-5 if dtype == "f32" else 3e-3)
+
+
+def test_decode_batch_above_the_persistent_kernel_limit(lm, hip, oracle):
+    # more than 1024 sequences: the matrix-core decode kernel keeps its per-sequence prefix sums in LDS and hands
+    # larger batches to the vector kernel; same results expected, ragged lengths included
+    B, Hq, Hkv, L, D = 1100, 4, 2, 96, 64
+    q, k, v = inputs(oracle, (B, Hq, D), (B, Hkv, L, D), "bf16", 9600)
+    lens = oracle.gen_uniform_int(B, 9601, 1, L).astype(np.int32)
+    got = run_decode(lm, hip, q, k, v, "bf16", kv_len=lens)
+    assert rel_err(got, oracle.decode_attn(q, k, v, kv_len=lens, nthreads=NT)) <= 2e-3
+    # and exactly at the limit the persistent kernel still runs
+    got = run_decode(lm, hip, q[:1024], k[:1024], v[:1024], "bf16", kv_len=lens[:1024], num_splits=2)
+    assert rel_err(got, oracle.decode_attn(q[:1024], k[:1024], v[:1024], kv_len=lens[:1024], nthreads=NT)) <= 2e-3
