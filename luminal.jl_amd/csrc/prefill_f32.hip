@@ -32,7 +32,7 @@ constexpr float kLazyRescale = 8.0f;  // see prefill_mfma.hip: the running max i
 typedef float floatx4_t __attribute__((ext_vector_type(4)));
 
 template <int D, bool CAUSAL>
-__global__ __launch_bounds__(256, 2) void prefill_f32_kernel(PrefillArgs a, int n_q_tiles, int n_bh_groups) {
+__global__ __launch_bounds__(256, (D <= 96 ? 3 : 2)) void prefill_f32_kernel(PrefillArgs a, int n_q_tiles, int n_bh_groups) {
   constexpr int KJ = D / 8;         // 128-bit K fragments per tile (4 MFMAs each)
   constexpr int DB = D / 32;        // 32-row blocks of O^T
   constexpr int CPR = D / 4;        // 16-byte chunks per K/V row
