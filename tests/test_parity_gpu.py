@@ -485,3 +485,64 @@ def test_decode_batch_above_the_persistent_kernel_limit(lm, hip, oracle):
     # and exactly at the limit the persistent kernel still runs
     got = run_decode(lm, hip, q[:1024], k[:1024], v[:1024], "bf16", kv_len=lens[:1024], num_splits=2)
     assert rel_err(got, oracle.decode_attn(q[:1024], k[:1024], v[:1024], kv_len=lens[:1024], nthreads=NT)) <= 2e-3
+
+
+def _padded(lm, hip, x, dtype, row_pad, rng):
+    """Upload x (B,H,S,D) into a buffer whose rows are D + row_pad apart (padding filled with NaN);
+    returns (array, element strides (b, h, s))."""
+    B, H, S, D = x.shape
+    buf = np.full((B, H, S, D + row_pad), np.nan, np.float32)
+    buf[..., :D] = x
+    return lm.to_device(buf, hip, dtype), (H * S * (D + row_pad), S * (D + row_pad), D + row_pad)
+
+
+@pytest.mark.parametrize("seed", range(24))
+def test_prefill_random_shapes_strides_and_options(lm, hip, oracle, seed):
+    """Seeded sweep over what the entry point dispatches on: element type, head dim (matrix-core and vector kernels),
+    GQA group and head map, causal, ragged kv_len, row strides (16-byte aligned and not), fp32 output of half inputs."""
+    rng = np.random.default_rng(9700 + seed)
+    dtype = ["f32", "f16", "bf16"][seed % 3]
+    D = int(rng.choice([16, 32, 40, 64, 80, 96, 128]))
+    Hkv = int(rng.integers(1, 4)); G = int(rng.choice([1, 2, 4])); Hq = Hkv * G
+    B = int(rng.integers(1, 4))
+    Sq, Sk = int(rng.integers(1, 260)), int(rng.integers(1, 330))
+    causal = bool(rng.integers(0, 2)); head_map = int(rng.integers(0, 2))
+    pad_q, pad_kv = int(rng.choice([0, 8, 3])), int(rng.choice([0, 8, 16, 5]))
+    q, k, v = inputs(oracle, (B, Hq, Sq, D), (B, Hkv, Sk, D), dtype, 9800 + seed)
+    lens = rng.integers(1, Sk + 1, size=B).astype(np.int32) if rng.integers(0, 2) else None
+    dq, qs = _padded(lm, hip, q, dtype, pad_q, rng)
+    dk, ks = _padded(lm, hip, k, dtype, pad_kv, rng)
+    dv, vs = _padded(lm, hip, v, dtype, pad_kv, rng)
+    odt = "f32" if dtype == "bf16" or rng.integers(0, 2) else dtype
+    out = lm.HipArray((B, Hq, Sq, D), odt, hip)
+    dl = None if lens is None else lm.to_device(lens, hip)
+    p = lm.binding.AttnParams()
+    p.out, p.q, p.k, p.v = out.ptr, dq.ptr, dk.ptr, dv.ptr
+    p.kv_len = dl.ptr if dl is not None else None
+    p.B, p.Hq, p.Hkv, p.Sq, p.Sk, p.D = B, Hq, Hkv, Sq, Sk, D
+    for arr, st in ((p.q_stride, qs), (p.k_stride, ks), (p.v_stride, vs)):
+        arr[0], arr[1], arr[2] = st
+    p.dtype, p.scale, p.causal, p.head_map = lm.binding.DTYPE_CODES[dtype], lm.default_scale(D), int(causal), head_map
+    p.out_f32 = int(odt == "f32")
+    lm.binding.flash_attn_fwd(p)
+    want = oracle.flash_attn(q, k, v, causal=causal, head_map=head_map, kv_len=lens, nthreads=NT)
+    case = dict(dtype=dtype, D=D, B=B, Hq=Hq, Hkv=Hkv, Sq=Sq, Sk=Sk, causal=causal, head_map=head_map, pad_q=pad_q, pad_kv=pad_kv,
+                lens=None if lens is None else lens.tolist(), out=odt)
+    tol = TOL[dtype] if odt == "f32" or dtype == "f32" else 3e-3  # a half-precision result adds its own rounding
+    assert rel_err(out.to_host(), want) <= tol, case
+
+
+@pytest.mark.parametrize("seed", range(12))
+def test_decode_random_shapes_and_options(lm, hip, oracle, seed):
+    rng = np.random.default_rng(9900 + seed)
+    dtype = ["f32", "f16", "bf16"][seed % 3]
+    D = int(rng.choice([32, 64, 96, 128, 256] if dtype != "f32" else [32, 64, 128]))
+    Hkv = int(rng.integers(1, 5)); G = int(rng.choice([1, 2, 4, 8])); Hq = Hkv * G
+    B = int(rng.integers(1, 6)); L = int(rng.integers(1, 700))
+    head_map = int(rng.integers(0, 2)); splits = int(rng.choice([0, 1, 2, 5]))
+    q, k, v = inputs(oracle, (B, Hq, D), (B, Hkv, L, D), dtype, 9950 + seed)
+    lens = rng.integers(1, L + 1, size=B).astype(np.int32) if rng.integers(0, 2) else None
+    got = run_decode(lm, hip, q, k, v, dtype, kv_len=lens, head_map=head_map, num_splits=splits)
+    want = oracle.decode_attn(q, k, v, kv_len=lens, head_map=head_map, nthreads=NT)
+    assert rel_err(got, want) <= TOL[dtype], dict(dtype=dtype, D=D, B=B, Hq=Hq, Hkv=Hkv, L=L, head_map=head_map, splits=splits,
+                                                   lens=None if lens is None else lens.tolist())
