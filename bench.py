@@ -263,7 +263,7 @@ def other_configs(lm, dev):
         log("[other] %s: %.1f us, %.2f TFLOP/s" % (name, ev * 1e3, res[name]["TFLOP/s"]))
 
     flash("C1 causal fp32 B=1 H=8 S=128 D=64", 1, 8, 8, 128, 128, 64, "f32", True, 4.0 * 8 * 64 * 128 * 129 / 2)
-    # the reference's element type on the C2 shape (not a BASELINE config): fp32 matrix-core kernel
+    # the reference's element type on the C2 shape (an extra line, not one of the five configurations): fp32 matrix-core kernel
     flash("C2 shape in fp32 (causal B=1 H=32 S=4096 D=96)", 1, 32, 32, 4096, 4096, 96, "f32", True, 4.0 * 32 * 96 * 4096 * 4097 / 2)
     res["C2 shape in fp32 (causal B=1 H=32 S=4096 D=96)"]["frac_of_fp32_mfma_peak"] = \
         res["C2 shape in fp32 (causal B=1 H=32 S=4096 D=96)"]["TFLOP/s"] / PEAK_FP32_TFLOPS
