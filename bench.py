@@ -62,6 +62,18 @@ def time_steps(fn, steps, warmup, binding):
     return (t1 - t0) * 1e3 / steps, e1.elapsed_ms_since(e0) / steps
 
 
+def per_launch_us(fn, n, binding):
+    """Median and minimum of n launches timed one by one with HIP events (after the main timed region)."""
+    evs = [(binding.Event(), binding.Event()) for _ in range(n)]
+    for a, b in evs:
+        a.record()
+        fn()
+        b.record()
+    binding.sync()
+    us = sorted(b.elapsed_ms_since(a) * 1e3 for a, b in evs)
+    return {"median": us[len(us) // 2], "min": us[0], "n": n}
+
+
 def attn_params(lm, out, q, k, v, dtype, causal, scale, head_map=0, kv_len=None):
     p = lm.binding.AttnParams()
     p.out, p.q, p.k, p.v = out.ptr, q.ptr, k.ptr, v.ptr
@@ -109,13 +121,14 @@ def prefill_leg(lm, dev, steps, warmup, cpu_seconds):
     kern_tflops = flops / (ev_ms * 1e-3) / 1e12
     log("[prefill] C2 causal fp16 B=1 H=32 S=4096 D=96: %.1f us/step wall, %.1f us/launch events, %.1f TFLOP/s (%.1f%% of %g)"
         % (wall_ms * 1e3, ev_ms * 1e3, kern_tflops, 100 * kern_tflops / PEAK_FP16_TFLOPS, PEAK_FP16_TFLOPS))
+    each = per_launch_us(fn, 20, lm.binding)
     sustained = mfma_sustained(lm, dev, dq)
     res = {
         "ms_per_step": wall_ms, "value": tflops,
         "roofline": {"bound": "mfma", "achieved": kern_tflops, "peak": PEAK_FP16_TFLOPS, "unit": "TFLOP/s",
                      "frac": kern_tflops / PEAK_FP16_TFLOPS, "traffic": PREFILL_TRAFFIC_BYTES,
                      "kernel": "prefill_mfma_kernel<MfmaF16, 96, causal>", "launch_us": ev_ms * 1e3,
-                     "algorithmic_flops_per_launch": flops,
+                     "algorithmic_flops_per_launch": flops, "launch_us_one_by_one": each,
                      # what a bare MFMA loop sustains on this GPU right now (clock management under load):
                      # on all-zero operands and on the Q tensor of this workload
                      "mfma_sustained_tflops": sustained,
@@ -215,7 +228,8 @@ def decode_leg(lm, dev, steps, warmup, cpu_seconds, num_splits=0):
         "roofline": {"bound": "hbm", "achieved": kern_gbs, "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": kern_gbs / PEAK_HBM_GBS,
                      "traffic": DECODE_TRAFFIC_BYTES if num_splits == 0 else None,
                      "kernel": "decode_mfma_kernel<Mfma16BF16,128> + decode_merge_kernel",
-                     "launch_us": ev_ms * 1e3, "algorithmic_bytes_per_launch": algo_bytes},
+                     "launch_us": ev_ms * 1e3, "algorithmic_bytes_per_launch": algo_bytes,
+                     "launch_us_one_by_one": per_launch_us(fn, 20, lm.binding)},
     }
     if cpu_seconds > 0:
         import oracle
