@@ -210,7 +210,9 @@ int lmh_flash_attn_fwd(const lmh_attn_params *p) {
   const int64_t esz = (int64_t)elem_bytes(p->dtype), vec = 16 / esz;
   bool mfma_ok = (prefill_mfma_supported(p->dtype, p->D) || prefill_f32_mfma_supported(p->dtype, p->D)) && p->scale > 0.f &&
                  aligned16(p->q) && aligned16(p->k) && aligned16(p->v) && aligned16(p->out);
-  mfma_ok = mfma_ok && (int64_t)p->Sk * a.ks[2] * esz < (int64_t(1) << 31) && (int64_t)p->Sk * a.vs[2] * esz < (int64_t(1) << 31);
+  // (offsets from 0x7ffffff0 up are what the half-precision kernel uses as "out of range")
+  constexpr int64_t kMaxSliceBytes = 0x7ffffff0;
+  mfma_ok = mfma_ok && (int64_t)p->Sk * a.ks[2] * esz < kMaxSliceBytes && (int64_t)p->Sk * a.vs[2] * esz < kMaxSliceBytes;
   for (int i = 0; i < 3 && mfma_ok; i++)
     mfma_ok = (a.qs[i] % vec == 0) && (a.ks[i] % vec == 0) && (a.vs[i] % vec == 0) && (a.os[i] % vec == 0);
   if (mfma_ok && p->dtype == LMH_F32) return launch_prefill_f32_mfma(a, (hipStream_t)p->stream);

@@ -14,9 +14,11 @@
 //   * the same registers, converted to half precision, are directly the B operand of the second
 //     product O^T = V^T P^T (M = head dim, N = queries, contraction over keys), so P never
 //     touches LDS;
-//   * K and V tiles (64 keys) are staged row-major in LDS; the K fragment is a plain 128-bit LDS
-//     read (contraction over the contiguous head dim), the V^T fragment uses the gfx950 transposing
-//     LDS read ds_read_b64_tr_b16, which hands each lane 4 consecutive keys of its head-dim column;
+//   * K and V tiles (64 keys) go from global memory straight into double-buffered LDS, row-major,
+//     with LDS-writing buffer loads (no register staging, no LDS store instructions); the K
+//     fragment is a plain 128-bit LDS read (contraction over the contiguous head dim), the V^T
+//     fragment uses the gfx950 transposing LDS read ds_read_b64_tr_b16, which hands each lane 4
+//     consecutive keys of its head-dim column;
 //   * causal: key tiles beyond the workgroup's last query are never loaded, a wave skips tiles that
 //     lie entirely above its diagonal, and only diagonal tiles pay for masking;
 //   * blockIdx -> work mapping keeps all query tiles of a head on one XCD (private L2) and, for
@@ -31,18 +33,21 @@ constexpr int BM = 128;  // query rows per workgroup
 constexpr int BN = 64;   // keys per tile
 // LDS row paddings in elements. K rows are read 16 bytes per lane, one row per lane: a stride of
 // D + 8 elements spreads 16 consecutive rows over all banks (5 cycles per 1 KB fragment per CU,
-// against 16 unpadded). V rows go through the transposing read (4 rows x 32 bytes per 16 lanes),
-// which is conflict-free when the stride is 96 elements modulo 128 (5.6 cycles per fragment, against
-// 8 at D + 8 and 16 at a multiple of 128 bytes): no padding for D = 96, +32 for D = 64 and 128.
+// against 16 unpadded). V rows go through the transposing read (4 rows x 32 bytes per 16 lanes); in
+// a microbenchmark its cost depends on the stride (5.6 cycles per fragment at 96 elements modulo
+// 128, 8 at D + 8, 16 at a multiple of 128 bytes), in the kernel D = 64 measures the same with 0, 8,
+// 16 or 32 elements of padding, and 0 lets a fourth workgroup fit on a CU.
 constexpr int kPadK = 8;
-template <int D> constexpr int pad_v() { return D == 96 ? 0 : 32; }
+template <int D> constexpr int pad_v() { return D == 128 ? 32 : 0; }
 constexpr float kLog2e = 1.4426950408889634f;
 // The running max is only raised (and the output rescaled) when a row's scores outgrow it by more
 // than this many powers of two; until then P is computed against the stale max and may reach
 // 2^kLazyRescale, which fp16/bf16/fp32 all hold. The quotient O / l does not depend on the reference
 // max, so the result is unchanged while most tiles skip the D-wide rescale.
 constexpr float kLazyRescale = 8.0f;
-typedef unsigned int u32x4_t __attribute__((ext_vector_type(4)));
+// Byte offset no K/V slice reaches (the host routes larger ones elsewhere): a buffer load there
+// is out of range and returns zeros.
+constexpr int kOutOfRange = 0x7ffffff0;
 
 typedef short shortx8_t __attribute__((ext_vector_type(8)));
 typedef __attribute__((address_space(3))) shortx4_t lds_shortx4_t;
@@ -93,7 +98,6 @@ __global__ __launch_bounds__(256, (D <= 96 ? 3 : 2)) void prefill_mfma_kernel(Pr
   constexpr int KS = D / 16;       // k-steps of the S^T product
   constexpr int DB = D / 32;       // 32-row blocks of O^T
   constexpr int CPR = D / 8;       // 16-byte chunks per K/V row
-  constexpr int CH = BN * CPR / 256;  // chunks per thread per tile
   constexpr int LDK = D + kPadK;   // LDS row strides in elements
   constexpr int LDV = D + pad_v<D>();
 
@@ -150,39 +154,66 @@ __global__ __launch_bounds__(256, (D <= 96 ? 3 : 2)) void prefill_mfma_kernel(Pr
   float l_i = 0.f;        // this lane's half of the running sum
   const float c = a.scale * kLog2e;
 
-  // ---- tile staging: global -> registers (prefetched two tiles ahead) -> LDS ----
-  // Buffer loads: the descriptor's size is the end of the last valid key row, so rows past n_keys
-  // read as zero without a branch, and the per-lane byte offsets are loop invariants — a tile costs
-  // one scalar offset update instead of per-lane 64-bit address arithmetic.
-  const __amdgpu_buffer_rsrc_t k_rsrc =
-      __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t *>(kp), 0, (int)((int64_t)n_keys * a.ks[2] * 2), 0x00020000);
-  const __amdgpu_buffer_rsrc_t v_rsrc =
-      __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t *>(vp), 0, (int)((int64_t)n_keys * a.vs[2] * 2), 0x00020000);
-  int k_voff[CH], v_voff[CH], k_lds_off[CH], v_lds_off[CH];
+  // ---- tile staging: global memory -> LDS directly (buffer_load_dwordx4 ... lds), one tile ahead ----
+  // A tile of 64 rows x LD elements is LD / 8 blocks of 1 KB. One wave-wide load fills one block:
+  // lane l's 16 bytes land at block + 16 l, fetched from that lane's own global offset, so the
+  // padded row layout needs no register staging and no LDS store instructions. Lanes that fall on
+  // a padding chunk fetch out of range. The descriptor's size is the end of the last valid key row:
+  // rows past n_keys arrive as zeros without a branch, and the per-lane offsets are loop
+  // invariants. Wave w issues blocks w, w + 4, ...
+  // The load is written in asm because the compiler, when it knows of an LDS-writing load in
+  // flight, waits for it before the next LDS read of the same array — which would serialise the
+  // prefetch of tile kt + 1 with the fragment reads of tile kt. The wait that matters (this wave's
+  // loads have landed, then the workgroup barrier) is written out at the top of the loop.
+  typedef int32_t i32x4_t __attribute__((ext_vector_type(4)));
+  typedef __attribute__((address_space(3))) void lds_void_t;
+  constexpr int KI = LDK / 8, VI = LDV / 8;            // 1 KB blocks per tile
+  constexpr int KJ = (KI + 3) / 4, VJ = (VI + 3) / 4;  // blocks per wave (rounded up)
+  const int wave_u = __builtin_amdgcn_readfirstlane(wave);
+  __builtin_assume(wave_u >= 0 && wave_u < 4);
+  auto make_desc = [](const uint16_t *base, int bytes) {
+    const uint64_t p = (uint64_t)base;
+    i32x4_t d;
+    d[0] = __builtin_amdgcn_readfirstlane((int)(uint32_t)p);
+    d[1] = __builtin_amdgcn_readfirstlane((int)((p >> 32) & 0xffff));  // stride 0: raw buffer
+    d[2] = __builtin_amdgcn_readfirstlane(bytes);
+    d[3] = 0x00020000;
+    return d;
+  };
+  const i32x4_t k_desc = make_desc(kp, (int)((int64_t)n_keys * a.ks[2] * 2));
+  const i32x4_t v_desc = make_desc(vp, (int)((int64_t)n_keys * a.vs[2] * 2));
+  int k_voff[KJ], v_voff[VJ];
 #pragma unroll
-  for (int r = 0; r < CH; r++) {
-    const int id = tid + 256 * r;
-    const int row = id / CPR, col = id % CPR;
-    k_voff[r] = (int)((row * a.ks[2] + col * 8) * 2);
-    v_voff[r] = (int)((row * a.vs[2] + col * 8) * 2);
-    k_lds_off[r] = row * LDK + col * 8;
-    v_lds_off[r] = row * LDV + col * 8;
+  for (int j = 0; j < KJ; j++) {
+    const int ch = (wave + 4 * j) * 64 + lane;
+    const int row = ch / KI, col = ch % KI;
+    k_voff[j] = col < CPR ? (int)((row * a.ks[2] + col * 8) * 2) : kOutOfRange;
+  }
+#pragma unroll
+  for (int j = 0; j < VJ; j++) {
+    const int ch = (wave + 4 * j) * 64 + lane;
+    const int row = ch / VI, col = ch % VI;
+    v_voff[j] = col < CPR ? (int)((row * a.vs[2] + col * 8) * 2) : kOutOfRange;
   }
   const int k_tile_bytes = (int)(BN * a.ks[2] * 2), v_tile_bytes = (int)(BN * a.vs[2] * 2);
-  u32x4_t kreg[CH], vreg[CH];
-  auto load_tile = [&](int kt) {
-#pragma unroll
-    for (int r = 0; r < CH; r++) {
-      kreg[r] = __builtin_amdgcn_raw_buffer_load_b128(k_rsrc, k_voff[r], kt * k_tile_bytes, 0);
-      vreg[r] = __builtin_amdgcn_raw_buffer_load_b128(v_rsrc, v_voff[r], kt * v_tile_bytes, 0);
-    }
+  const uint32_t k_lds0 = (uint32_t)(uintptr_t)(lds_void_t *)&Ks2[0][0] + wave_u * 1024;
+  const uint32_t v_lds0 = (uint32_t)(uintptr_t)(lds_void_t *)&Vs2[0][0] + wave_u * 1024;
+#pragma clang diagnostic push
+#pragma clang diagnostic ignored "-Winline-asm"  // m0 is a reserved register; it is only written here
+  auto load_block = [](i32x4_t desc, uint32_t lds_addr, int voff, int soff) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
+                 :: "s"(lds_addr), "v"(voff), "s"(desc), "s"(soff) : "memory", "m0");
   };
-  auto store_tile = [&](int buf) {
+#pragma clang diagnostic pop
+  auto load_tile = [&](int kt, int buf) {
 #pragma unroll
-    for (int r = 0; r < CH; r++) {
-      *reinterpret_cast<u32x4_t *>(&Ks2[buf][k_lds_off[r]]) = kreg[r];
-      *reinterpret_cast<u32x4_t *>(&Vs2[buf][v_lds_off[r]]) = vreg[r];
-    }
+    for (int j = 0; j < KJ; j++)
+      if (wave_u + 4 * j < KI)
+        load_block(k_desc, k_lds0 + buf * (BN * LDK * 2) + j * 4096, k_voff[j], kt * k_tile_bytes);
+#pragma unroll
+    for (int j = 0; j < VJ; j++)
+      if (wave_u + 4 * j < VI)
+        load_block(v_desc, v_lds0 + buf * (BN * LDV * 2) + j * 4096, v_voff[j], kt * v_tile_bytes);
   };
 
   // lane-constant pieces of the LDS addresses
@@ -193,18 +224,19 @@ __global__ __launch_bounds__(256, (D <= 96 ? 3 : 2)) void prefill_mfma_kernel(Pr
   const int v_frag_off = (4 * g + (i16 >> 2)) * LDV + 16 * ((lane >> 4) & 1) + 4 * (i16 & 3);
   // + (kb*32 + 16*t [+8]) * LDV + db*32
 
-  if (n_kv_tiles > 0) {
-    load_tile(0);
-    store_tile(0);
-  }
-  if (n_kv_tiles > 1) load_tile(1);
+  if (n_kv_tiles > 0) load_tile(0, 0);
+  // The compiler does not model the asm loads or the asm wait below. Make it wait for Q here;
+  // otherwise it puts its own vmcnt(0) in front of the first MFMA inside the loop, after the
+  // prefetch of the next tile has been issued.
+#pragma unroll
+  for (int ks = 0; ks < KS; ks++) asm volatile("" :: "v"(qreg[ks]));
 
   for (int kt = 0; kt < n_kv_tiles; kt++) {
     // One barrier per tile: tile kt (written one iteration ago) becomes visible, and every wave is
     // done with tile kt-1, whose buffer now takes tile kt+1 from the registers.
-    __syncthreads();
-    if (kt + 1 < n_kv_tiles) store_tile((kt + 1) & 1);
-    if (kt + 2 < n_kv_tiles) load_tile(kt + 2);  // in flight while tiles kt and kt+1 are computed
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wave's blocks of tile kt are in LDS
+    __syncthreads();  // ... and everyone's; tile kt-1 has been consumed, its buffer is free
+    if (kt + 1 < n_kv_tiles) load_tile(kt + 1, (kt + 1) & 1);  // in flight while tile kt is computed
     const uint16_t *Ks = Ks2[kt & 1];
     const uint16_t *Vs = Vs2[kt & 1];
 
