@@ -29,8 +29,8 @@
 namespace lmh {
 namespace {
 
-constexpr int BM = 128;  // query rows per workgroup
-constexpr int BN = 64;   // keys per tile
+constexpr int BN = 64;   // keys a wave takes per tile
+constexpr int kNumCUs = 256;
 // LDS row paddings in elements. K rows are read 16 bytes per lane, one row per lane: a stride of
 // D + 8 elements spreads 16 consecutive rows over all banks (5 cycles per 1 KB fragment per CU,
 // against 16 unpadded). V rows go through the transposing read (4 rows x 32 bytes per 16 lanes); in
@@ -92,17 +92,27 @@ struct MfmaBF16 {
   }
 };
 
-template <typename MT, int D, bool CAUSAL>
+// KSPLIT = 1: the four waves own 4 x 32 query rows and walk the same 64-key tiles.
+// KSPLIT = 2: for launches too small to fill the chip. The workgroup owns 64 query rows; waves 0-1
+// take them against the first 32 keys of every tile, waves 2-3 against the second 32, each pair
+// with its own running max / sum / output, merged through LDS at the end. Twice the workgroups,
+// and a wave's share of a tile is half as long.
+template <typename MT, int D, bool CAUSAL, int KSPLIT>
 __global__ __launch_bounds__(256, (D <= 96 ? 3 : 2)) void prefill_mfma_kernel(PrefillArgs a, int n_q_tiles, int n_bh_groups) {
   using vec8 = typename MT::vec8;
+  constexpr int BM = 128 / KSPLIT;  // query rows per workgroup
+  constexpr int BT = BN;            // keys per staged tile
+  constexpr int RG = 4 / KSPLIT;    // waves (32-row groups) per key group
+  constexpr int NKB = 2 / KSPLIT;   // 32-key blocks a wave takes per tile
+  constexpr int BW = 32 * NKB;      // ... in keys
   constexpr int KS = D / 16;       // k-steps of the S^T product
   constexpr int DB = D / 32;       // 32-row blocks of O^T
   constexpr int CPR = D / 8;       // 16-byte chunks per K/V row
   constexpr int LDK = D + kPadK;   // LDS row strides in elements
   constexpr int LDV = D + pad_v<D>();
 
-  __shared__ __attribute__((aligned(16))) uint16_t Ks2[2][BN * LDK];  // double-buffered tiles
-  __shared__ __attribute__((aligned(16))) uint16_t Vs2[2][BN * LDV];
+  __shared__ __attribute__((aligned(16))) uint16_t Ks2[2][BT * LDK];  // double-buffered tiles
+  __shared__ __attribute__((aligned(16))) uint16_t Vs2[2][BT * LDV];
 
   // ---- which (b, hq, query tile) this workgroup owns ----
   const int bid = blockIdx.x;
@@ -122,7 +132,8 @@ __global__ __launch_bounds__(256, (D <= 96 ? 3 : 2)) void prefill_mfma_kernel(Pr
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = tid >> 6;
   const int n = lane & 31, g = lane >> 5;
-  const int wave_q_lo = q0 + wave * 32;
+  const int kg = wave / RG;  // key group of this wave (always 0 when KSPLIT == 1)
+  const int wave_q_lo = q0 + (wave % RG) * 32;
   const int wave_q_hi = wave_q_lo + 31;
   const int qi = wave_q_lo + n;
 
@@ -130,7 +141,7 @@ __global__ __launch_bounds__(256, (D <= 96 ? 3 : 2)) void prefill_mfma_kernel(Pr
   n_keys = min(max(n_keys, 0), a.Sk);
   int k_end = n_keys;
   if (CAUSAL) k_end = min(k_end, q0 + BM);
-  const int n_kv_tiles = (k_end + BN - 1) / BN;
+  const int n_kv_tiles = (k_end + BT - 1) / BT;
 
   const uint16_t *qp = reinterpret_cast<const uint16_t *>(a.q) + b * a.qs[0] + hq * a.qs[1];
   const uint16_t *kp = reinterpret_cast<const uint16_t *>(a.k) + b * a.ks[0] + kvh * a.ks[1];
@@ -155,7 +166,7 @@ __global__ __launch_bounds__(256, (D <= 96 ? 3 : 2)) void prefill_mfma_kernel(Pr
   const float c = a.scale * kLog2e;
 
   // ---- tile staging: global memory -> LDS directly (buffer_load_dwordx4 ... lds), one tile ahead ----
-  // A tile of 64 rows x LD elements is LD / 8 blocks of 1 KB. One wave-wide load fills one block:
+  // A tile of BT rows x LD elements is BT * LD / 512 blocks of 1 KB. One wave-wide load fills one block:
   // lane l's 16 bytes land at block + 16 l, fetched from that lane's own global offset, so the
   // padded row layout needs no register staging and no LDS store instructions. Lanes that fall on
   // a padding chunk fetch out of range. The descriptor's size is the end of the last valid key row:
@@ -167,7 +178,8 @@ __global__ __launch_bounds__(256, (D <= 96 ? 3 : 2)) void prefill_mfma_kernel(Pr
   // loads have landed, then the workgroup barrier) is written out at the top of the loop.
   typedef int32_t i32x4_t __attribute__((ext_vector_type(4)));
   typedef __attribute__((address_space(3))) void lds_void_t;
-  constexpr int KI = LDK / 8, VI = LDV / 8;            // 1 KB blocks per tile
+  constexpr int KC = LDK / 8, VC = LDV / 8;            // 16-byte chunks per LDS row
+  constexpr int KI = KC * BT / 64, VI = VC * BT / 64;  // 1 KB blocks per tile
   constexpr int KJ = (KI + 3) / 4, VJ = (VI + 3) / 4;  // blocks per wave (rounded up)
   const int wave_u = __builtin_amdgcn_readfirstlane(wave);
   __builtin_assume(wave_u >= 0 && wave_u < 4);
@@ -186,16 +198,16 @@ __global__ __launch_bounds__(256, (D <= 96 ? 3 : 2)) void prefill_mfma_kernel(Pr
 #pragma unroll
   for (int j = 0; j < KJ; j++) {
     const int ch = (wave + 4 * j) * 64 + lane;
-    const int row = ch / KI, col = ch % KI;
+    const int row = ch / KC, col = ch % KC;
     k_voff[j] = col < CPR ? (int)((row * a.ks[2] + col * 8) * 2) : kOutOfRange;
   }
 #pragma unroll
   for (int j = 0; j < VJ; j++) {
     const int ch = (wave + 4 * j) * 64 + lane;
-    const int row = ch / VI, col = ch % VI;
+    const int row = ch / VC, col = ch % VC;
     v_voff[j] = col < CPR ? (int)((row * a.vs[2] + col * 8) * 2) : kOutOfRange;
   }
-  const int k_tile_bytes = (int)(BN * a.ks[2] * 2), v_tile_bytes = (int)(BN * a.vs[2] * 2);
+  const int k_tile_bytes = (int)(BT * a.ks[2] * 2), v_tile_bytes = (int)(BT * a.vs[2] * 2);
   const uint32_t k_lds0 = (uint32_t)(uintptr_t)(lds_void_t *)&Ks2[0][0] + wave_u * 1024;
   const uint32_t v_lds0 = (uint32_t)(uintptr_t)(lds_void_t *)&Vs2[0][0] + wave_u * 1024;
 #pragma clang diagnostic push
@@ -209,11 +221,11 @@ __global__ __launch_bounds__(256, (D <= 96 ? 3 : 2)) void prefill_mfma_kernel(Pr
 #pragma unroll
     for (int j = 0; j < KJ; j++)
       if (wave_u + 4 * j < KI)
-        load_block(k_desc, k_lds0 + buf * (BN * LDK * 2) + j * 4096, k_voff[j], kt * k_tile_bytes);
+        load_block(k_desc, k_lds0 + buf * (BT * LDK * 2) + j * 4096, k_voff[j], kt * k_tile_bytes);
 #pragma unroll
     for (int j = 0; j < VJ; j++)
       if (wave_u + 4 * j < VI)
-        load_block(v_desc, v_lds0 + buf * (BN * LDV * 2) + j * 4096, v_voff[j], kt * v_tile_bytes);
+        load_block(v_desc, v_lds0 + buf * (BT * LDV * 2) + j * 4096, v_voff[j], kt * v_tile_bytes);
   };
 
   // lane-constant pieces of the LDS addresses
@@ -237,35 +249,36 @@ __global__ __launch_bounds__(256, (D <= 96 ? 3 : 2)) void prefill_mfma_kernel(Pr
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wave's blocks of tile kt are in LDS
     __syncthreads();  // ... and everyone's; tile kt-1 has been consumed, its buffer is free
     if (kt + 1 < n_kv_tiles) load_tile(kt + 1, (kt + 1) & 1);  // in flight while tile kt is computed
-    const uint16_t *Ks = Ks2[kt & 1];
-    const uint16_t *Vs = Vs2[kt & 1];
+    const uint16_t *Ks = Ks2[kt & 1] + kg * (BW * LDK);
+    const uint16_t *Vs = Vs2[kt & 1] + kg * (BW * LDV);
 
-    const int k0 = kt * BN;
-    if (CAUSAL && k0 > wave_q_hi) continue;  // whole tile above this wave's diagonal
+    const int k0 = kt * BT + kg * BW;         // first key of this wave's share of the tile
+    if (CAUSAL && k0 > wave_q_hi) continue;   // all of it above this wave's diagonal
+    if (KSPLIT > 1 && k0 >= k_end) continue;  // ... or past the last key (second half of the last tile)
 
-    // ---- S^T = K Q^T for two 32-key blocks: all fragments are fetched first, then the two
+    // ---- S^T = K Q^T for the wave's 32-key blocks: all fragments are fetched first, then the
     // accumulator chains alternate so that neither waits on LDS or on its own previous MFMA ----
-    vec8 kf[2][KS];
+    vec8 kf[NKB][KS];
 #pragma unroll
     for (int ks = 0; ks < KS; ks++)
 #pragma unroll
-      for (int kb = 0; kb < 2; kb++)
+      for (int kb = 0; kb < NKB; kb++)
         kf[kb][ks] = *reinterpret_cast<const vec8 *>(&Ks[k_frag_off + kb * 32 * LDK + 16 * ks]);
-    floatx16_t sacc[2];
+    floatx16_t sacc[NKB];
 #pragma unroll
-    for (int kb = 0; kb < 2; kb++)
+    for (int kb = 0; kb < NKB; kb++)
 #pragma unroll
       for (int i = 0; i < 16; i++) sacc[kb][i] = 0.f;
 #pragma unroll
     for (int ks = 0; ks < KS; ks++)
 #pragma unroll
-      for (int kb = 0; kb < 2; kb++) sacc[kb] = MT::mfma(kf[kb][ks], qreg[ks], sacc[kb]);
+      for (int kb = 0; kb < NKB; kb++) sacc[kb] = MT::mfma(kf[kb][ks], qreg[ks], sacc[kb]);
 
     // ---- masking (diagonal tiles and the ragged last tile only) ----
-    const bool need_mask = (k0 + BN > n_keys) || (CAUSAL && k0 + BN - 1 > wave_q_lo);
+    const bool need_mask = (k0 + BW > n_keys) || (CAUSAL && k0 + BW - 1 > wave_q_lo);
     if (need_mask) {
 #pragma unroll
-      for (int kb = 0; kb < 2; kb++)
+      for (int kb = 0; kb < NKB; kb++)
 #pragma unroll
         for (int i = 0; i < 16; i++) {
           const int key = k0 + kb * 32 + 8 * (i >> 2) + 4 * g + (i & 3);
@@ -276,7 +289,7 @@ __global__ __launch_bounds__(256, (D <= 96 ? 3 : 2)) void prefill_mfma_kernel(Pr
     // ---- online softmax; all statistics are per lane (one query column) ----
     float mx = sacc[0][0];
 #pragma unroll
-    for (int kb = 0; kb < 2; kb++)
+    for (int kb = 0; kb < NKB; kb++)
 #pragma unroll
       for (int i = 0; i < 16; i++) mx = fmaxf(mx, sacc[kb][i]);
     mx = fmaxf(mx, __shfl_xor(mx, 32));
@@ -292,9 +305,9 @@ __global__ __launch_bounds__(256, (D <= 96 ? 3 : 2)) void prefill_mfma_kernel(Pr
         for (int i = 0; i < 16; i++) oacc[db][i] *= alpha;
     }
     const float mc = m_i * c;
-    vec8 pf[2][2], pf_lo[2][2];
+    vec8 pf[NKB][2], pf_lo[NKB][2];
 #pragma unroll
-    for (int kb = 0; kb < 2; kb++)
+    for (int kb = 0; kb < NKB; kb++)
 #pragma unroll
       for (int t = 0; t < 2; t++) {
 #pragma unroll
@@ -309,7 +322,7 @@ __global__ __launch_bounds__(256, (D <= 96 ? 3 : 2)) void prefill_mfma_kernel(Pr
 
     // ---- O^T += V^T P^T ----
 #pragma unroll
-    for (int kb = 0; kb < 2; kb++) {
+    for (int kb = 0; kb < NKB; kb++) {
 #pragma unroll
       for (int t = 0; t < 2; t++) {
 #pragma unroll
@@ -323,6 +336,34 @@ __global__ __launch_bounds__(256, (D <= 96 ? 3 : 2)) void prefill_mfma_kernel(Pr
         }
       }
     }
+  }
+
+  // ---- key groups: fold group 1's (m, l, O) into group 0's; lane for lane the same layout ----
+  if (KSPLIT > 1) {
+    constexpr int NF = DB * 16 + 2;  // floats per lane
+    static_assert(KSPLIT == 1 || RG * NF * 64 * 4 <= (int)sizeof(Ks2), "merge buffer must fit in the K tiles");
+    float *xch = reinterpret_cast<float *>(&Ks2[0][0]) + (wave % RG) * (NF * 64) + lane;  // [NF][64 lanes]
+    __syncthreads();  // every wave has read its last tile
+    if (kg == 1) {
+      xch[0] = m_i;
+      xch[64] = l_i;
+#pragma unroll
+      for (int db = 0; db < DB; db++)
+#pragma unroll
+        for (int i = 0; i < 16; i++) xch[(2 + db * 16 + i) * 64] = oacc[db][i];
+    }
+    __syncthreads();
+    if (kg == 1) return;
+    const float m1 = xch[0], l1 = xch[64];
+    const float m_new = fmaxf(m_i, m1);
+    // a group that saw no key has m = -inf, l = 0, O = 0
+    const float a0 = m_i == -INFINITY ? 0.f : __builtin_amdgcn_exp2f((m_i - m_new) * c);
+    const float a1 = m1 == -INFINITY ? 0.f : __builtin_amdgcn_exp2f((m1 - m_new) * c);
+    l_i = l_i * a0 + l1 * a1;
+#pragma unroll
+    for (int db = 0; db < DB; db++)
+#pragma unroll
+      for (int i = 0; i < 16; i++) oacc[db][i] = oacc[db][i] * a0 + xch[(2 + db * 16 + i) * 64] * a1;
   }
 
   // ---- epilogue: out[qi][d] = O^T[d][qi] / l ----
@@ -353,17 +394,30 @@ __global__ __launch_bounds__(256, (D <= 96 ? 3 : 2)) void prefill_mfma_kernel(Pr
   }
 }
 
-template <typename MT, int D>
-int launch_for_d(const PrefillArgs &a, hipStream_t stream) {
-  const int n_q_tiles = (a.Sq + BM - 1) / BM;
+template <typename MT, int D, int KSPLIT>
+int launch_split(const PrefillArgs &a, hipStream_t stream) {
+  const int n_q_tiles = (a.Sq + 128 / KSPLIT - 1) / (128 / KSPLIT);
   const int n_bh_groups = (a.B * a.Hq + 7) / 8;
   dim3 grid(8 * n_bh_groups * n_q_tiles), block(256);
   if (a.causal)
-    hipLaunchKernelGGL((prefill_mfma_kernel<MT, D, true>), grid, block, 0, stream, a, n_q_tiles, n_bh_groups);
+    hipLaunchKernelGGL((prefill_mfma_kernel<MT, D, true, KSPLIT>), grid, block, 0, stream, a, n_q_tiles, n_bh_groups);
   else
-    hipLaunchKernelGGL((prefill_mfma_kernel<MT, D, false>), grid, block, 0, stream, a, n_q_tiles, n_bh_groups);
+    hipLaunchKernelGGL((prefill_mfma_kernel<MT, D, false, KSPLIT>), grid, block, 0, stream, a, n_q_tiles, n_bh_groups);
   LMH_HIP_TRY(hipGetLastError());
   return LMH_OK;
+}
+
+template <typename MT, int D>
+int launch_for_d(const PrefillArgs &a, hipStream_t stream) {
+  // With fewer than two 128-row workgroups per CU the launch is bound by how long one workgroup
+  // takes to walk its keys, not by the matrix pipes: split the keys of a tile between wave pairs.
+  // Measured on 256 CUs: at exactly two per CU the split still wins for causal launches (41.8 vs
+  // 46.7 us at B=1 H=32 S=2048 D=96) and loses for non-causal ones (79.8 vs 66.6 us); at three per
+  // CU it loses for both.
+  const int64_t wgs = (int64_t)((a.B * a.Hq + 7) / 8) * 8 * ((a.Sq + 127) / 128);
+  const int64_t limit = a.causal ? 2 * kNumCUs : 2 * kNumCUs - 1;
+  if (wgs <= limit && a.Sk >= 4 * BN) return launch_split<MT, D, 2>(a, stream);
+  return launch_split<MT, D, 1>(a, stream);
 }
 
 template <typename MT>

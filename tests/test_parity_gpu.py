@@ -234,6 +234,39 @@ def test_prefill_sequence_without_keys_is_written_as_zeros(lm, hip, oracle, dtyp
 
 
 @pytest.mark.parametrize("dtype", ["f16", "bf16"])
+@pytest.mark.parametrize("D", [64, 96, 128])
+@pytest.mark.parametrize("causal", [False, True])
+def test_prefill_small_launch_splits_keys_between_wave_pairs(lm, hip, oracle, dtype, D, causal):
+    # few workgroups and >= 256 keys: 64-row workgroups whose wave pairs take alternate 32-key blocks and are
+    # merged at the end. Lengths put the last key in the first block, the second block, on a block edge, and nowhere.
+    B, Hq, Hkv, Sq, Sk = 7, 4, 2, 150, 700
+    q, k, v = inputs(oracle, (B, Hq, Sq, D), (B, Hkv, Sk, D), dtype, 7470 + D)
+    lens = np.array([700, 20, 33, 64, 97, 0, 641], np.int32)
+    kp, vp = k.copy(), v.copy()
+    for b, n in enumerate(lens):
+        kp[b, :, n:] = np.nan
+        vp[b, :, n:] = np.nan
+    got = run_flash(lm, hip, q, kp, vp, dtype, causal, kv_len=lens)
+    want = oracle.flash_attn(q, k, v, causal=causal, kv_len=np.maximum(lens, 1), nthreads=NT)
+    assert np.all(got[5] == 0)
+    keep = [0, 1, 2, 3, 4, 6]
+    assert rel_err(got[keep], want[keep]) <= TOL[dtype]
+
+
+@pytest.mark.parametrize("causal", [False, True])
+def test_prefill_small_and_large_launches_agree(lm, hip, oracle, causal):
+    # the same two heads alone (key-split workgroups) and as part of a launch that fills the chip (128-row workgroups)
+    S, D = 512, 96
+    q, k, v = inputs(oracle, (1, 160, S, D), (1, 160, S, D), "f16", 7490, 0.5)
+    small = run_flash(lm, hip, q[:, :2], k[:, :2], v[:, :2], "f16", causal, out_dtype="f32")
+    large = run_flash(lm, hip, q, k, v, "f16", causal, out_dtype="f32")
+    want = oracle.flash_attn(q[:, :2], k[:, :2], v[:, :2], causal=causal, nthreads=NT)
+    assert rel_err(small, want) <= TOL["f16"]
+    assert rel_err(large[:, :2], want) <= TOL["f16"]
+    assert rel_err(small, large[:, :2]) <= TOL["f16"]
+
+
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
 def test_unusual_head_dim_and_scale_take_the_vector_path(lm, hip, oracle, dtype):
     q, k, v = inputs(oracle, (1, 2, 90, 80), (1, 2, 90, 80), dtype, 7500)
     assert rel_err(run_flash(lm, hip, q, k, v, dtype, True), oracle.flash_attn(q, k, v, causal=True)) <= 2e-3
