@@ -306,6 +306,33 @@ def other_configs(lm, dev):
     res["C4 decode bf16 B=16 Hq=32 Hkv=8 L=4096 D=128 (4 caches rotated)"] = {
         "launch_us": ev * 1e3, "GB/s": nbytes / (ev * 1e-3) / 1e9, "frac_of_hbm_peak": nbytes / (ev * 1e-3) / 1e9 / PEAK_HBM_GBS}
     log("[other] C4 decode: %.1f us, %.0f GB/s" % (ev * 1e3, nbytes / (ev * 1e-3) / 1e9))
+
+    # the two operators in front of attention: rotary embedding of a prompt's Q, and the cache append (K rotated on
+    # the way in) for a whole prompt and for one decode step. Algorithmic bytes = every element read once, written once.
+    def hbm_line(name, fn, nbytes, n=20):
+        _, ev = time_steps(fn, n, 5, lm.binding)
+        res[name] = {"launch_us": ev * 1e3, "GB/s": nbytes / (ev * 1e-3) / 1e9, "frac_of_hbm_peak": nbytes / (ev * 1e-3) / 1e9 / PEAK_HBM_GBS}
+        log("[other] %s: %.1f us, %.0f GB/s" % (name, ev * 1e3, res[name]["GB/s"]))
+
+    B, H, S, D = 1, 32, 4096, 96
+    x = lm.HipArray((B, H, S, D), "f16", dev).copy_from_host(rng.standard_normal((B, H, S, D), dtype=np.float32))
+    y = lm.HipArray((B, H, S, D), "f16", dev)
+    rp = lm.binding.RopeParams()
+    rp.out, rp.x, rp.pos0, rp.prev_seq = y.ptr, x.ptr, None, 0
+    rp.B, rp.H, rp.S, rp.D = B, H, S, D
+    rp.dtype, rp.base, rp.pairing, rp.stream = lm.binding.DTYPE_CODES["f16"], 10000.0, lm.binding.ROPE_HALF_SPLIT, None
+    hbm_line("rotary embedding fp16 B=1 H=32 S=4096 D=96 (C2's Q)", lambda: lm.binding.rope(rp), 2.0 * B * H * S * D * 2)
+
+    for T, label in ((4096, "whole prompt T=4096"), (1, "one decode step T=1")):
+        B, Hkv, L, D = 16, 8, 4096, 128
+        kc, vc = caches[0]
+        kn = lm.HipArray((B, Hkv, T, D), "bf16", dev).copy_from_host(rng.standard_normal((B, Hkv, T, D), dtype=np.float32))
+        vn = lm.HipArray((B, Hkv, T, D), "bf16", dev).copy_from_host(rng.standard_normal((B, Hkv, T, D), dtype=np.float32))
+        ap = lm.binding.KvAppendParams()
+        ap.k_cache, ap.v_cache, ap.k_new, ap.v_new, ap.pos, ap.pos_all = kc.ptr, vc.ptr, kn.ptr, vn.ptr, None, (0 if T > 1 else L - 1)
+        ap.B, ap.Hkv, ap.T, ap.D, ap.Lmax = B, Hkv, T, D, L
+        ap.dtype, ap.rope_k, ap.pairing, ap.base, ap.stream = lm.binding.DTYPE_CODES["bf16"], 1, lm.binding.ROPE_HALF_SPLIT, 10000.0, None
+        hbm_line("cache append + rotary K bf16 B=16 Hkv=8 D=128, %s" % label, lambda: lm.binding.kv_append(ap), 4.0 * B * Hkv * T * D * 2)
     return res
 
 

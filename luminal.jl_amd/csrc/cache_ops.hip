@@ -9,8 +9,12 @@
 //     are written in place at pos[b] .. pos[b]+T-1 (per-sequence positions, device int32[B]), with
 //     the rotary embedding of K optionally fused into the same pass.
 //
-// Both are a few bytes of traffic per element and purely HBM/latency-bound; one thread handles one
-// rotated pair (rope) or one 16-byte chunk (append).
+// Both are a few bytes of traffic per element and HBM-bound. The kernels that run for the usual head
+// dims move 16-byte chunks: a thread owns the chunk of pairs (j .. j+V-1) — chunk c of the first half
+// of the row and chunk c of the second half, or one chunk of interleaved pairs — and, for the
+// standalone rotary embedding, evaluates its sin / cos once and walks the heads with them (the angle
+// does not depend on the head). Rows whose head dim or alignment does not allow 16-byte chunks take
+// the one-element-per-thread kernels.
 #include "common.hpp"
 #include "dtypes.hpp"
 
@@ -82,6 +86,150 @@ __global__ __launch_bounds__(256) void kv_append_kernel(KvAppendArgs a) {
   }
 }
 
+// 16 bytes of a row, as raw elements
+template <typename E>
+union Chunk {
+  uint4 u;
+  typename E::raw e[E::kVec];
+};
+
+// x0[i], x1[i] -> rotated in place by (sn[i], cs[i]); same expressions as rope_pair
+template <typename E>
+__device__ inline void rotate_chunks(Chunk<E> &c0, Chunk<E> &c1, const float *sn, const float *cs) {
+#pragma unroll
+  for (int i = 0; i < E::kVec; i++) {
+    const float x0 = E::ld(c0.e[i]), x1 = E::ld(c1.e[i]);
+    c0.e[i] = E::st(x0 * cs[i] - x1 * sn[i]);
+    c1.e[i] = E::st(x0 * sn[i] + x1 * cs[i]);
+  }
+}
+template <typename E>
+__device__ inline void rotate_interleaved(Chunk<E> &c, const float *sn, const float *cs) {
+#pragma unroll
+  for (int i = 0; i < E::kVec / 2; i++) {
+    const float x0 = E::ld(c.e[2 * i]), x1 = E::ld(c.e[2 * i + 1]);
+    c.e[2 * i] = E::st(x0 * cs[i] - x1 * sn[i]);
+    c.e[2 * i + 1] = E::st(x0 * sn[i] + x1 * cs[i]);
+  }
+}
+template <typename E>
+__device__ inline void sincos_pairs(float pos, int j0, int n, int D, float log2_base, float *sn, float *cs) {
+#pragma unroll
+  for (int i = 0; i < E::kVec; i++) {
+    if (i >= n) break;
+    const float freq = (float)(j0 + i) * 2.0f / (float)D;
+    const float inv_freq = 1.0f / exp2f(freq * log2_base);
+    sincosf(pos * inv_freq, &sn[i], &cs[i]);
+  }
+}
+
+// Rotary embedding, 16-byte chunks. grid.x covers (b, s, chunk), grid.y blocks of heads.
+// IL = false: thread owns pairs j = c V .. c V + V - 1, i.e. chunk c of each half of the row.
+// IL = true : thread owns pairs j = c V/2 .. , i.e. chunk c of the row.
+template <typename E, bool IL>
+__global__ __launch_bounds__(256) void rope_vec_kernel(RopeArgs a, int heads_per_block) {
+  using raw = typename E::raw;
+  constexpr int V = E::kVec;
+  const int half = a.D / 2;
+  const int cpr = IL ? a.D / V : half / V;  // chunks (threads) per row
+  const int64_t total = (int64_t)a.B * a.S * cpr;
+  const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= total) return;
+  const int c = (int)(idx % cpr);
+  const int s = (int)((idx / cpr) % a.S);
+  const int b = (int)(idx / ((int64_t)cpr * a.S));
+  const float pos = (float)((a.pos0 ? a.pos0[b] : a.prev_seq) + s);
+  float sn[V], cs[V];
+  sincos_pairs<E>(pos, IL ? c * (V / 2) : c * V, IL ? V / 2 : V, a.D, a.log2_base, sn, cs);
+  const int h0 = blockIdx.y * heads_per_block, h1 = min(a.H, h0 + heads_per_block);
+  for (int h = h0; h < h1; h++) {
+    const raw *xp = reinterpret_cast<const raw *>(a.x) + b * a.xs[0] + h * a.xs[1] + (int64_t)s * a.xs[2];
+    raw *op = reinterpret_cast<raw *>(a.out) + b * a.os[0] + h * a.os[1] + (int64_t)s * a.os[2];
+    if (IL) {
+      Chunk<E> ch;
+      ch.u = *reinterpret_cast<const uint4 *>(xp + c * V);
+      rotate_interleaved<E>(ch, sn, cs);
+      *reinterpret_cast<uint4 *>(op + c * V) = ch.u;
+    } else {
+      Chunk<E> c0, c1;
+      c0.u = *reinterpret_cast<const uint4 *>(xp + c * V);
+      c1.u = *reinterpret_cast<const uint4 *>(xp + half + c * V);
+      rotate_chunks<E>(c0, c1, sn, cs);
+      *reinterpret_cast<uint4 *>(op + c * V) = c0.u;
+      *reinterpret_cast<uint4 *>(op + half + c * V) = c1.u;
+    }
+  }
+}
+
+// Cache append, 16-byte chunks: a thread moves chunk c of each half of one new K row and one new V row
+// (D is a multiple of 2 V), rotating K on the way when asked to.
+template <typename E>
+__global__ __launch_bounds__(256) void kv_append_vec_kernel(KvAppendArgs a) {
+  using raw = typename E::raw;
+  constexpr int V = E::kVec;
+  const int half = a.D / 2;
+  const int cpr = half / V;
+  const int64_t total = (int64_t)a.B * a.Hkv * a.T * cpr;
+  const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= total) return;
+  const int c = (int)(idx % cpr);
+  const int t = (int)((idx / cpr) % a.T);
+  const int h = (int)((idx / ((int64_t)cpr * a.T)) % a.Hkv);
+  const int b = (int)(idx / ((int64_t)cpr * a.T * a.Hkv));
+  const int row = (a.pos ? a.pos[b] : a.pos_all) + t;
+  if (row < 0 || row >= a.Lmax) return;  // a full cache drops the row instead of writing out of bounds
+  const int64_t src = (((int64_t)b * a.Hkv + h) * a.T + t) * a.D;
+  const raw *kn = reinterpret_cast<const raw *>(a.k_new) + src;
+  const raw *vn = reinterpret_cast<const raw *>(a.v_new) + src;
+  raw *kc = reinterpret_cast<raw *>(a.k_cache) + b * a.ks[0] + h * a.ks[1] + (int64_t)row * a.ks[2];
+  raw *vc = reinterpret_cast<raw *>(a.v_cache) + b * a.vs[0] + h * a.vs[1] + (int64_t)row * a.vs[2];
+  const int d0 = c * V, d1 = half + c * V;
+  Chunk<E> k0, k1;
+  k0.u = *reinterpret_cast<const uint4 *>(kn + d0);
+  k1.u = *reinterpret_cast<const uint4 *>(kn + d1);
+  const uint4 v0 = *reinterpret_cast<const uint4 *>(vn + d0), v1 = *reinterpret_cast<const uint4 *>(vn + d1);
+  if (a.rope_k) {
+    float sn[V], cs[V];
+    if (a.interleaved) {
+      sincos_pairs<E>((float)row, d0 / 2, V / 2, a.D, a.log2_base, sn, cs);
+      rotate_interleaved<E>(k0, sn, cs);
+      sincos_pairs<E>((float)row, d1 / 2, V / 2, a.D, a.log2_base, sn, cs);
+      rotate_interleaved<E>(k1, sn, cs);
+    } else {
+      sincos_pairs<E>((float)row, d0, V, a.D, a.log2_base, sn, cs);
+      rotate_chunks<E>(k0, k1, sn, cs);
+    }
+  }
+  *reinterpret_cast<uint4 *>(kc + d0) = k0.u;
+  *reinterpret_cast<uint4 *>(kc + d1) = k1.u;
+  *reinterpret_cast<uint4 *>(vc + d0) = v0;
+  *reinterpret_cast<uint4 *>(vc + d1) = v1;
+}
+
+bool chunks_ok(const void *p0, const void *p1, const int64_t *s0, const int64_t *s1, int vec) {
+  if ((reinterpret_cast<uintptr_t>(p0) | reinterpret_cast<uintptr_t>(p1)) & 15u) return false;
+  for (int i = 0; i < 3; i++)
+    if (s0[i] % vec != 0 || s1[i] % vec != 0) return false;
+  return true;
+}
+
+template <typename E>
+void launch_rope_vec(const RopeArgs &a, hipStream_t stream) {
+  const int cpr = a.interleaved ? a.D / E::kVec : a.D / 2 / E::kVec;
+  const int64_t blocks_x = ((int64_t)a.B * a.S * cpr + 255) / 256;
+  // about 1024 workgroups fill the chip; beyond that, more heads per thread amortise the sin / cos
+  // (C2's Q, 25 MB: 16.9 us with one head per thread, 11.0 us at 3; large tensors lose ~5 % to the longer threads)
+  int blocks_y = (int)((1024 + blocks_x - 1) / blocks_x);
+  blocks_y = blocks_y < 1 ? 1 : (blocks_y > a.H ? a.H : blocks_y);
+  const int heads_per_block = (a.H + blocks_y - 1) / blocks_y;
+  blocks_y = (a.H + heads_per_block - 1) / heads_per_block;
+  dim3 grid((unsigned)blocks_x, (unsigned)blocks_y), block(256);
+  if (a.interleaved)
+    hipLaunchKernelGGL((rope_vec_kernel<E, true>), grid, block, 0, stream, a, heads_per_block);
+  else
+    hipLaunchKernelGGL((rope_vec_kernel<E, false>), grid, block, 0, stream, a, heads_per_block);
+}
+
 int grid_for(int64_t total) {
   int64_t blocks = (total + 255) / 256;
   return (int)(blocks < 1 ? 1 : (blocks > 65536 ? 65536 : blocks));
@@ -90,6 +238,19 @@ int grid_for(int64_t total) {
 }  // namespace
 
 int launch_rope(const RopeArgs &a, int dtype, hipStream_t stream) {
+  const int vec = dtype == LMH_F32 ? 4 : 8;
+  const int64_t vec_threads = (int64_t)a.B * a.S * (a.D / vec);
+  if (a.D % (a.interleaved ? vec : 2 * vec) == 0 && chunks_ok(a.x, a.out, a.xs, a.os, vec) &&
+      a.H <= 65535 && vec_threads / 256 < (int64_t(1) << 31)) {
+    switch (dtype) {
+      case LMH_F32: launch_rope_vec<F32>(a, stream); break;
+      case LMH_F16: launch_rope_vec<F16>(a, stream); break;
+      case LMH_BF16: launch_rope_vec<BF16>(a, stream); break;
+      default: return fail(LMH_E_UNSUPPORTED, "rope: unknown dtype %d", dtype);
+    }
+    LMH_HIP_TRY(hipGetLastError());
+    return LMH_OK;
+  }
   const int64_t total = (int64_t)a.B * a.H * a.S * (a.D / 2);
   dim3 grid(grid_for(total)), block(256);
   switch (dtype) {
@@ -103,6 +264,21 @@ int launch_rope(const RopeArgs &a, int dtype, hipStream_t stream) {
 }
 
 int launch_kv_append(const KvAppendArgs &a, int dtype, hipStream_t stream) {
+  const int vec = dtype == LMH_F32 ? 4 : 8;
+  const int64_t vec_blocks = ((int64_t)a.B * a.Hkv * a.T * (a.D / (2 * vec)) + 255) / 256;
+  if (a.D % (2 * vec) == 0 && chunks_ok(a.k_cache, a.v_cache, a.ks, a.vs, vec) &&
+      ((reinterpret_cast<uintptr_t>(a.k_new) | reinterpret_cast<uintptr_t>(a.v_new)) & 15u) == 0 &&
+      vec_blocks >= 64 && vec_blocks < (int64_t(1) << 31)) {  // a decode step's few rows: one element per thread is quicker
+    dim3 grid((unsigned)vec_blocks), block(256);
+    switch (dtype) {
+      case LMH_F32: hipLaunchKernelGGL(kv_append_vec_kernel<F32>, grid, block, 0, stream, a); break;
+      case LMH_F16: hipLaunchKernelGGL(kv_append_vec_kernel<F16>, grid, block, 0, stream, a); break;
+      case LMH_BF16: hipLaunchKernelGGL(kv_append_vec_kernel<BF16>, grid, block, 0, stream, a); break;
+      default: return fail(LMH_E_UNSUPPORTED, "kv append: unknown dtype %d", dtype);
+    }
+    LMH_HIP_TRY(hipGetLastError());
+    return LMH_OK;
+  }
   const int64_t total = (int64_t)a.B * a.Hkv * a.T * a.D;
   dim3 grid(grid_for(total)), block(256);
   switch (dtype) {

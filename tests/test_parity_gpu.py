@@ -389,8 +389,9 @@ def test_rerun_is_bitwise_deterministic(lm, hip, oracle):
 # ---------------------------------------------------------------------------------------------
 @pytest.mark.parametrize("dtype", ["f32", "f16", "bf16"])
 @pytest.mark.parametrize("interleaved", [False, True])
-def test_rope(lm, hip, oracle, dtype, interleaved):
-    B, H, S, D = 2, 3, 37, 64
+@pytest.mark.parametrize("D", [64, 96, 20])  # 20: no 16-byte chunks, one element per thread
+def test_rope(lm, hip, oracle, dtype, interleaved, D):
+    B, H, S = 2, 3, 37
     x = oracle.round_to(oracle.gen_normal((B, H, S, D), 9000), dtype)
     dx = lm.to_device(x, hip, dtype)
     got = lm.apply_rotary_embeddings(dx, prev_seq=100, interleaved=interleaved).to_host()
@@ -412,8 +413,10 @@ def test_rope_reference_graph_replay_fp32(lm, hip, oracle):
 
 
 @pytest.mark.parametrize("dtype", ["f32", "bf16"])
-def test_kv_append_in_place(lm, hip, oracle, dtype):
-    B, Hkv, Lmax, D, T = 3, 2, 50, 128, 2
+@pytest.mark.parametrize("D", [128, 24, 20])  # 24: 16-byte chunks for fp32 only; 20: for neither
+@pytest.mark.parametrize("interleaved", [False, True])
+def test_kv_append_in_place(lm, hip, oracle, dtype, D, interleaved):
+    B, Hkv, Lmax, T = 3, 2, 50, 2
     kc = oracle.round_to(oracle.gen_normal((B, Hkv, Lmax, D), 9200), dtype)
     vc = oracle.round_to(oracle.gen_normal((B, Hkv, Lmax, D), 9201), dtype)
     kn = oracle.round_to(oracle.gen_normal((B, Hkv, T, D), 9202), dtype)
@@ -425,9 +428,31 @@ def test_kv_append_in_place(lm, hip, oracle, dtype):
     np.testing.assert_array_equal(dv.to_host(), oracle.kv_append(vc, vn, pos))
     # fused rotary embedding of K: equals rope at the row position, then append; V untouched
     dk2, dv2 = lm.to_device(kc, hip, dtype), lm.to_device(vc, hip, dtype)
-    lm.kv_append(dk2, dv2, dkn, dvn, lm.to_device(pos, hip), rope_k=True)
-    kn_rot = oracle.round_to(oracle.rope(kn, pos0=pos), dtype)
+    lm.kv_append(dk2, dv2, dkn, dvn, lm.to_device(pos, hip), rope_k=True, interleaved=interleaved)
+    kn_rot = oracle.round_to(oracle.rope(kn, pos0=pos, interleaved=interleaved), dtype)
     tol = 2e-5 if dtype == "f32" else 8e-3
+    assert rel_err(dk2.to_host(), oracle.kv_append(kc, kn_rot, pos)) <= tol
+    np.testing.assert_array_equal(dv2.to_host(), oracle.kv_append(vc, vn, pos))
+
+
+@pytest.mark.parametrize("dtype", ["f32", "f16", "bf16"])
+@pytest.mark.parametrize("interleaved", [False, True])
+def test_kv_append_whole_prompt(lm, hip, oracle, dtype, interleaved):
+    # enough rows for the 16-byte-chunk kernel; the last sequence runs into the end of the cache
+    B, Hkv, Lmax, D, T = 3, 4, 400, 64, 250
+    kc = oracle.round_to(oracle.gen_normal((B, Hkv, Lmax, D), 9250), dtype)
+    vc = oracle.round_to(oracle.gen_normal((B, Hkv, Lmax, D), 9251), dtype)
+    kn = oracle.round_to(oracle.gen_normal((B, Hkv, T, D), 9252), dtype)
+    vn = oracle.round_to(oracle.gen_normal((B, Hkv, T, D), 9253), dtype)
+    pos = np.array([0, 150, 300], np.int32)
+    dk, dv, dkn, dvn = (lm.to_device(a, hip, dtype) for a in (kc, vc, kn, vn))
+    lm.kv_append(dk, dv, dkn, dvn, lm.to_device(pos, hip))
+    np.testing.assert_array_equal(dk.to_host(), oracle.kv_append(kc, kn, pos))
+    np.testing.assert_array_equal(dv.to_host(), oracle.kv_append(vc, vn, pos))
+    dk2, dv2 = lm.to_device(kc, hip, dtype), lm.to_device(vc, hip, dtype)
+    lm.kv_append(dk2, dv2, dkn, dvn, lm.to_device(pos, hip), rope_k=True, interleaved=interleaved)
+    kn_rot = oracle.round_to(oracle.rope(kn, pos0=pos, interleaved=interleaved), dtype)
+    tol = {"f32": 1e-4, "f16": 2e-3, "bf16": 8e-3}[dtype]  # fp32: angles up to 550 rad, fp32 angle rounding
     assert rel_err(dk2.to_host(), oracle.kv_append(kc, kn_rot, pos)) <= tol
     np.testing.assert_array_equal(dv2.to_host(), oracle.kv_append(vc, vn, pos))
 
