@@ -23,25 +23,33 @@
 namespace lmh {
 namespace {
 
-constexpr int BM = 128;  // query rows per workgroup
-constexpr int BN = 32;   // keys per tile
+constexpr int BN = 32;   // keys a wave takes per tile
+constexpr int kNumCUs = 256;
 constexpr int kPadK = 4;  // floats: a row stride of D + 4 puts 16 consecutive rows' 16-byte reads on distinct banks
 constexpr int kPadV = 8;  // floats: rows key and key + 4 (the two halves of a wave) land 32 banks apart
 constexpr float kLog2e = 1.4426950408889634f;
 constexpr float kLazyRescale = 8.0f;  // see prefill_mfma.hip: the running max is raised only when outgrown by 2^8
 typedef float floatx4_t __attribute__((ext_vector_type(4)));
 
-template <int D, bool CAUSAL>
-__global__ __launch_bounds__(256, (D <= 96 ? 3 : 2)) void prefill_f32_kernel(PrefillArgs a, int n_q_tiles, int n_bh_groups) {
+// KSPLIT = 1: the four waves own 4 x 32 query rows and walk the same 32-key tiles.
+// KSPLIT = 2, 4: for launches far too small to fill the chip (the reference's own test sizes), where the
+// time is one wave's walk over its keys at 64 cycles per MFMA. The workgroup owns 128 / KSPLIT query rows
+// and stages tiles of 32 KSPLIT keys; wave group kg takes keys 32 kg .. 32 kg + 31 of every tile with its
+// own running max / sum / output, and the groups are merged through LDS at the end.
+template <int D, bool CAUSAL, int KSPLIT>
+__global__ __launch_bounds__(256, (KSPLIT > 1 ? 1 : D <= 96 ? 3 : 2)) void prefill_f32_kernel(PrefillArgs a, int n_q_tiles, int n_bh_groups) {
+  constexpr int BM = 128 / KSPLIT;  // query rows per workgroup
+  constexpr int BT = BN * KSPLIT;   // keys per staged tile
+  constexpr int RG = 4 / KSPLIT;    // waves (32-row groups) per key group
   constexpr int KJ = D / 8;         // 128-bit K fragments per tile (4 MFMAs each)
   constexpr int DB = D / 32;        // 32-row blocks of O^T
   constexpr int CPR = D / 4;        // 16-byte chunks per K/V row
-  constexpr int CH = BN * CPR / 256;  // chunks per thread per tile
+  constexpr int CH = BT * CPR / 256;  // chunks per thread per tile
   constexpr int LDK = D + kPadK;    // LDS row strides in floats
   constexpr int LDV = D + kPadV;
 
-  __shared__ __attribute__((aligned(16))) float Ks2[2][BN * LDK];  // double-buffered tiles
-  __shared__ __attribute__((aligned(16))) float Vs2[2][BN * LDV];
+  __shared__ __attribute__((aligned(16))) float Ks2[2][BT * LDK];  // double-buffered tiles
+  __shared__ __attribute__((aligned(16))) float Vs2[2][BT * LDV];
 
   // ---- which (b, hq, query tile) this workgroup owns: see prefill_mfma.hip ----
   const int bid = blockIdx.x;
@@ -58,7 +66,8 @@ __global__ __launch_bounds__(256, (D <= 96 ? 3 : 2)) void prefill_f32_kernel(Pre
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = tid >> 6;
   const int n = lane & 31, g = lane >> 5;
-  const int wave_q_lo = q0 + wave * 32;
+  const int kg = wave / RG;  // key group of this wave (always 0 when KSPLIT == 1)
+  const int wave_q_lo = q0 + (wave % RG) * 32;
   const int wave_q_hi = wave_q_lo + 31;
   const int qi = wave_q_lo + n;
 
@@ -66,7 +75,7 @@ __global__ __launch_bounds__(256, (D <= 96 ? 3 : 2)) void prefill_f32_kernel(Pre
   n_keys = min(max(n_keys, 0), a.Sk);
   int k_end = n_keys;
   if (CAUSAL) k_end = min(k_end, q0 + BM);
-  const int n_kv_tiles = (k_end + BN - 1) / BN;
+  const int n_kv_tiles = (k_end + BT - 1) / BT;
 
   const float *qp = reinterpret_cast<const float *>(a.q) + b * a.qs[0] + hq * a.qs[1];
   const float *kp = reinterpret_cast<const float *>(a.k) + b * a.ks[0] + kvh * a.ks[1];
@@ -106,7 +115,7 @@ __global__ __launch_bounds__(256, (D <= 96 ? 3 : 2)) void prefill_f32_kernel(Pre
     k_lds_off[r] = row * LDK + col * 4;
     v_lds_off[r] = row * LDV + col * 4;
   }
-  const int k_tile_bytes = (int)(BN * a.ks[2] * 4), v_tile_bytes = (int)(BN * a.vs[2] * 4);
+  const int k_tile_bytes = (int)(BT * a.ks[2] * 4), v_tile_bytes = (int)(BT * a.vs[2] * 4);
   typedef unsigned int u32x4_t __attribute__((ext_vector_type(4)));
   u32x4_t kreg[CH], vreg[CH];
   auto load_tile = [&](int kt) {
@@ -139,11 +148,12 @@ __global__ __launch_bounds__(256, (D <= 96 ? 3 : 2)) void prefill_f32_kernel(Pre
     __syncthreads();
     if (kt + 1 < n_kv_tiles) store_tile((kt + 1) & 1);
     if (kt + 2 < n_kv_tiles) load_tile(kt + 2);
-    const float *Ks = Ks2[kt & 1];
-    const float *Vs = Vs2[kt & 1];
+    const float *Ks = Ks2[kt & 1] + kg * (BN * LDK);
+    const float *Vs = Vs2[kt & 1] + kg * (BN * LDV);
 
-    const int k0 = kt * BN;
-    if (CAUSAL && k0 > wave_q_hi) continue;  // whole tile above this wave's diagonal
+    const int k0 = kt * BT + kg * BN;         // first key of this wave's share of the tile
+    if (CAUSAL && k0 > wave_q_hi) continue;   // all of it above this wave's diagonal
+    if (KSPLIT > 1 && k0 >= k_end) continue;  // ... or past the last key
 
     // ---- S^T = K Q^T: 32 keys x 32 queries, contraction over the head dim two elements per MFMA ----
     floatx16_t sacc;
@@ -202,6 +212,40 @@ __global__ __launch_bounds__(256, (D <= 96 ? 3 : 2)) void prefill_f32_kernel(Pre
     }
   }
 
+  // ---- key groups: fold the other groups' (m, l, O) into group 0's; lane for lane the same layout ----
+  if (KSPLIT > 1) {
+    constexpr int NF = DB * 16 + 2;  // floats per lane
+    static_assert(KSPLIT == 1 || (KSPLIT - 1) * RG * NF * 64 * 4 <= (int)sizeof(Ks2), "merge buffer must fit in the K tiles");
+    float *xch = &Ks2[0][0] + (wave % RG) * (NF * 64) + lane;  // [KSPLIT - 1][RG][NF][64 lanes]
+    __syncthreads();  // every wave has read its last tile
+    if (kg > 0) {
+      float *w = xch + (kg - 1) * (RG * NF * 64);
+      w[0] = m_i;
+      w[64] = l_i;
+#pragma unroll
+      for (int db = 0; db < DB; db++)
+#pragma unroll
+        for (int i = 0; i < 16; i++) w[(2 + db * 16 + i) * 64] = oacc[db][i];
+    }
+    __syncthreads();
+    if (kg > 0) return;
+#pragma unroll
+    for (int og = 1; og < KSPLIT; og++) {
+      const float *r = xch + (og - 1) * (RG * NF * 64);
+      const float m1 = r[0], l1 = r[64];
+      const float m_new = fmaxf(m_i, m1);
+      // a group that saw no key has m = -inf, l = 0, O = 0
+      const float a0 = m_i == -INFINITY ? 0.f : __builtin_amdgcn_exp2f((m_i - m_new) * c);
+      const float a1 = m1 == -INFINITY ? 0.f : __builtin_amdgcn_exp2f((m1 - m_new) * c);
+      m_i = m_new;
+      l_i = l_i * a0 + l1 * a1;
+#pragma unroll
+      for (int db = 0; db < DB; db++)
+#pragma unroll
+        for (int i = 0; i < 16; i++) oacc[db][i] = oacc[db][i] * a0 + r[(2 + db * 16 + i) * 64] * a1;
+    }
+  }
+
   // ---- epilogue: out[qi][d] = O^T[d][qi] / l ----
   const float l_tot = l_i + __shfl_xor(l_i, 32);
   const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
@@ -218,17 +262,27 @@ __global__ __launch_bounds__(256, (D <= 96 ? 3 : 2)) void prefill_f32_kernel(Pre
   }
 }
 
-template <int D>
-int launch_for_d(const PrefillArgs &a, hipStream_t stream) {
-  const int n_q_tiles = (a.Sq + BM - 1) / BM;
+template <int D, int KSPLIT>
+int launch_split(const PrefillArgs &a, hipStream_t stream) {
+  const int n_q_tiles = (a.Sq + 128 / KSPLIT - 1) / (128 / KSPLIT);
   const int n_bh_groups = (a.B * a.Hq + 7) / 8;
   dim3 grid(8 * n_bh_groups * n_q_tiles), block(256);
   if (a.causal)
-    hipLaunchKernelGGL((prefill_f32_kernel<D, true>), grid, block, 0, stream, a, n_q_tiles, n_bh_groups);
+    hipLaunchKernelGGL((prefill_f32_kernel<D, true, KSPLIT>), grid, block, 0, stream, a, n_q_tiles, n_bh_groups);
   else
-    hipLaunchKernelGGL((prefill_f32_kernel<D, false>), grid, block, 0, stream, a, n_q_tiles, n_bh_groups);
+    hipLaunchKernelGGL((prefill_f32_kernel<D, false, KSPLIT>), grid, block, 0, stream, a, n_q_tiles, n_bh_groups);
   LMH_HIP_TRY(hipGetLastError());
   return LMH_OK;
+}
+
+template <int D>
+int launch_for_d(const PrefillArgs &a, hipStream_t stream) {
+  // The key-split workgroups hold tiles of 64 or 128 keys in LDS, one workgroup per CU: use them only while
+  // every workgroup still gets a CU of its own. (Four-way needs 143 KB at D = 64 and does not fit beyond.)
+  const int64_t wgs = (int64_t)((a.B * a.Hq + 7) / 8) * 8 * ((a.Sq + 127) / 128);
+  if (D == 64 && 4 * wgs <= kNumCUs && a.Sk >= 4 * BN) return launch_split<D, (D == 64 ? 4 : 1)>(a, stream);
+  if (2 * wgs <= kNumCUs && a.Sk >= 2 * BN) return launch_split<D, 2>(a, stream);
+  return launch_split<D, 1>(a, stream);
 }
 
 }  // namespace

@@ -266,6 +266,26 @@ def test_prefill_small_and_large_launches_agree(lm, hip, oracle, causal):
     assert rel_err(small, large[:, :2]) <= TOL["f16"]
 
 
+@pytest.mark.parametrize("D", [64, 96, 128])
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("B", [1, 9])  # 4 heads: 8 or 72 workgroups of 128 rows -> four-way (D = 64) / two-way key split
+def test_fp32_tiny_launch_splits_keys_between_waves(lm, hip, oracle, D, causal, B):
+    Hq, Hkv, Sq, Sk = 4, 2, 100, 300
+    q, k, v = inputs(oracle, (B, Hq, Sq, D), (B, Hkv, Sk, D), "f32", 7480 + D)
+    lens = np.array(([300, 20, 33, 64, 97, 0, 129, 256, 290])[:B], np.int32)
+    kp, vp = k.copy(), v.copy()
+    for b, n in enumerate(lens):
+        kp[b, :, n:] = np.nan
+        vp[b, :, n:] = np.nan
+    got = run_flash(lm, hip, q, kp, vp, "f32", causal, kv_len=lens)
+    want = oracle.flash_attn(q, k, v, causal=causal, kv_len=np.maximum(lens, 1), nthreads=NT)
+    keep = [b for b in range(B) if lens[b] > 0]
+    for b in range(B):
+        if lens[b] == 0:
+            assert np.all(got[b] == 0)
+    assert rel_err(got[keep], want[keep]) <= TOL["f32"]
+
+
 @pytest.mark.parametrize("dtype", ["f16", "bf16"])
 def test_unusual_head_dim_and_scale_take_the_vector_path(lm, hip, oracle, dtype):
     q, k, v = inputs(oracle, (1, 2, 90, 80), (1, 2, 90, 80), dtype, 7500)
