@@ -28,6 +28,9 @@ constexpr int kNumCUs = 256;
 constexpr int kPadK = 4;  // floats: a row stride of D + 4 puts 16 consecutive rows' 16-byte reads on distinct banks
 constexpr int kPadV = 8;  // floats: rows key and key + 4 (the two halves of a wave) land 32 banks apart
 constexpr float kLog2e = 1.4426950408889634f;
+// Byte offset no K/V slice reaches (the host routes larger ones elsewhere): a buffer load there is out of
+// range and returns zeros.
+constexpr int kOutOfRange = 0x7ffffff0;
 constexpr float kLazyRescale = 8.0f;  // see prefill_mfma.hip: the running max is raised only when outgrown by 2^8
 typedef float floatx4_t __attribute__((ext_vector_type(4)));
 
@@ -43,7 +46,10 @@ __global__ __launch_bounds__(256, (KSPLIT > 1 ? 1 : D <= 96 ? 3 : 2)) void prefi
   constexpr int RG = 4 / KSPLIT;    // waves (32-row groups) per key group
   constexpr int KJ = D / 8;         // 128-bit K fragments per tile (4 MFMAs each)
   constexpr int DB = D / 32;        // 32-row blocks of O^T
-  constexpr int CPR = D / 4;        // 16-byte chunks per K/V row
+  constexpr int CPR = D / 4;        // 16-byte chunks per K/V row of the tiling
+  // the tensors' own head dim a.D may be smaller than the tiled D (any multiple of 8): the missing
+  // columns are never fetched (zeros in Q, K and V) and never stored.
+  const int cpr = a.D / 4;
   constexpr int CH = BT * CPR / 256;  // chunks per thread per tile
   constexpr int LDK = D + kPadK;    // LDS row strides in floats
   constexpr int LDV = D + kPadV;
@@ -86,7 +92,7 @@ __global__ __launch_bounds__(256, (KSPLIT > 1 ? 1 : D <= 96 ? 3 : 2)) void prefi
 #pragma unroll
   for (int j = 0; j < KJ; j++) {
     float4 raw = make_float4(0.f, 0.f, 0.f, 0.f);
-    if (qi < a.Sq) raw = *reinterpret_cast<const float4 *>(qp + (int64_t)qi * a.qs[2] + 8 * j + 4 * g);
+    if (qi < a.Sq && 8 * j + 4 * g < a.D) raw = *reinterpret_cast<const float4 *>(qp + (int64_t)qi * a.qs[2] + 8 * j + 4 * g);
     qf[j] = (floatx4_t){raw.x, raw.y, raw.z, raw.w};
   }
 
@@ -110,8 +116,8 @@ __global__ __launch_bounds__(256, (KSPLIT > 1 ? 1 : D <= 96 ? 3 : 2)) void prefi
   for (int r = 0; r < CH; r++) {
     const int id = tid + 256 * r;
     const int row = id / CPR, col = id % CPR;
-    k_voff[r] = (int)((row * a.ks[2] + col * 4) * 4);
-    v_voff[r] = (int)((row * a.vs[2] + col * 4) * 4);
+    k_voff[r] = col < cpr ? (int)((row * a.ks[2] + col * 4) * 4) : kOutOfRange;
+    v_voff[r] = col < cpr ? (int)((row * a.vs[2] + col * 4) * 4) : kOutOfRange;
     k_lds_off[r] = row * LDK + col * 4;
     v_lds_off[r] = row * LDV + col * 4;
   }
@@ -256,6 +262,7 @@ __global__ __launch_bounds__(256, (KSPLIT > 1 ? 1 : D <= 96 ? 3 : 2)) void prefi
 #pragma unroll
       for (int i4 = 0; i4 < 4; i4++) {
         const int d = db * 32 + 8 * i4 + 4 * g;
+        if (d >= a.D) continue;
         *reinterpret_cast<float4 *>(op + d) = make_float4(oacc[db][4 * i4 + 0] * inv, oacc[db][4 * i4 + 1] * inv,
                                                           oacc[db][4 * i4 + 2] * inv, oacc[db][4 * i4 + 3] * inv);
       }
@@ -287,14 +294,12 @@ int launch_for_d(const PrefillArgs &a, hipStream_t stream) {
 
 }  // namespace
 
-bool prefill_f32_mfma_supported(int dtype, int D) { return dtype == LMH_F32 && (D == 64 || D == 96 || D == 128); }
+bool prefill_f32_mfma_supported(int dtype, int D) { return dtype == LMH_F32 && D >= 8 && D <= 128 && D % 8 == 0; }
 
 int launch_prefill_f32_mfma(const PrefillArgs &a, hipStream_t stream) {
-  switch (a.D) {
-    case 64: return launch_for_d<64>(a, stream);
-    case 96: return launch_for_d<96>(a, stream);
-    case 128: return launch_for_d<128>(a, stream);
-  }
+  if (a.D <= 64) return launch_for_d<64>(a, stream);
+  if (a.D <= 96) return launch_for_d<96>(a, stream);
+  if (a.D <= 128) return launch_for_d<128>(a, stream);
   return fail(LMH_E_UNSUPPORTED, "fp32 MFMA flash attention: head dim %d not tiled", a.D);
 }
 

@@ -107,7 +107,9 @@ __global__ __launch_bounds__(256, (D <= 96 ? 3 : 2)) void prefill_mfma_kernel(Pr
   constexpr int BW = 32 * NKB;      // ... in keys
   constexpr int KS = D / 16;       // k-steps of the S^T product
   constexpr int DB = D / 32;       // 32-row blocks of O^T
-  constexpr int CPR = D / 8;       // 16-byte chunks per K/V row
+  // D is the tiled head dim; the tensors' own head dim a.D may be smaller (any multiple of 8): the
+  // missing columns are never fetched (zeros in Q, K and V) and never stored.
+  const int cpr = a.D / 8;         // 16-byte chunks per K/V row in memory
   constexpr int LDK = D + kPadK;   // LDS row strides in elements
   constexpr int LDV = D + pad_v<D>();
 
@@ -152,7 +154,7 @@ __global__ __launch_bounds__(256, (D <= 96 ? 3 : 2)) void prefill_mfma_kernel(Pr
 #pragma unroll
   for (int ks = 0; ks < KS; ks++) {
     uint4 raw = make_uint4(0, 0, 0, 0);
-    if (qi < a.Sq) raw = *reinterpret_cast<const uint4 *>(qp + (int64_t)qi * a.qs[2] + 16 * ks + 8 * g);
+    if (qi < a.Sq && 16 * ks + 8 * g < a.D) raw = *reinterpret_cast<const uint4 *>(qp + (int64_t)qi * a.qs[2] + 16 * ks + 8 * g);
     qreg[ks] = __builtin_bit_cast(vec8, raw);
   }
 
@@ -199,13 +201,13 @@ __global__ __launch_bounds__(256, (D <= 96 ? 3 : 2)) void prefill_mfma_kernel(Pr
   for (int j = 0; j < KJ; j++) {
     const int ch = (wave + 4 * j) * 64 + lane;
     const int row = ch / KC, col = ch % KC;
-    k_voff[j] = col < CPR ? (int)((row * a.ks[2] + col * 8) * 2) : kOutOfRange;
+    k_voff[j] = col < cpr ? (int)((row * a.ks[2] + col * 8) * 2) : kOutOfRange;
   }
 #pragma unroll
   for (int j = 0; j < VJ; j++) {
     const int ch = (wave + 4 * j) * 64 + lane;
     const int row = ch / VC, col = ch % VC;
-    v_voff[j] = col < CPR ? (int)((row * a.vs[2] + col * 8) * 2) : kOutOfRange;
+    v_voff[j] = col < cpr ? (int)((row * a.vs[2] + col * 8) * 2) : kOutOfRange;
   }
   const int k_tile_bytes = (int)(BT * a.ks[2] * 2), v_tile_bytes = (int)(BT * a.vs[2] * 2);
   const uint32_t k_lds0 = (uint32_t)(uintptr_t)(lds_void_t *)&Ks2[0][0] + wave_u * 1024;
@@ -378,6 +380,7 @@ __global__ __launch_bounds__(256, (D <= 96 ? 3 : 2)) void prefill_mfma_kernel(Pr
 #pragma unroll
       for (int i4 = 0; i4 < 4; i4++) {
         const int d = db * 32 + 8 * i4 + 4 * g;
+        if (d >= a.D) continue;
         if (a.out_f32) {
           *reinterpret_cast<float4 *>(op32 + d) =
               make_float4(oacc[db][4 * i4 + 0] * inv, oacc[db][4 * i4 + 1] * inv, oacc[db][4 * i4 + 2] * inv,
@@ -422,18 +425,17 @@ int launch_for_d(const PrefillArgs &a, hipStream_t stream) {
 
 template <typename MT>
 int launch_for_type(const PrefillArgs &a, hipStream_t stream) {
-  switch (a.D) {
-    case 64: return launch_for_d<MT, 64>(a, stream);
-    case 96: return launch_for_d<MT, 96>(a, stream);
-    case 128: return launch_for_d<MT, 128>(a, stream);
-  }
+  // the smallest tiling that holds the head dim; the padding costs its share of the MFMAs
+  if (a.D <= 64) return launch_for_d<MT, 64>(a, stream);
+  if (a.D <= 96) return launch_for_d<MT, 96>(a, stream);
+  if (a.D <= 128) return launch_for_d<MT, 128>(a, stream);
   return fail(LMH_E_UNSUPPORTED, "MFMA flash attention: head dim %d not tiled", a.D);
 }
 
 }  // namespace
 
 bool prefill_mfma_supported(int dtype, int D) {
-  return (dtype == LMH_F16 || dtype == LMH_BF16) && (D == 64 || D == 96 || D == 128);
+  return (dtype == LMH_F16 || dtype == LMH_BF16) && D >= 8 && D <= 128 && D % 8 == 0;
 }
 
 int launch_prefill_mfma(const PrefillArgs &a, int dtype, hipStream_t stream) {

@@ -286,9 +286,23 @@ def test_fp32_tiny_launch_splits_keys_between_waves(lm, hip, oracle, D, causal, 
     assert rel_err(got[keep], want[keep]) <= TOL["f32"]
 
 
+@pytest.mark.parametrize("dtype", ["f32", "f16", "bf16"])
+@pytest.mark.parametrize("D", [8, 40, 72, 80, 104, 120])
+@pytest.mark.parametrize("Sq,Sk", [(70, 70), (200, 700)])  # the second takes the key-split workgroups
+def test_head_dims_between_the_tilings_run_padded_on_the_matrix_cores(lm, hip, oracle, dtype, D, Sq, Sk):
+    q, k, v = inputs(oracle, (2, 4, Sq, D), (2, 2, Sk, D), dtype, 7460 + D)
+    lens = np.array([Sk, Sk // 3], np.int32)
+    kp, vp = k.copy(), v.copy()
+    kp[1, :, lens[1]:] = np.nan
+    vp[1, :, lens[1]:] = np.nan
+    for causal in (False, True):
+        got = run_flash(lm, hip, q, kp, vp, dtype, causal, kv_len=lens)
+        assert rel_err(got, oracle.flash_attn(q, k, v, causal=causal, kv_len=lens, nthreads=NT)) <= TOL[dtype]
+
+
 @pytest.mark.parametrize("dtype", ["f16", "bf16"])
 def test_unusual_head_dim_and_scale_take_the_vector_path(lm, hip, oracle, dtype):
-    q, k, v = inputs(oracle, (1, 2, 90, 80), (1, 2, 90, 80), dtype, 7500)
+    q, k, v = inputs(oracle, (1, 2, 90, 20), (1, 2, 90, 20), dtype, 7500)  # not a multiple of 8
     assert rel_err(run_flash(lm, hip, q, k, v, dtype, True), oracle.flash_attn(q, k, v, causal=True)) <= 2e-3
     q, k, v = inputs(oracle, (1, 2, 90, 64), (1, 2, 90, 64), dtype, 7501)
     for scale in (-0.2, 0.0):
