@@ -333,6 +333,38 @@ def other_configs(lm, dev):
         ap.B, ap.Hkv, ap.T, ap.D, ap.Lmax = B, Hkv, T, D, L
         ap.dtype, ap.rope_k, ap.pairing, ap.base, ap.stream = lm.binding.DTYPE_CODES["bf16"], 1, lm.binding.ROPE_HALF_SPLIT, 10000.0, None
         hbm_line("cache append + rotary K bf16 B=16 Hkv=8 D=128, %s" % label, lambda: lm.binding.kv_append(ap), 4.0 * B * Hkv * T * D * 2)
+
+    # one whole decode step of an attention layer (rotary q, append with rotary K, split-KV attention, merge: 4
+    # kernels), driven from the host step by step and as one recorded HIP graph; wall clock per step. On the C4
+    # shape the GPU is the bottleneck either way; a single short sequence is bound by the host's launches.
+    for B, L in ((16, 4096), (1, 512)):
+        Hq, Hkv, D = 32, 8, 128
+        g = lm.Graph()
+        tq, tkn, tvn = lm.tensor(g, (B, Hq, 1, D), "bf16"), lm.tensor(g, (B, Hkv, 1, D), "bf16"), lm.tensor(g, (B, Hkv, 1, D), "bf16")
+        tkc, tvc = lm.tensor(g, (B, Hkv, L, D), "bf16"), lm.tensor(g, (B, Hkv, L, D), "bf16")
+        tpos, tlen = lm.tensor(g, (B,), "i32"), lm.tensor(g, (B,), "i32")
+        lm.cached_self_attention_core(tq, tkn, tvn, tkc, tvc, tpos, tlen, rope_base=10000.0, out_dtype="f32")
+        cg = lm.compile(g, dev)
+        cg({tpos.id: np.full(B, L - 1, np.int32), tlen.id: np.full(B, L, np.int32)})
+
+        def wall_us(n=200):
+            for _ in range(20):
+                cg({})
+            lm.binding.sync()
+            t0 = time.perf_counter()
+            for _ in range(n):
+                cg({})
+            lm.binding.sync(cg._stream)
+            lm.binding.sync()
+            return (time.perf_counter() - t0) / n * 1e6
+
+        eager = wall_us()
+        cg.capture()
+        replay = wall_us()
+        cg.release()
+        res["decode step of a layer bf16 B=%d Hq=32 Hkv=8 L=%d D=128 (rotary q + append + attention), wall clock" % (B, L)] = {
+            "us_per_step_4_launches_from_the_host": eager, "us_per_step_one_hip_graph": replay}
+        log("[other] decode step B=%d L=%d, wall clock: %.1f us as 4 host launches, %.1f us as one HIP graph" % (B, L, eager, replay))
     return res
 
 

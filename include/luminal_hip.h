@@ -75,6 +75,26 @@ int lmh_event_destroy(void *event);
 int lmh_event_record(void *event, void *stream);
 int lmh_event_elapsed_ms(float *ms, void *start, void *stop);
 
+/* ---- a compiled step list as one launch: replaces the closure compile() returns in the reference
+ * (reference src/Compiler.jl:250-255: a Julia loop over execute_op! calls with captured buffers).
+ * Every entry point above enqueues on the stream it is given and allocates nothing, so a sequence of
+ * them on persistent buffers can be recorded once into a HIP graph and replayed; per-step values
+ * (positions, lengths) live in device memory, so one recording serves every decode position.
+ *   lmh_stream_create      a stream that can be captured (the null stream cannot); default priority,
+ *                          blocking with respect to the null stream
+ *   lmh_graph_capture_begin / _end   record what is enqueued on `stream` in between; _end returns an
+ *                          executable graph (and must be called even after a failed call in between)
+ *   lmh_graph_launch       replay on `stream`
+ * Nothing may be allocated, freed, copied to the host or synchronised on the capturing stream between
+ * begin and end, and lmh_memset stays outside (it would record a memset node; clear buffers before the
+ * capture or with a kernel). ---- */
+int lmh_stream_create(void **stream);
+int lmh_stream_destroy(void *stream);
+int lmh_graph_capture_begin(void *stream);
+int lmh_graph_capture_end(void *stream, void **graph_exec);
+int lmh_graph_launch(void *graph_exec, void *stream);
+int lmh_graph_destroy(void *graph_exec);
+
 /* Measurement aid with no counterpart in the reference: a plain copy kernel (reads `bytes`,
  * writes `bytes`; both pointers and the size multiples of 16) used to calibrate HBM traffic
  * counters against a known transfer. */

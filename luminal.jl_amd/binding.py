@@ -24,7 +24,8 @@ EXPORTS = [
     "lmh_memset", "lmh_memcpy_h2d", "lmh_memcpy_d2h", "lmh_memcpy_d2d", "lmh_sync", "lmh_event_create",
     "lmh_event_destroy", "lmh_event_record", "lmh_event_elapsed_ms", "lmh_flash_attn_fwd",
     "lmh_decode_workspace_bytes", "lmh_decode_auto_splits", "lmh_decode_attn", "lmh_calib_copy", "lmh_calib_mfma", "lmh_rope",
-    "lmh_kv_append",
+    "lmh_kv_append", "lmh_stream_create", "lmh_stream_destroy", "lmh_graph_capture_begin", "lmh_graph_capture_end",
+    "lmh_graph_launch", "lmh_graph_destroy",
 ]
 
 
@@ -124,6 +125,12 @@ def load():
     L.lmh_calib_mfma.argtypes = [vp, vp, ctypes.c_size_t, ctypes.c_int, ctypes.POINTER(ctypes.c_double), vp]
     L.lmh_rope.argtypes = [ctypes.POINTER(RopeParams)]
     L.lmh_kv_append.argtypes = [ctypes.POINTER(KvAppendParams)]
+    L.lmh_stream_create.argtypes = [ctypes.POINTER(vp)]
+    L.lmh_stream_destroy.argtypes = [vp]
+    L.lmh_graph_capture_begin.argtypes = [vp]
+    L.lmh_graph_capture_end.argtypes = [vp, ctypes.POINTER(vp)]
+    L.lmh_graph_launch.argtypes = [vp, vp]
+    L.lmh_graph_destroy.argtypes = [vp]
     for name in ("lmh_rope", "lmh_kv_append", "lmh_calib_copy", "lmh_calib_mfma", "lmh_init", "lmh_device_name", "lmh_malloc", "lmh_free", "lmh_memset", "lmh_memcpy_h2d",
                  "lmh_memcpy_d2h", "lmh_memcpy_d2d", "lmh_sync", "lmh_event_create", "lmh_event_destroy",
                  "lmh_event_record", "lmh_event_elapsed_ms", "lmh_flash_attn_fwd", "lmh_decode_attn"):
@@ -217,6 +224,34 @@ def rope(params):
 
 def kv_append(params):
     check(load().lmh_kv_append(ctypes.byref(params)))
+
+
+def stream_create():
+    s = ctypes.c_void_p()
+    check(load().lmh_stream_create(ctypes.byref(s)))
+    return s
+
+
+def stream_destroy(stream):
+    check(load().lmh_stream_destroy(stream))
+
+
+def graph_capture_begin(stream):
+    check(load().lmh_graph_capture_begin(stream))
+
+
+def graph_capture_end(stream):
+    g = ctypes.c_void_p()
+    check(load().lmh_graph_capture_end(stream, ctypes.byref(g)))
+    return g
+
+
+def graph_launch(graph_exec, stream):
+    check(load().lmh_graph_launch(graph_exec, stream))
+
+
+def graph_destroy(graph_exec):
+    check(load().lmh_graph_destroy(graph_exec))
 
 
 def calib_copy(dst, src, nbytes, stream=None):

@@ -138,6 +138,53 @@ int lmh_sync(void *stream) {
   return LMH_OK;
 }
 
+int lmh_stream_create(void **stream) {
+  if (!stream) return fail(LMH_E_NULL, "lmh_stream_create: null result pointer");
+  hipStream_t s;
+  LMH_HIP_TRY(hipStreamCreate(&s));  // default flags and priority
+  *stream = s;
+  return LMH_OK;
+}
+
+int lmh_stream_destroy(void *stream) {
+  if (!stream) return LMH_OK;
+  LMH_HIP_TRY(hipStreamDestroy((hipStream_t)stream));
+  return LMH_OK;
+}
+
+int lmh_graph_capture_begin(void *stream) {
+  if (!stream) return fail(LMH_E_NULL, "lmh_graph_capture_begin: the null stream cannot be captured");
+  // thread-local: API calls of other host threads (a finalizer freeing memory) do not break the capture
+  LMH_HIP_TRY(hipStreamBeginCapture((hipStream_t)stream, hipStreamCaptureModeThreadLocal));
+  return LMH_OK;
+}
+
+int lmh_graph_capture_end(void *stream, void **graph_exec) {
+  if (!stream || !graph_exec) return fail(LMH_E_NULL, "lmh_graph_capture_end: null stream or result pointer");
+  *graph_exec = nullptr;
+  hipGraph_t graph = nullptr;
+  LMH_HIP_TRY(hipStreamEndCapture((hipStream_t)stream, &graph));
+  if (!graph) return fail(LMH_E_HIP, "lmh_graph_capture_end: the capture was invalidated");
+  hipGraphExec_t exec = nullptr;
+  const hipError_t e = hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0);
+  (void)hipGraphDestroy(graph);
+  LMH_HIP_TRY(e);
+  *graph_exec = exec;
+  return LMH_OK;
+}
+
+int lmh_graph_launch(void *graph_exec, void *stream) {
+  if (!graph_exec) return fail(LMH_E_NULL, "lmh_graph_launch: null graph");
+  LMH_HIP_TRY(hipGraphLaunch((hipGraphExec_t)graph_exec, (hipStream_t)stream));
+  return LMH_OK;
+}
+
+int lmh_graph_destroy(void *graph_exec) {
+  if (!graph_exec) return LMH_OK;
+  LMH_HIP_TRY(hipGraphExecDestroy((hipGraphExec_t)graph_exec));
+  return LMH_OK;
+}
+
 int lmh_event_create(void **event) {
   if (!event) return fail(LMH_E_NULL, "lmh_event_create: null result pointer");
   hipEvent_t e;

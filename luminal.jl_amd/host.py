@@ -396,8 +396,9 @@ class _Workspaces:
 _workspaces = _Workspaces()
 
 
-def execute_op_inplace(out, op, *inputs, stream=None):
-    """execute_op!(out, op, inputs...) (reference src/Execution.jl:565-578) for the two attention ops."""
+def execute_op_inplace(out, op, *inputs, stream=None, workspaces=None):
+    """execute_op!(out, op, inputs...) (reference src/Execution.jl:565-578) for the attention ops. `workspaces`
+    is where decode attention takes its split-KV scratch from (default: one buffer shared by all eager calls)."""
     if isinstance(op, FlashAttentionOp):
         q, k, v = inputs[:3]
         kv_len = inputs[3] if len(inputs) > 3 else None
@@ -443,7 +444,7 @@ def execute_op_inplace(out, op, *inputs, stream=None):
         p.out_f32 = int(out.dtype == "f32")
         p.num_splits = op.num_splits or binding.decode_auto_splits(p.B, p.Hkv, p.Lmax)
         need = binding.decode_workspace_bytes(p.B, p.Hq, p.Hkv, p.Lmax, p.D, p.num_splits)
-        p.workspace, p.workspace_bytes = _workspaces.get(need, q.device)
+        p.workspace, p.workspace_bytes = (workspaces or _workspaces).get(need, q.device)
         p.stream = stream
         binding.decode_attn(p)
         return out
@@ -505,11 +506,14 @@ def execute(graph, output_ids, initial_inputs, device=None, dtype=None):
 class CompiledGraph:
     """Pre-allocated node buffers + a step list (reference src/Compiler.jl:75-100). Calling it copies the
     inputs into their buffers, runs the steps in place and returns the buffer list; nothing is
-    allocated per call."""
+    allocated per call. After capture() the step list is one HIP graph launch."""
 
-    def __init__(self, steps, results):
+    def __init__(self, steps, results, workspaces=None):
         self.steps = steps
         self.results = results
+        self.workspaces = workspaces  # decode scratch owned by this graph: its address never changes
+        self._stream = None
+        self._exec = None
 
     def __call__(self, inputs, device=None):
         for k, v in inputs.items():
@@ -521,9 +525,50 @@ class CompiledGraph:
                 binding.memcpy_d2d(self.results[k].ptr, v.ptr, v.nbytes)
             else:
                 self.results[k].copy_from_host(v)
-        for step in self.steps:
-            step()
+        if self._exec is not None:
+            # the copies above ran on the null stream, which the capture stream (created blocking) waits for
+            binding.graph_launch(self._exec, self._stream)
+        else:
+            for step in self.steps:
+                step(None)
         return self.results
+
+    def capture(self):
+        """Record the step list once into a HIP graph; later calls replay it with one launch. The buffers keep
+        their addresses and per-step values (positions, lengths) are device tensors, so the recording is
+        valid for every later call. Runs the steps once eagerly first (on whatever the buffers hold), so
+        that the library's first-use set-up does not happen inside the capture."""
+        if self._exec is not None:
+            return self
+        for step in self.steps:
+            step(None)
+        binding.sync()
+        stream = binding.stream_create()
+        try:
+            binding.graph_capture_begin(stream)
+            try:
+                for step in self.steps:
+                    step(stream)
+            except Exception:
+                try:
+                    binding.graph_capture_end(stream)  # leave the stream usable; the recording is dropped
+                except binding.LuminalHipError:
+                    pass
+                raise
+            self._exec = binding.graph_capture_end(stream)
+        except Exception:
+            binding.stream_destroy(stream)
+            raise
+        self._stream = stream
+        return self
+
+    def release(self):
+        """Drop the HIP graph and its stream (the buffers stay)."""
+        if self._exec is not None:
+            binding.sync(self._stream)
+            binding.graph_destroy(self._exec)
+            binding.stream_destroy(self._stream)
+            self._exec = self._stream = None
 
 
 def compile(graph, device=None):
@@ -540,12 +585,14 @@ def compile(graph, device=None):
             continue
         results.append(HipArray(graph.shapes[node_id], graph.dtypes[node_id], device).fill_bytes(0))
     steps = []
+    workspaces = _Workspaces()
     for node_id, node in enumerate(graph.nodes):
         if isinstance(node.op, InputTensor):
             continue
         args = [_pick(results, ref) for ref in node.inputs]
-        steps.append(lambda out=results[node_id], op=node.op, args=args: execute_op_inplace(out, op, *args))
-    return CompiledGraph(steps, results)
+        steps.append(lambda stream, out=results[node_id], op=node.op, args=args:
+                     execute_op_inplace(out, op, *args, stream=stream, workspaces=workspaces))
+    return CompiledGraph(steps, results, workspaces)
 
 
 # ---------------------------------------------------------------------------------------------

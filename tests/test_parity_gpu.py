@@ -552,6 +552,53 @@ def test_compiled_decode_step_graph_serves_every_position(lm, hip, oracle):
     assert np.array_equal(res[kc2.id][1].to_host()[:, :, :S], v)
 
 
+@pytest.mark.parametrize("dtype,Lmax", [("f32", 32), ("bf16", 4096)])  # the long cache takes the split-KV kernels + merge
+def test_decode_step_recorded_as_one_hip_graph(lm, hip, oracle, dtype, Lmax):
+    """The same step graph, recorded once into a HIP graph after the first position and replayed for every later
+    one, must give bit for bit what an unrecorded twin gives, with the program's own eager launches and
+    synchronisations between the replays (reference src/Compiler.jl:250-255: the compiled step closure)."""
+    B, Hq, Hkv, S, D = 2, 8, 2, 20, 64
+    q, k, v = inputs(oracle, (B, Hq, S, D), (B, Hkv, S, D), dtype, 9450)
+    want = oracle.flash_attn(oracle.round_to(oracle.rope(q), dtype), oracle.round_to(oracle.rope(k), dtype), v, causal=True)
+
+    def build():
+        g = lm.Graph()
+        tq, tkn, tvn = lm.tensor(g, (B, Hq, 1, D), dtype), lm.tensor(g, (B, Hkv, 1, D), dtype), lm.tensor(g, (B, Hkv, 1, D), dtype)
+        tkc, tvc = lm.tensor(g, (B, Hkv, Lmax, D), dtype), lm.tensor(g, (B, Hkv, Lmax, D), dtype)
+        tpos, tlen = lm.tensor(g, (B,), "i32"), lm.tensor(g, (B,), "i32")
+        out, _, _ = lm.cached_self_attention_core(tq, tkn, tvn, tkc, tvc, tpos, tlen, rope_base=10000.0, out_dtype="f32")
+        return lm.compile(g, hip), (tq, tkn, tvn, tpos, tlen), out
+
+    cg, ids, out = build()
+    twin, ids2, out2 = build()
+
+    def feed(handles, t):
+        tq, tkn, tvn, tpos, tlen = handles
+        return {tq.id: lm.to_device(np.ascontiguousarray(q[:, :, t:t + 1]), hip, dtype),
+                tkn.id: lm.to_device(np.ascontiguousarray(k[:, :, t:t + 1]), hip, dtype),
+                tvn.id: lm.to_device(np.ascontiguousarray(v[:, :, t:t + 1]), hip, dtype),
+                tpos.id: np.full(B, t, np.int32), tlen.id: np.full(B, t + 1, np.int32)}
+
+    xq, xk, xv = inputs(oracle, (1, 4, 200, 64), (1, 4, 200, 64), "f16", 9460)
+    x_want = oracle.flash_attn(xq, xk, xv, causal=True)
+    tol = 2e-5 if dtype == "f32" else 1e-2  # bf16: q and k are rounded again after the rotation
+    for t in range(S):
+        if t == 1:
+            cg.capture()  # its eager warm-up repeats step 0 on the buffers as they are: same cache row, same values
+            assert cg._exec is not None
+        got = cg(feed(ids, t))[out.id].to_host()
+        ref = twin(feed(ids2, t))[out2.id].to_host()
+        assert np.array_equal(got, ref), t
+        assert rel_err(got, want[:, :, t]) <= tol, t
+        # unrelated eager work and a synchronisation between the replays
+        assert rel_err(run_flash(lm, hip, xq, xk, xv, "f16", True), x_want) <= TOL["f16"]
+        lm.binding.sync()
+    cg.release()
+    assert cg._exec is None
+    got = cg(feed(ids, S - 1))[out.id].to_host()  # eager again after release
+    assert rel_err(got, want[:, :, S - 1]) <= tol
+
+
 @pytest.mark.parametrize("dtype", ["f32", "f16"])
 def test_self_attention_core_is_rope_plus_gqa_flash(lm, hip, oracle, dtype):
     """Prefill form of the attention layer core: rotary nodes on Q and K, then one flash node reading the Hkv heads
