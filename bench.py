@@ -261,12 +261,17 @@ def decode_leg(lm, dev, steps, warmup, cpu_seconds, num_splits=0):
     return res
 
 
-def other_configs(lm, dev):
-    """Short timings of the remaining contract configurations (20 launches each)."""
+def other_configs(lm, dev, check=False):
+    """Short timings of the remaining contract configurations (20 launches each). With `check`, C1, C3 and C4 are
+    also compared with the CPU oracle on the whole output (the parity gate of the five configurations: C2 and C5
+    are checked in their own legs)."""
     res = {}
     rng = np.random.default_rng(9)
+    if check:
+        import oracle
+        nthreads = oracle.max_threads()
 
-    def flash(name, B, Hq, Hkv, Sq, Sk, D, dtype, causal, flops):
+    def flash(name, B, Hq, Hkv, Sq, Sk, D, dtype, causal, flops, tol=None):
         q = lm.HipArray((B, Hq, Sq, D), dtype, dev).copy_from_host(rng.standard_normal((B, Hq, Sq, D), dtype=np.float32))
         k = lm.HipArray((B, Hkv, Sk, D), dtype, dev).copy_from_host(rng.standard_normal((B, Hkv, Sk, D), dtype=np.float32))
         v = lm.HipArray((B, Hkv, Sk, D), dtype, dev).copy_from_host(rng.standard_normal((B, Hkv, Sk, D), dtype=np.float32))
@@ -275,13 +280,19 @@ def other_configs(lm, dev):
         _, ev = time_steps(lambda: lm.binding.flash_attn_fwd(p), 20, 5, lm.binding)
         res[name] = {"launch_us": ev * 1e3, "TFLOP/s": flops / (ev * 1e-3) / 1e12}
         log("[other] %s: %.1f us, %.2f TFLOP/s" % (name, ev * 1e3, res[name]["TFLOP/s"]))
+        if check and tol is not None:
+            qh, kh, vh = (np.asarray(x.to_host(), np.float32) for x in (q, k, v))  # the element-type-rounded inputs
+            want = oracle.flash_attn(qh, kh, vh, scale=lm.default_scale(D), causal=causal, nthreads=nthreads)
+            err = float(np.max(np.abs(np.asarray(o.to_host(), np.float32) - want)) / np.max(np.abs(want)))
+            res[name]["parity"] = {"max_rel_err": err, "tolerance": tol, "checked": "whole output vs CPU oracle"}
+            log("[other] %s: GPU vs oracle rel err %.2e (tolerance %g)" % (name, err, tol))
 
-    flash("C1 causal fp32 B=1 H=8 S=128 D=64", 1, 8, 8, 128, 128, 64, "f32", True, 4.0 * 8 * 64 * 128 * 129 / 2)
+    flash("C1 causal fp32 B=1 H=8 S=128 D=64", 1, 8, 8, 128, 128, 64, "f32", True, 4.0 * 8 * 64 * 128 * 129 / 2, tol=1e-5)
     # the reference's element type on the C2 shape (an extra line, not one of the five configurations): fp32 matrix-core kernel
     flash("C2 shape in fp32 (causal B=1 H=32 S=4096 D=96)", 1, 32, 32, 4096, 4096, 96, "f32", True, 4.0 * 32 * 96 * 4096 * 4097 / 2)
     res["C2 shape in fp32 (causal B=1 H=32 S=4096 D=96)"]["frac_of_fp32_mfma_peak"] = \
         res["C2 shape in fp32 (causal B=1 H=32 S=4096 D=96)"]["TFLOP/s"] / PEAK_FP32_TFLOPS
-    flash("C3 cross fp16 B=4 H=20 Sq=448 Sk=1500 D=64", 4, 20, 20, 448, 1500, 64, "f16", False, 4.0 * 4 * 20 * 448 * 1500 * 64)
+    flash("C3 cross fp16 B=4 H=20 Sq=448 Sk=1500 D=64", 4, 20, 20, 448, 1500, 64, "f16", False, 4.0 * 4 * 20 * 448 * 1500 * 64, tol=2e-3)
 
     # C4: B=16 L=4096 decode; 268 MB would sit in the 256 MB last-level cache, so rotate over 4 caches
     B, Hq, Hkv, L, D = 16, 32, 8, 4096, 128
@@ -306,6 +317,15 @@ def other_configs(lm, dev):
     res["C4 decode bf16 B=16 Hq=32 Hkv=8 L=4096 D=128 (4 caches rotated)"] = {
         "launch_us": ev * 1e3, "GB/s": nbytes / (ev * 1e-3) / 1e9, "frac_of_hbm_peak": nbytes / (ev * 1e-3) / 1e9 / PEAK_HBM_GBS}
     log("[other] C4 decode: %.1f us, %.0f GB/s" % (ev * 1e3, nbytes / (ev * 1e-3) / 1e9))
+    if check:
+        lm.binding.decode_attn(ps[0])
+        qh = np.asarray(q.to_host(), np.float32)
+        kh, vh = (np.asarray(x.to_host(), np.float32) for x in caches[0])
+        want = oracle.decode_attn(qh, kh, vh, scale=lm.default_scale(D), nthreads=nthreads)
+        err = float(np.max(np.abs(np.asarray(o.to_host(), np.float32) - want)) / np.max(np.abs(want)))
+        res["C4 decode bf16 B=16 Hq=32 Hkv=8 L=4096 D=128 (4 caches rotated)"]["parity"] = {
+            "max_rel_err": err, "tolerance": 2e-3, "checked": "whole output vs CPU oracle"}
+        log("[other] C4 decode: GPU vs oracle rel err %.2e (tolerance 2e-3)" % err)
 
     # the two operators in front of attention: rotary embedding of a prompt's Q, and the cache append (K rotated on
     # the way in) for a whole prompt and for one decode step. Algorithmic bytes = every element read once, written once.
@@ -420,7 +440,15 @@ def main():
     if args.only in ("all", "decode"):
         line["decode"] = decode_leg(lm, dev, args.steps, args.warmup, args.cpu_seconds, args.decode_splits)
     if args.only in ("all", "other"):
-        line["other_configs"] = other_configs(lm, dev)
+        line["other_configs"] = other_configs(lm, dev, check=args.cpu_seconds > 0)
+    gate = [("C2", line.get("parity"))] + [("C5", line.get("decode", {}).get("parity"))] + \
+        [(k.split()[0], v.get("parity")) for k, v in line.get("other_configs", {}).items() if isinstance(v, dict) and "parity" in v]
+    gate = [(n, p) for n, p in gate if p]
+    if gate:
+        line["parity_gate"] = {"configs": [n for n, _ in gate], "all_pass": all(p["max_rel_err"] <= p["tolerance"] for _, p in gate)}
+        if not line["parity_gate"]["all_pass"]:
+            log("PARITY GATE FAILED: " + ", ".join("%s %.2e > %g" % (n, p["max_rel_err"], p["tolerance"]) for n, p in gate if p["max_rel_err"] > p["tolerance"]))
+            line["value"] = None  # no throughput is reported for a kernel that disagrees with the oracle
     print(json.dumps(line))
 
 
