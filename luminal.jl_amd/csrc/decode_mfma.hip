@@ -317,15 +317,17 @@ __global__ __launch_bounds__(kWaves * 64) void decode_mfma_kernel(DecodeArgs a, 
 template <typename MT, int D>
 int launch_for_d(const DecodeArgs &a, hipStream_t stream) {
   // Persistent launch: as many workgroups as the chip holds at once (never more than there are units).
-  static int wgs_per_device = 0;  // same for every device this library runs on (gfx950 only)
-  if (wgs_per_device == 0) {
+  // Same for every device this library runs on (gfx950 only); initialised once, thread-safely.
+  static const int wgs_per_device = [] {
     int dev = 0, per_cu = 0;
     hipDeviceProp_t prop;
-    LMH_HIP_TRY(hipGetDevice(&dev));
-    LMH_HIP_TRY(hipGetDeviceProperties(&prop, dev));
-    LMH_HIP_TRY(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, decode_mfma_kernel<MT, D>, kWaves * 64, 0));
-    wgs_per_device = (per_cu < 1 ? 1 : per_cu) * prop.multiProcessorCount;
-  }
+    if (hipGetDevice(&dev) != hipSuccess || hipGetDeviceProperties(&prop, dev) != hipSuccess ||
+        hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, decode_mfma_kernel<MT, D>, kWaves * 64, 0) != hipSuccess) {
+      (void)hipGetLastError();
+      return 256;  // one workgroup per CU: correct for any value, only the balance changes
+    }
+    return (per_cu < 1 ? 1 : per_cu) * prop.multiProcessorCount;
+  }();
   const int group = a.Hq / a.Hkv;
   const int g_chunks = (group + 15) / 16;
   const int64_t max_units = (int64_t)a.B * a.Hkv * g_chunks * a.num_splits;

@@ -142,3 +142,19 @@ def test_rope_and_kv_append_argument_errors(lm):
     with pytest.raises(lm.LuminalHipError) as e:
         b.kv_append(a)
     assert e.value.code == b.LMH_E_SHAPE
+
+
+def test_graph_recording_argument_errors(lm):
+    # the null stream cannot be captured and a null graph cannot be launched; both are refused before any HIP call
+    b = lm.binding
+    with pytest.raises(lm.LuminalHipError) as e:
+        b.graph_capture_begin(None)
+    assert e.value.code == b.LMH_E_NULL and "null stream" in str(e.value)
+    with pytest.raises(lm.LuminalHipError) as e:
+        b.graph_launch(None, None)
+    assert e.value.code == b.LMH_E_NULL
+    with pytest.raises(lm.LuminalHipError) as e:
+        b.check(b.load().lmh_graph_capture_end(None, None))
+    assert e.value.code == b.LMH_E_NULL
+    assert b.load().lmh_graph_destroy(None) == 0
+    assert b.load().lmh_stream_destroy(None) == 0
