@@ -374,7 +374,7 @@ def other_configs(lm, dev, check=False):
             t0 = time.perf_counter()
             for _ in range(n):
                 cg({})
-            lm.binding.sync(cg._stream)
+            lm.binding.sync(cg.cache.get("hip_stream"))
             lm.binding.sync()
             return (time.perf_counter() - t0) / n * 1e6
 

@@ -75,8 +75,9 @@ int lmh_event_destroy(void *event);
 int lmh_event_record(void *event, void *stream);
 int lmh_event_elapsed_ms(float *ms, void *start, void *stop);
 
-/* ---- a compiled step list as one launch: replaces the closure compile() returns in the reference
- * (reference src/Compiler.jl:250-255: a Julia loop over execute_op! calls with captured buffers).
+/* ---- a compiled step list as one launch: what execute_with_capture(device, f, cache) is meant to do
+ * in the reference (reference src/Device.jl:108-121, called from the compiled step closure at
+ * src/Compiler.jl:98; stubbed out there because freed transient workspaces invalidated the recording).
  * Every entry point above enqueues on the stream it is given and allocates nothing, so a sequence of
  * them on persistent buffers can be recorded once into a HIP graph and replayed; per-step values
  * (positions, lengths) live in device memory, so one recording serves every decode position.

@@ -503,17 +503,67 @@ def execute(graph, output_ids, initial_inputs, device=None, dtype=None):
     return final[ids[0]] if single else final
 
 
+def execute_with_capture(device, f, cache):
+    """execute_with_capture(device, f, cache) (reference src/Device.jl:108-121, called from the compiled step
+    closure, src/Compiler.jl:98): run `f` on `device`; where the device supports it, record what `f` enqueues
+    into a graph kept in `cache` and replay it on later calls. The reference stubs this out for CUDA (its
+    recording was invalidated by transient workspaces that were freed); here `f(stream)` must enqueue only on
+    the stream it is given and only on buffers that outlive the recording. Every call runs `f`'s work exactly
+    once: the first call runs it eagerly (the library's first-use set-up stays outside the recording), the second
+    records and replays, later ones replay."""
+    if not isinstance(device, HIPDevice):
+        return f(None)
+    if "hip_exec" not in cache:
+        if not cache.get("hip_warm"):
+            cache["hip_warm"] = True
+            return f(None)
+        binding.sync()
+        stream = binding.stream_create()
+        try:
+            binding.graph_capture_begin(stream)
+            try:
+                f(stream)
+            except Exception:
+                try:
+                    binding.graph_capture_end(stream)  # leave the stream usable; the recording is dropped
+                except binding.LuminalHipError:
+                    pass
+                raise
+            cache["hip_exec"] = binding.graph_capture_end(stream)
+        except Exception:
+            binding.stream_destroy(stream)
+            raise
+        cache["hip_stream"] = stream
+    # work enqueued on the null stream before this call is waited for: the capture stream was created blocking
+    binding.graph_launch(cache["hip_exec"], cache["hip_stream"])
+    return None
+
+
+def release_capture(cache):
+    """Drop the recording execute_with_capture keeps in `cache` (its buffers are untouched)."""
+    if "hip_exec" in cache:
+        binding.sync(cache["hip_stream"])
+        binding.graph_destroy(cache.pop("hip_exec"))
+        binding.stream_destroy(cache.pop("hip_stream"))
+    cache.pop("hip_warm", None)
+
+
 class CompiledGraph:
     """Pre-allocated node buffers + a step list (reference src/Compiler.jl:75-100). Calling it copies the
     inputs into their buffers, runs the steps in place and returns the buffer list; nothing is
-    allocated per call. After capture() the step list is one HIP graph launch."""
+    allocated per call. After capture() the steps go through execute_with_capture: one HIP graph launch."""
 
-    def __init__(self, steps, results, workspaces=None):
+    def __init__(self, steps, results, workspaces=None, device=None):
         self.steps = steps
         self.results = results
         self.workspaces = workspaces  # decode scratch owned by this graph: its address never changes
-        self._stream = None
-        self._exec = None
+        self.device = device
+        self.cache = {}
+        self.use_capture = False
+
+    def _run(self, stream):
+        for step in self.steps:
+            step(stream)
 
     def __call__(self, inputs, device=None):
         for k, v in inputs.items():
@@ -525,50 +575,23 @@ class CompiledGraph:
                 binding.memcpy_d2d(self.results[k].ptr, v.ptr, v.nbytes)
             else:
                 self.results[k].copy_from_host(v)
-        if self._exec is not None:
-            # the copies above ran on the null stream, which the capture stream (created blocking) waits for
-            binding.graph_launch(self._exec, self._stream)
+        if self.use_capture:
+            execute_with_capture(self.device, self._run, self.cache)
         else:
-            for step in self.steps:
-                step(None)
+            self._run(None)
+            self.cache["hip_warm"] = True
         return self.results
 
     def capture(self):
-        """Record the step list once into a HIP graph; later calls replay it with one launch. The buffers keep
-        their addresses and per-step values (positions, lengths) are device tensors, so the recording is
-        valid for every later call. Runs the steps once eagerly first (on whatever the buffers hold), so
-        that the library's first-use set-up does not happen inside the capture."""
-        if self._exec is not None:
-            return self
-        for step in self.steps:
-            step(None)
-        binding.sync()
-        stream = binding.stream_create()
-        try:
-            binding.graph_capture_begin(stream)
-            try:
-                for step in self.steps:
-                    step(stream)
-            except Exception:
-                try:
-                    binding.graph_capture_end(stream)  # leave the stream usable; the recording is dropped
-                except binding.LuminalHipError:
-                    pass
-                raise
-            self._exec = binding.graph_capture_end(stream)
-        except Exception:
-            binding.stream_destroy(stream)
-            raise
-        self._stream = stream
+        """From the next call on, run the step list as one recorded HIP graph. Buffer addresses are fixed and
+        per-step values (positions, lengths) are device tensors, so one recording is valid for every call."""
+        self.use_capture = True
         return self
 
     def release(self):
-        """Drop the HIP graph and its stream (the buffers stay)."""
-        if self._exec is not None:
-            binding.sync(self._stream)
-            binding.graph_destroy(self._exec)
-            binding.stream_destroy(self._stream)
-            self._exec = self._stream = None
+        """Back to step-by-step execution; drops the recording and its stream (the buffers stay)."""
+        self.use_capture = False
+        release_capture(self.cache)
 
 
 def compile(graph, device=None):
@@ -592,7 +615,7 @@ def compile(graph, device=None):
         args = [_pick(results, ref) for ref in node.inputs]
         steps.append(lambda stream, out=results[node_id], op=node.op, args=args:
                      execute_op_inplace(out, op, *args, stream=stream, workspaces=workspaces))
-    return CompiledGraph(steps, results, workspaces)
+    return CompiledGraph(steps, results, workspaces, device)
 
 
 # ---------------------------------------------------------------------------------------------
@@ -685,6 +708,6 @@ __all__ = [
     "AbstractDevice", "CPUDevice", "HIPDevice", "HipArray", "get_device", "to_device", "from_device", "Graph",
     "GraphTensor", "tensor", "add_op", "FlashAttentionOp", "DecodeAttentionOp", "flash_attention", "decode_attention",
     "RotaryEmbeddingOp", "KVAppendOp", "rotary_embedding", "kv_cache_append", "self_attention_core",
-    "cached_self_attention_core", "execute_op", "execute_op_inplace", "execute", "compile", "CompiledGraph", "HEADMAP_INTERLEAVED",
+    "cached_self_attention_core", "execute_op", "execute_op_inplace", "execute", "compile", "CompiledGraph", "execute_with_capture", "release_capture", "HEADMAP_INTERLEAVED",
     "HEADMAP_BLOCKED", "LuminalHipError", "apply_rotary_embeddings", "kv_append", "KVCacheState", "encode", "decode", "f32_to_bf16_bits", "bf16_bits_to_f32", "default_scale",
 ]

@@ -103,3 +103,12 @@ def test_self_attention_core_without_rope_is_one_flash_node(lm):
     kinds = [type(x.op).__name__ for x in g.nodes[n + 1:]]
     assert kinds == ["RotaryEmbeddingOp", "RotaryEmbeddingOp", "FlashAttentionOp"]
     assert g.nodes[n + 1].op.prev_seq == 3 and g.nodes[out2.id].op.causal is True
+
+
+def test_execute_with_capture_without_a_hip_device_just_runs(lm):
+    # reference src/Device.jl:121: execute_with_capture(::AbstractDevice, f, cache) = f()
+    calls, cache = [], {}
+    assert lm.execute_with_capture(lm.CPUDevice(), lambda stream: calls.append(stream) or 7, cache) == 7
+    assert calls == [None] and cache == {}
+    lm.release_capture(cache)  # nothing recorded: a no-op
+    assert cache == {}
