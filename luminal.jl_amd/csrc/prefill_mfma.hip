@@ -246,8 +246,8 @@ __global__ __launch_bounds__(256, (D <= 96 ? 3 : 2)) void prefill_mfma_kernel(Pr
   for (int ks = 0; ks < KS; ks++) asm volatile("" :: "v"(qreg[ks]));
 
   for (int kt = 0; kt < n_kv_tiles; kt++) {
-    // One barrier per tile: tile kt (written one iteration ago) becomes visible, and every wave is
-    // done with tile kt-1, whose buffer now takes tile kt+1 from the registers.
+    // One barrier per tile: tile kt (fetched during the previous iteration) becomes visible, and every
+    // wave is done with tile kt-1, whose buffer the fetch of tile kt+1 now overwrites.
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wave's blocks of tile kt are in LDS
     __syncthreads();  // ... and everyone's; tile kt-1 has been consumed, its buffer is free
     if (kt + 1 < n_kv_tiles) load_tile(kt + 1, (kt + 1) & 1);  // in flight while tile kt is computed
