@@ -198,6 +198,18 @@ def test_fp32_large_logits_and_late_maximum(lm, hip, oracle):
         assert rel_err(got, oracle.flash_attn(q, k, v, scale=1.0, causal=causal)) <= 1e-5
 
 
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
+@pytest.mark.parametrize("H,S", [(2, 200), (2, 700), (160, 520)])  # 128-row, key-split, and 128-row workgroups in a full launch
+def test_half_large_logits_and_late_maximum(lm, hip, oracle, dtype, H, S):
+    # as above for the half-precision kernels: P is held against a stale max until a row outgrows it by 2^8
+    q, k, v = inputs(oracle, (1, H, S, 64), (1, H, S, 64), dtype, 7410)
+    k[:, :, -1] = oracle.round_to(k[:, :, -1] * 6.0, dtype)
+    k[:, :, S // 2] = oracle.round_to(k[:, :, S // 2] * 3.0, dtype)
+    for causal in (False, True):
+        got = run_flash(lm, hip, q, k, v, dtype, causal, scale=1.0)
+        assert rel_err(got, oracle.flash_attn(q, k, v, scale=1.0, causal=causal, nthreads=NT)) <= TOL[dtype]
+
+
 @pytest.mark.parametrize("dtype", ["f32", "f16", "bf16"])
 @pytest.mark.parametrize("head_map", [0, 1])
 def test_gqa_prefill_both_head_maps(lm, hip, oracle, dtype, head_map):
