@@ -50,12 +50,13 @@ __global__ __launch_bounds__(256, (KSPLIT > 1 ? 1 : D <= 96 ? 3 : 2)) void prefi
   // the tensors' own head dim a.D may be smaller than the tiled D (any multiple of 8): the missing
   // columns are never fetched (zeros in Q, K and V) and never stored.
   const int cpr = a.D / 4;
-  constexpr int CH = BT * CPR / 256;  // chunks per thread per tile
   constexpr int LDK = D + kPadK;    // LDS row strides in floats
   constexpr int LDV = D + kPadV;
 
-  __shared__ __attribute__((aligned(16))) float Ks2[2][BT * LDK];  // double-buffered tiles
-  __shared__ __attribute__((aligned(16))) float Vs2[2][BT * LDV];
+  constexpr int KC = LDK / 4, VC = LDV / 4;                            // 16-byte chunks per LDS row
+  constexpr int KI = (BT * KC + 63) / 64, VI = (BT * VC + 63) / 64;  // 1 KB blocks per tile (the last may be half used)
+  __shared__ __attribute__((aligned(16))) float Ks2[2][KI * 256];     // double-buffered tiles, whole blocks
+  __shared__ __attribute__((aligned(16))) float Vs2[2][VI * 256];
 
   // ---- which (b, hq, query tile) this workgroup owns: see prefill_mfma.hip ----
   const int bid = blockIdx.x;
@@ -105,55 +106,72 @@ __global__ __launch_bounds__(256, (KSPLIT > 1 ? 1 : D <= 96 ? 3 : 2)) void prefi
   float l_i = 0.f;        // this lane's half of the running sum
   const float c = a.scale * kLog2e;
 
-  // ---- tile staging: global -> registers (prefetched two tiles ahead) -> LDS; rows past n_keys read as
-  // zero through the buffer descriptor's bounds ----
-  const __amdgpu_buffer_rsrc_t k_rsrc =
-      __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(kp), 0, (int)((int64_t)n_keys * a.ks[2] * 4), 0x00020000);
-  const __amdgpu_buffer_rsrc_t v_rsrc =
-      __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(vp), 0, (int)((int64_t)n_keys * a.vs[2] * 4), 0x00020000);
-  int k_voff[CH], v_voff[CH], k_lds_off[CH], v_lds_off[CH];
+  // ---- tile staging: global memory -> LDS directly (buffer_load_dwordx4 ... lds), one tile ahead; see
+  // prefill_mfma.hip. A wave-wide load fills a 1 KB block, lane l's 16 bytes at block + 16 l from that lane's
+  // own global offset; lanes on a padding chunk, past the tile's last row or past the tensors' head dim fetch
+  // out of range (zeros), rows past n_keys read as zero through the descriptor's bounds. ----
+  typedef int32_t i32x4_t __attribute__((ext_vector_type(4)));
+  typedef __attribute__((address_space(3))) void lds_void_t;
+  constexpr int KBW = (KI + 3) / 4, VBW = (VI + 3) / 4;  // blocks per wave (rounded up)
+  const int wave_u = __builtin_amdgcn_readfirstlane(wave);
+  __builtin_assume(wave_u >= 0 && wave_u < 4);
+  auto make_desc = [](const float *base, int bytes) {
+    const uint64_t p = (uint64_t)base;
+    i32x4_t d;
+    d[0] = __builtin_amdgcn_readfirstlane((int)(uint32_t)p);
+    d[1] = __builtin_amdgcn_readfirstlane((int)((p >> 32) & 0xffff));  // stride 0: raw buffer
+    d[2] = __builtin_amdgcn_readfirstlane(bytes);
+    d[3] = 0x00020000;
+    return d;
+  };
+  const i32x4_t k_desc = make_desc(kp, (int)((int64_t)n_keys * a.ks[2] * 4));
+  const i32x4_t v_desc = make_desc(vp, (int)((int64_t)n_keys * a.vs[2] * 4));
+  int k_voff[KBW], v_voff[VBW];
 #pragma unroll
-  for (int r = 0; r < CH; r++) {
-    const int id = tid + 256 * r;
-    const int row = id / CPR, col = id % CPR;
-    k_voff[r] = col < cpr ? (int)((row * a.ks[2] + col * 4) * 4) : kOutOfRange;
-    v_voff[r] = col < cpr ? (int)((row * a.vs[2] + col * 4) * 4) : kOutOfRange;
-    k_lds_off[r] = row * LDK + col * 4;
-    v_lds_off[r] = row * LDV + col * 4;
+  for (int j = 0; j < KBW; j++) {
+    const int ch = (wave + 4 * j) * 64 + lane;
+    const int row = ch / KC, col = ch % KC;
+    k_voff[j] = (row < BT && col < cpr) ? (int)((row * a.ks[2] + col * 4) * 4) : kOutOfRange;
+  }
+#pragma unroll
+  for (int j = 0; j < VBW; j++) {
+    const int ch = (wave + 4 * j) * 64 + lane;
+    const int row = ch / VC, col = ch % VC;
+    v_voff[j] = (row < BT && col < cpr) ? (int)((row * a.vs[2] + col * 4) * 4) : kOutOfRange;
   }
   const int k_tile_bytes = (int)(BT * a.ks[2] * 4), v_tile_bytes = (int)(BT * a.vs[2] * 4);
-  typedef unsigned int u32x4_t __attribute__((ext_vector_type(4)));
-  u32x4_t kreg[CH], vreg[CH];
-  auto load_tile = [&](int kt) {
-#pragma unroll
-    for (int r = 0; r < CH; r++) {
-      kreg[r] = __builtin_amdgcn_raw_buffer_load_b128(k_rsrc, k_voff[r], kt * k_tile_bytes, 0);
-      vreg[r] = __builtin_amdgcn_raw_buffer_load_b128(v_rsrc, v_voff[r], kt * v_tile_bytes, 0);
-    }
+  const uint32_t k_lds0 = (uint32_t)(uintptr_t)(lds_void_t *)&Ks2[0][0] + wave_u * 1024;
+  const uint32_t v_lds0 = (uint32_t)(uintptr_t)(lds_void_t *)&Vs2[0][0] + wave_u * 1024;
+#pragma clang diagnostic push
+#pragma clang diagnostic ignored "-Winline-asm"  // m0 is a reserved register; it is only written here
+  auto load_block = [](i32x4_t desc, uint32_t lds_addr, int voff, int soff) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
+                 :: "s"(lds_addr), "v"(voff), "s"(desc), "s"(soff) : "memory", "m0");
   };
-  auto store_tile = [&](int buf) {
+#pragma clang diagnostic pop
+  auto load_tile = [&](int kt, int buf) {
 #pragma unroll
-    for (int r = 0; r < CH; r++) {
-      *reinterpret_cast<u32x4_t *>(&Ks2[buf][k_lds_off[r]]) = kreg[r];
-      *reinterpret_cast<u32x4_t *>(&Vs2[buf][v_lds_off[r]]) = vreg[r];
-    }
+    for (int j = 0; j < KBW; j++)
+      if (wave_u + 4 * j < KI) load_block(k_desc, k_lds0 + buf * (KI * 1024) + j * 4096, k_voff[j], kt * k_tile_bytes);
+#pragma unroll
+    for (int j = 0; j < VBW; j++)
+      if (wave_u + 4 * j < VI) load_block(v_desc, v_lds0 + buf * (VI * 1024) + j * 4096, v_voff[j], kt * v_tile_bytes);
   };
 
   const int k_frag_off = n * LDK + 4 * g;  // + 8 * j
   const int v_frag_off = 4 * g * LDV + n;  // + (8 * (i / 4) + i % 4) * LDV + 32 * db
 
-  if (n_kv_tiles > 0) {
-    load_tile(0);
-    store_tile(0);
-  }
-  if (n_kv_tiles > 1) load_tile(1);
+  if (n_kv_tiles > 0) load_tile(0, 0);
+  // The compiler does not model the asm loads or the asm wait below: make it wait for Q here, not inside the loop.
+#pragma unroll
+  for (int j = 0; j < KJ; j++) asm volatile("" :: "v"(qf[j]));
 
   for (int kt = 0; kt < n_kv_tiles; kt++) {
-    // One barrier per tile: tile kt (written one iteration ago) becomes visible, and every wave is
-    // done with tile kt-1, whose buffer now takes tile kt+1 from the registers.
+    // One barrier per tile: tile kt (fetched during the previous iteration) becomes visible, and every
+    // wave is done with tile kt-1, whose buffer the fetch of tile kt+1 now overwrites.
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wave's blocks of tile kt are in LDS
     __syncthreads();
-    if (kt + 1 < n_kv_tiles) store_tile((kt + 1) & 1);
-    if (kt + 2 < n_kv_tiles) load_tile(kt + 2);
+    if (kt + 1 < n_kv_tiles) load_tile(kt + 1, (kt + 1) & 1);
     const float *Ks = Ks2[kt & 1] + kg * (BN * LDK);
     const float *Vs = Vs2[kt & 1] + kg * (BN * LDV);
 
