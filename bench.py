@@ -335,13 +335,24 @@ def other_configs(lm, dev, check=False):
         log("[other] %s: %.1f us, %.0f GB/s" % (name, ev * 1e3, res[name]["GB/s"]))
 
     B, H, S, D = 1, 32, 4096, 96
-    x = lm.HipArray((B, H, S, D), "f16", dev).copy_from_host(rng.standard_normal((B, H, S, D), dtype=np.float32))
+    # 12 inputs of 25 MB in rotation, more than the 256 MB last-level cache holds: every launch reads from HBM
+    xs = [lm.HipArray((B, H, S, D), "f16", dev).copy_from_host(rng.standard_normal((B, H, S, D), dtype=np.float32)) for _ in range(12)]
     y = lm.HipArray((B, H, S, D), "f16", dev)
-    rp = lm.binding.RopeParams()
-    rp.out, rp.x, rp.pos0, rp.prev_seq = y.ptr, x.ptr, None, 0
-    rp.B, rp.H, rp.S, rp.D = B, H, S, D
-    rp.dtype, rp.base, rp.pairing, rp.stream = lm.binding.DTYPE_CODES["f16"], 10000.0, lm.binding.ROPE_HALF_SPLIT, None
-    hbm_line("rotary embedding fp16 B=1 H=32 S=4096 D=96 (C2's Q)", lambda: lm.binding.rope(rp), 2.0 * B * H * S * D * 2)
+    rps = []
+    for x in xs:
+        rp = lm.binding.RopeParams()
+        rp.out, rp.x, rp.pos0, rp.prev_seq = y.ptr, x.ptr, None, 0
+        rp.B, rp.H, rp.S, rp.D = B, H, S, D
+        rp.dtype, rp.base, rp.pairing, rp.stream = lm.binding.DTYPE_CODES["f16"], 10000.0, lm.binding.ROPE_HALF_SPLIT, None
+        rps.append(rp)
+    rstate = {"i": 0}
+
+    def rope_step():
+        lm.binding.rope(rps[rstate["i"] % len(rps)])
+        rstate["i"] += 1
+
+    hbm_line("rotary embedding fp16 B=1 H=32 S=4096 D=96 (C2's Q, 12 inputs rotated)", rope_step, 2.0 * B * H * S * D * 2, n=36)
+    del xs
 
     for T, label in ((4096, "whole prompt T=4096"), (1, "one decode step T=1")):
         B, Hkv, L, D = 16, 8, 4096, 128

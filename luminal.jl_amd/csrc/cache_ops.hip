@@ -185,9 +185,9 @@ __global__ __launch_bounds__(256) void kv_append_vec_kernel(KvAppendArgs a) {
   raw *vc = reinterpret_cast<raw *>(a.v_cache) + b * a.vs[0] + h * a.vs[1] + (int64_t)row * a.vs[2];
   const int d0 = c * V, d1 = half + c * V;
   Chunk<E> k0, k1;
-  k0.u = *reinterpret_cast<const uint4 *>(kn + d0);
-  k1.u = *reinterpret_cast<const uint4 *>(kn + d1);
-  const uint4 v0 = *reinterpret_cast<const uint4 *>(vn + d0), v1 = *reinterpret_cast<const uint4 *>(vn + d1);
+  k0.u = load_stream_128(kn + d0);
+  k1.u = load_stream_128(kn + d1);
+  const uint4 v0 = load_stream_128(vn + d0), v1 = load_stream_128(vn + d1);
   if (a.rope_k) {
     float sn[V], cs[V];
     if (a.interleaved) {

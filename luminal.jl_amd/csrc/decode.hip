@@ -175,7 +175,7 @@ __global__ __launch_bounds__(kWaves * 64) void decode_split_kernel(DecodeArgs a,
       const int key = it0 + (wave * kUnroll + u) * KPW + slot;
       valid[u] = key < end;
       if (valid[u] && lane_active) {
-        kr[u].load(kbase + (int64_t)key * a.ks[2]);
+        kr[u].load_stream(kbase + (int64_t)key * a.ks[2]);
       } else {
         kr[u].zero();
       }
@@ -184,7 +184,7 @@ __global__ __launch_bounds__(kWaves * 64) void decode_split_kernel(DecodeArgs a,
     for (int u = 0; u < kUnroll; u++) {
       const int key = it0 + (wave * kUnroll + u) * KPW + slot;
       if (valid[u] && lane_active) {
-        vr[u].load(vbase + (int64_t)key * a.vs[2]);
+        vr[u].load_stream(vbase + (int64_t)key * a.vs[2]);
       } else {
         vr[u].zero();
       }

@@ -173,8 +173,8 @@ __global__ __launch_bounds__(kWaves * 64) void decode_mfma_kernel(DecodeArgs a, 
       kreg[r] = make_uint4(0, 0, 0, 0);
       vreg[r] = make_uint4(0, 0, 0, 0);
       if (key < end) {
-        kreg[r] = *reinterpret_cast<const uint4 *>(kbase + (int64_t)key * a.ks[2] + col * 8);
-        vreg[r] = *reinterpret_cast<const uint4 *>(vbase + (int64_t)key * a.vs[2] + col * 8);
+        kreg[r] = load_stream_128(kbase + (int64_t)key * a.ks[2] + col * 8);
+        vreg[r] = load_stream_128(vbase + (int64_t)key * a.vs[2] + col * 8);
       }
     }
   };
