@@ -353,6 +353,34 @@ def test_decode_equals_last_row_of_causal_prefill_on_gpu(lm, hip, oracle):
     assert rel_err(dec, full[:, :, L - 1]) <= 4e-3  # two results, each within 2e-3 of the oracle
 
 
+def test_decode_alternating_batches_on_one_workspace_repeat_bitwise(lm, hip, oracle):
+    """Two different ragged batches alternate on the one split-KV workspace, 12 times each: a merge that picked
+    up a partial of the other batch (one call earlier) or an unset slot would not reproduce the first result bit
+    for bit."""
+    B, Hq, Hkv, L, D = 24, 32, 8, 2048, 128
+    lens = (np.arange(B) * 83 % L + 1).astype(np.int32)  # 1 .. L, ragged
+    sets = []
+    for seed in (9700, 9710):
+        q = oracle.round_to(oracle.gen_normal((B, Hq, D), seed), "bf16")
+        kc = oracle.round_to(oracle.gen_normal((B, Hkv, L, D), seed + 1), "bf16")
+        vc = oracle.round_to(oracle.gen_normal((B, Hkv, L, D), seed + 2), "bf16")
+        want = oracle.decode_attn(q, kc, vc, kv_len=lens, nthreads=NT)
+        sets.append((tuple(lm.to_device(x, hip, "bf16") for x in (q, kc, vc)), want))
+    dl = lm.to_device(lens, hip)
+    op = lm.DecodeAttentionOp(lm.default_scale(D), 0, 16)  # 16 splits of 128 keys
+    first = [None, None]
+    for rep in range(12):
+        for i, ((dq, dk, dv), want) in enumerate(sets):
+            out = lm.HipArray((B, Hq, D), "f32", hip)
+            lm.host.execute_op_inplace(out, op, dq, dk, dv, dl)
+            got = out.to_host()
+            if first[i] is None:
+                first[i] = got
+                assert rel_err(got, want) <= TOL["bf16"]
+            else:
+                assert np.array_equal(got, first[i]), (rep, i)
+
+
 def test_decode_without_kv_len_and_poisoned_tail(lm, hip, oracle):
     B, Hq, Hkv, L, D = 2, 8, 2, 1000, 128
     q, k, v = inputs(oracle, (B, Hq, D), (B, Hkv, L, D), "bf16", 7900)
