@@ -431,7 +431,7 @@ def main():
     log("[bench] device:", lm.binding.device_name())
 
     line = {
-        "metric": "attention TFLOP/s (prefill) + KV-read GB/s (decode), % roofline, 1xMI355X",
+        "metric": "attention TFLOP/s (prefill) + KV-read GB/s (decode), % roofline, 1×MI355X",
         "value": None, "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": None, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f16",
         "data": "synthetic",
