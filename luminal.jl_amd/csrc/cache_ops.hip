@@ -161,49 +161,59 @@ __global__ __launch_bounds__(256) void rope_vec_kernel(RopeArgs a, int heads_per
   }
 }
 
-// Cache append, 16-byte chunks: a thread moves chunk c of each half of one new K row and one new V row
-// (D is a multiple of 2 V), rotating K on the way when asked to.
+// Cache append, 16-byte chunks: a thread owns chunk c of each half of the new rows at (b, t) and walks the KV
+// heads of its block (D is a multiple of 2 V), rotating K on the way when asked to. The angle depends on the row
+// position and the pair, not on the head, so the sin / cos are evaluated once per thread (they were 17 % of a
+// whole-prompt append when every (b, head, t) thread evaluated its own). grid.x covers (b, t, chunk), grid.y
+// blocks of heads.
 template <typename E>
-__global__ __launch_bounds__(256) void kv_append_vec_kernel(KvAppendArgs a) {
+__global__ __launch_bounds__(256) void kv_append_vec_kernel(KvAppendArgs a, int heads_per_block) {
   using raw = typename E::raw;
   constexpr int V = E::kVec;
   const int half = a.D / 2;
   const int cpr = half / V;
-  const int64_t total = (int64_t)a.B * a.Hkv * a.T * cpr;
+  const int64_t total = (int64_t)a.B * a.T * cpr;
   const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (idx >= total) return;
   const int c = (int)(idx % cpr);
   const int t = (int)((idx / cpr) % a.T);
-  const int h = (int)((idx / ((int64_t)cpr * a.T)) % a.Hkv);
-  const int b = (int)(idx / ((int64_t)cpr * a.T * a.Hkv));
+  const int b = (int)(idx / ((int64_t)cpr * a.T));
   const int row = (a.pos ? a.pos[b] : a.pos_all) + t;
   if (row < 0 || row >= a.Lmax) return;  // a full cache drops the row instead of writing out of bounds
-  const int64_t src = (((int64_t)b * a.Hkv + h) * a.T + t) * a.D;
-  const raw *kn = reinterpret_cast<const raw *>(a.k_new) + src;
-  const raw *vn = reinterpret_cast<const raw *>(a.v_new) + src;
-  raw *kc = reinterpret_cast<raw *>(a.k_cache) + b * a.ks[0] + h * a.ks[1] + (int64_t)row * a.ks[2];
-  raw *vc = reinterpret_cast<raw *>(a.v_cache) + b * a.vs[0] + h * a.vs[1] + (int64_t)row * a.vs[2];
   const int d0 = c * V, d1 = half + c * V;
-  Chunk<E> k0, k1;
-  k0.u = load_stream_128(kn + d0);
-  k1.u = load_stream_128(kn + d1);
-  const uint4 v0 = load_stream_128(vn + d0), v1 = load_stream_128(vn + d1);
+  float sn0[V], cs0[V], sn1[V / 2], cs1[V / 2];
   if (a.rope_k) {
-    float sn[V], cs[V];
     if (a.interleaved) {
-      sincos_pairs<E>((float)row, d0 / 2, V / 2, a.D, a.log2_base, sn, cs);
-      rotate_interleaved<E>(k0, sn, cs);
-      sincos_pairs<E>((float)row, d1 / 2, V / 2, a.D, a.log2_base, sn, cs);
-      rotate_interleaved<E>(k1, sn, cs);
+      sincos_pairs<E>((float)row, d0 / 2, V / 2, a.D, a.log2_base, sn0, cs0);
+      sincos_pairs<E>((float)row, d1 / 2, V / 2, a.D, a.log2_base, sn1, cs1);
     } else {
-      sincos_pairs<E>((float)row, d0, V, a.D, a.log2_base, sn, cs);
-      rotate_chunks<E>(k0, k1, sn, cs);
+      sincos_pairs<E>((float)row, d0, V, a.D, a.log2_base, sn0, cs0);
     }
   }
-  *reinterpret_cast<uint4 *>(kc + d0) = k0.u;
-  *reinterpret_cast<uint4 *>(kc + d1) = k1.u;
-  *reinterpret_cast<uint4 *>(vc + d0) = v0;
-  *reinterpret_cast<uint4 *>(vc + d1) = v1;
+  const int h0 = blockIdx.y * heads_per_block, h1 = min(a.Hkv, h0 + heads_per_block);
+  for (int h = h0; h < h1; h++) {
+    const int64_t src = (((int64_t)b * a.Hkv + h) * a.T + t) * a.D;
+    const raw *kn = reinterpret_cast<const raw *>(a.k_new) + src;
+    const raw *vn = reinterpret_cast<const raw *>(a.v_new) + src;
+    raw *kc = reinterpret_cast<raw *>(a.k_cache) + b * a.ks[0] + h * a.ks[1] + (int64_t)row * a.ks[2];
+    raw *vc = reinterpret_cast<raw *>(a.v_cache) + b * a.vs[0] + h * a.vs[1] + (int64_t)row * a.vs[2];
+    Chunk<E> k0, k1;
+    k0.u = load_stream_128(kn + d0);
+    k1.u = load_stream_128(kn + d1);
+    const uint4 v0 = load_stream_128(vn + d0), v1 = load_stream_128(vn + d1);
+    if (a.rope_k) {
+      if (a.interleaved) {
+        rotate_interleaved<E>(k0, sn0, cs0);
+        rotate_interleaved<E>(k1, sn1, cs1);
+      } else {
+        rotate_chunks<E>(k0, k1, sn0, cs0);
+      }
+    }
+    *reinterpret_cast<uint4 *>(kc + d0) = k0.u;
+    *reinterpret_cast<uint4 *>(kc + d1) = k1.u;
+    *reinterpret_cast<uint4 *>(vc + d0) = v0;
+    *reinterpret_cast<uint4 *>(vc + d1) = v1;
+  }
 }
 
 bool chunks_ok(const void *p0, const void *p1, const int64_t *s0, const int64_t *s1, int vec) {
@@ -265,15 +275,21 @@ int launch_rope(const RopeArgs &a, int dtype, hipStream_t stream) {
 
 int launch_kv_append(const KvAppendArgs &a, int dtype, hipStream_t stream) {
   const int vec = dtype == LMH_F32 ? 4 : 8;
-  const int64_t vec_blocks = ((int64_t)a.B * a.Hkv * a.T * (a.D / (2 * vec)) + 255) / 256;
+  const int64_t vec_chunks = (int64_t)a.B * a.Hkv * a.T * (a.D / (2 * vec));  // 16-byte chunk pairs to move
+  const int64_t blocks_x = ((int64_t)a.B * a.T * (a.D / (2 * vec)) + 255) / 256;
   if (a.D % (2 * vec) == 0 && chunks_ok(a.k_cache, a.v_cache, a.ks, a.vs, vec) &&
       ((reinterpret_cast<uintptr_t>(a.k_new) | reinterpret_cast<uintptr_t>(a.v_new)) & 15u) == 0 &&
-      vec_blocks >= 64 && vec_blocks < (int64_t(1) << 31)) {  // a decode step's few rows: one element per thread is quicker
-    dim3 grid((unsigned)vec_blocks), block(256);
+      vec_chunks >= 64 * 256 && blocks_x < (int64_t(1) << 31) && a.Hkv <= 65535) {  // a decode step's few rows: one element per thread is quicker
+    // about 2048 workgroups keep enough loads in flight; beyond that a thread walks more heads with one set of sin / cos
+    int blocks_y = (int)((2048 + blocks_x - 1) / blocks_x);
+    blocks_y = blocks_y < 1 ? 1 : (blocks_y > a.Hkv ? a.Hkv : blocks_y);
+    const int heads_per_block = (a.Hkv + blocks_y - 1) / blocks_y;
+    blocks_y = (a.Hkv + heads_per_block - 1) / heads_per_block;
+    dim3 grid((unsigned)blocks_x, (unsigned)blocks_y), block(256);
     switch (dtype) {
-      case LMH_F32: hipLaunchKernelGGL(kv_append_vec_kernel<F32>, grid, block, 0, stream, a); break;
-      case LMH_F16: hipLaunchKernelGGL(kv_append_vec_kernel<F16>, grid, block, 0, stream, a); break;
-      case LMH_BF16: hipLaunchKernelGGL(kv_append_vec_kernel<BF16>, grid, block, 0, stream, a); break;
+      case LMH_F32: hipLaunchKernelGGL(kv_append_vec_kernel<F32>, grid, block, 0, stream, a, heads_per_block); break;
+      case LMH_F16: hipLaunchKernelGGL(kv_append_vec_kernel<F16>, grid, block, 0, stream, a, heads_per_block); break;
+      case LMH_BF16: hipLaunchKernelGGL(kv_append_vec_kernel<BF16>, grid, block, 0, stream, a, heads_per_block); break;
       default: return fail(LMH_E_UNSUPPORTED, "kv append: unknown dtype %d", dtype);
     }
     LMH_HIP_TRY(hipGetLastError());
