@@ -45,9 +45,25 @@ def log(*a):
     print(*a, file=sys.stderr, flush=True)
 
 
-def time_steps(fn, steps, warmup, binding):
-    """warmup untimed calls, then `steps` timed calls bracketed by a device sync on both sides.
-    Returns (wall ms per step, HIP-event ms per step)."""
+# The GPU raises its clocks over the first tens of milliseconds of load: from idle, C2 measured 141 us per launch
+# over the first 20 launches and 118 us from the 100th on. Every timed region is therefore preceded by this much
+# untimed work of the same kind (on top of the --warmup steps), so that what is timed is the steady state.
+CLOCK_SETTLE_MS = 100.0
+
+
+def settle_clocks(fn, binding, ms=CLOCK_SETTLE_MS):
+    t0 = time.perf_counter()
+    while (time.perf_counter() - t0) * 1e3 < ms:
+        for _ in range(8):
+            fn()
+        binding.sync()
+
+
+def time_steps(fn, steps, warmup, binding, settle_ms=CLOCK_SETTLE_MS):
+    """Clock settling, `warmup` untimed calls, then `steps` timed calls bracketed by a device sync on both
+    sides. Returns (wall ms per step, HIP-event ms per step)."""
+    if settle_ms > 0:
+        settle_clocks(fn, binding, settle_ms)
     for _ in range(warmup):
         fn()
     binding.sync()
@@ -434,7 +450,7 @@ def main():
         "metric": "attention TFLOP/s (prefill) + KV-read GB/s (decode), % roofline, 1×MI355X",
         "value": None, "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": None, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f16",
-        "data": "synthetic",
+        "data": "synthetic", "clock_settle_ms": CLOCK_SETTLE_MS,
         "config": {"workload": "C2 Phi-3-mini causal prefill attention: B=1 Hq=Hkv=32 S=4096 D=96, fp16 in/out, fp32 accumulate, scale 1/sqrt(96)"},
     }
     if args.only == "copy":
