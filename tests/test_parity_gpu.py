@@ -666,6 +666,49 @@ def test_decode_batch_above_the_persistent_kernel_limit(lm, hip, oracle):
     assert rel_err(got, oracle.decode_attn(q[:1024], k[:1024], v[:1024], kv_len=lens[:1024], nthreads=NT)) <= 2e-3
 
 
+@pytest.mark.parametrize("dtype", ["f32", "f16", "bf16"])
+def test_sequence_four_times_the_longest_benchmark_checked_through_properties(lm, hip, oracle, dtype):
+    """S = 16384, causal, D = 128: too long for the scalar oracle on every row, so the result is checked through what
+    does not depend on the size: rows below n depend on the first n keys only (oracle on that prefix), single rows
+    anywhere against float64 numpy, and a constant V comes back as that constant."""
+    B, H, S, D = 1, 4, 16384, 128
+    q, k, v = inputs(oracle, (B, H, S, D), (B, H, S, D), dtype, 9650, mul=0.7)
+    got = run_flash(lm, hip, q, k, v, dtype, True)
+    n = 1024
+    want = oracle.flash_attn(q[:, :, :n], k[:, :, :n], v[:, :, :n], causal=True, nthreads=NT)
+    assert rel_err(got[:, :, :n], want) <= TOL[dtype]
+    scale = 1.0 / np.sqrt(D)
+    rows = [n, 4095, 4096, 8191, 12345, S - 129, S - 128, S - 1]
+    want = np.empty((B, H, len(rows), D))
+    for r, i in enumerate(rows):
+        s = np.einsum("bhkd,bhd->bhk", k[:, :, :i + 1].astype(np.float64), q[:, :, i].astype(np.float64)) * scale
+        w = np.exp(s - s.max(-1, keepdims=True))
+        want[:, :, r] = np.einsum("bhk,bhkd->bhd", w, v[:, :, :i + 1].astype(np.float64)) / w.sum(-1)[..., None]
+    assert rel_err(got[:, :, rows], want) <= TOL[dtype]
+    const = np.full_like(v, 0.75)
+    got = run_flash(lm, hip, q, k, const, dtype, True)
+    # fp32: sum and weighted sum each carry ~sqrt(S) * 2^-24 of rounding, as the oracle's own fp32 loop would
+    assert np.abs(got - 0.75).max() <= (1e-5 if dtype == "f32" else 1e-3)
+
+
+def test_decode_over_a_cache_four_times_the_longest_benchmark_sequence(lm, hip, oracle):
+    """kv_len = 131072 (and one short neighbour in the same batch), bf16, GQA 4: float64 numpy on every head."""
+    B, Hq, Hkv, L, D = 2, 32, 8, 131072, 128
+    q, k, v = inputs(oracle, (B, Hq, D), (B, Hkv, L, D), "bf16", 9660)
+    lens = np.array([L, 777], np.int32)
+    got = run_decode(lm, hip, q, k, v, "bf16", kv_len=lens)
+    want = np.empty((B, Hq, D))
+    for b in range(B):
+        for hq in range(Hq):
+            kk, vv = k[b, hq % Hkv, :lens[b]].astype(np.float64), v[b, hq % Hkv, :lens[b]].astype(np.float64)
+            s = kk @ q[b, hq].astype(np.float64) / np.sqrt(D)
+            w = np.exp(s - s.max())
+            want[b, hq] = w @ vv / w.sum()
+    assert rel_err(got, want) <= 2e-3
+    for b in range(B):  # each sequence on its own scale: the long one averages 131072 rows, the short one 777
+        assert rel_err(got[b], want[b]) <= 2e-3
+
+
 def _padded(lm, hip, x, dtype, row_pad, rng):
     """Upload x (B,H,S,D) into a buffer whose rows are D + row_pad apart (padding filled with NaN);
     returns (array, element strides (b, h, s))."""
