@@ -6,6 +6,7 @@
 #   * to_device / from_device methods                                  (src/Device.jl:82-105)
 #   * execute_op / execute_op! methods for FlashAttentionOp on HipArray arguments; multiple
 #     dispatch prefers them over the generic method at src/Execution.jl:565-578
+#   * an execute_with_capture method that records a step into a HIP graph     (src/Device.jl:108-121)
 #   * DecodeAttentionOp + decode_attention, the fused form of the cached single-token attention
 #     subgraph (src/Whisper.jl:584-620) with the GQA head sharing of src/NN.jl:305-317
 # and calls the C ABI of include/luminal_hip.h through `ccall`. There are no AMDGPU.jl kernels here.
@@ -17,7 +18,7 @@ module LuminalHIP
 
 using Luminal
 import Luminal: AbstractDevice, Op, FlashAttentionOp, GraphTensor, add_op!, realized_dims,
-                to_device, from_device, execute_op, execute_op!
+                to_device, from_device, execute_op, execute_op!, execute_with_capture
 
 const libluminal_hip = get(ENV, "LUMINAL_HIP_LIB", joinpath(@__DIR__, "..", "lib", "libluminal_hip.so"))
 
@@ -112,6 +113,10 @@ struct DecodeParams
     stream::Ptr{Cvoid}
 end
 
+# The stream every executor below enqueues on: the null stream, except while execute_with_capture records.
+const _stream = Ref{Ptr{Cvoid}}(C_NULL)
+current_stream() = _stream[]
+
 const Z3 = (Int64(0), Int64(0), Int64(0))   # all-zero strides = contiguous
 const Z2 = (Int64(0), Int64(0))
 
@@ -124,7 +129,7 @@ function execute_op!(out::HipArray{TO,4}, op::FlashAttentionOp, q::HipArray{T,4}
     _, Hkv, Sk, _ = size(k)
     size(out) == size(q) || error("FlashAttentionOp: output shape $(size(out)) differs from q shape $(size(q))")
     p = Ref(AttnParams(out.ptr, q.ptr, k.ptr, v.ptr, C_NULL, B, Hq, Hkv, Sq, Sk, D, Z3, Z3, Z3, Z3,
-                       dtype_code(T), op.scale, Int32(op.causal), head_map, Int32(TO === Float32 && T !== Float32), C_NULL))
+                       dtype_code(T), op.scale, Int32(op.causal), head_map, Int32(TO === Float32 && T !== Float32), current_stream()))
     check(ccall((:lmh_flash_attn_fwd, libluminal_hip), Cint, (Ref{AttnParams},), p))
     return out
 end
@@ -173,7 +178,7 @@ function execute_op!(out::HipArray{TO,3}, op::DecodeAttentionOp, q::HipArray{T,3
     ws = workspace(need)
     p = Ref(DecodeParams(out.ptr, q.ptr, kc.ptr, vc.ptr, Ptr{Int32}(kv_len.ptr), B, Hq, Hkv, Lmax, D, Z2, Z2, Z3, Z3,
                          dtype_code(T), op.scale, op.head_map, Int32(TO === Float32 && T !== Float32), splits,
-                         ws === nothing ? C_NULL : ws.ptr, need, C_NULL))
+                         ws === nothing ? C_NULL : ws.ptr, need, current_stream()))
     check(ccall((:lmh_decode_attn, libluminal_hip), Cint, (Ref{DecodeParams},), p))
     return out
 end
@@ -197,7 +202,7 @@ function rope!(x::HipArray{T,4}; prev_seq::Integer=0, base::Real=10000.0f0,
                pos0::Union{Nothing,HipArray{Int32,1}}=nothing) where {T}
     B, H, S, D = size(x)
     p = Ref(RopeParams(x.ptr, x.ptr, pos0 === nothing ? Ptr{Int32}(C_NULL) : Ptr{Int32}(pos0.ptr), prev_seq, B, H, S, D,
-                       Z3, Z3, dtype_code(T), Float32(base), Int32(0), C_NULL))
+                       Z3, Z3, dtype_code(T), Float32(base), Int32(0), current_stream()))
     check(ccall((:lmh_rope, libluminal_hip), Cint, (Ref{RopeParams},), p))
     return x
 end
@@ -215,7 +220,7 @@ function kv_append!(kc::HipArray{T,4}, vc::HipArray{T,4}, k_new::HipArray{T,4}, 
                     pos::HipArray{Int32,1}; rope_k::Bool=false, base::Real=10000.0f0) where {T}
     B, Hkv, Lmax, D = size(kc)
     p = Ref(KvAppendParams(kc.ptr, vc.ptr, k_new.ptr, v_new.ptr, Ptr{Int32}(pos.ptr), 0, B, Hkv, size(k_new, 3), D, Lmax,
-                           Z3, Z3, dtype_code(T), Int32(rope_k), Int32(0), Float32(base), C_NULL))
+                           Z3, Z3, dtype_code(T), Int32(rope_k), Int32(0), Float32(base), current_stream()))
     check(ccall((:lmh_kv_append, libluminal_hip), Cint, (Ref{KvAppendParams},), p))
     return kc, vc
 end
@@ -256,7 +261,64 @@ function cached_self_attention_core!(out::HipArray{TO,3}, q::HipArray{T,4}, k_ne
     return execute_op!(out, DecodeAttentionOp(s, head_map), q3, kc, vc, kv_len)
 end
 
-export HIPDevice, HipArray, DecodeAttentionOp, decode_attention, get_device, functional, rope!, kv_append!,
+# ------------------------------------------------------------------------------------------
+# execute_with_capture(device, f, cache) (src/Device.jl:108-121; called by the compiled step closure,
+# src/Compiler.jl:98). The reference stubs its CUDA method out because transient workspaces freed after
+# the recording invalidated it. Here every buffer a step touches outlives the recording (the caches and
+# results belong to the compiled graph, the split-KV workspace to this module and it only grows before
+# the recording: the first call runs eagerly), and positions / lengths are device tensors, so one
+# recording serves every decode position. Every call runs f's work exactly once.
+# `f` must enqueue only through the executors of this module and must not upload or download.
+# ------------------------------------------------------------------------------------------
+function execute_with_capture(::HIPDevice, f, cache::Dict)
+    if !haskey(cache, :hip_exec)
+        if !get(cache, :hip_warm, false)
+            cache[:hip_warm] = true
+            return f()                       # first use: allocations and set-up stay outside the recording
+        end
+        check(ccall((:lmh_sync, libluminal_hip), Cint, (Ptr{Cvoid},), C_NULL))
+        sref = Ref{Ptr{Cvoid}}(C_NULL)
+        check(ccall((:lmh_stream_create, libluminal_hip), Cint, (Ref{Ptr{Cvoid}},), sref))
+        gref = Ref{Ptr{Cvoid}}(C_NULL)
+        check(ccall((:lmh_graph_capture_begin, libluminal_hip), Cint, (Ptr{Cvoid},), sref[]))
+        _stream[] = sref[]
+        try
+            f()
+        catch
+            _stream[] = C_NULL
+            ccall((:lmh_graph_capture_end, libluminal_hip), Cint, (Ptr{Cvoid}, Ref{Ptr{Cvoid}}), sref[], gref)
+            gref[] == C_NULL || ccall((:lmh_graph_destroy, libluminal_hip), Cint, (Ptr{Cvoid},), gref[])
+            ccall((:lmh_stream_destroy, libluminal_hip), Cint, (Ptr{Cvoid},), sref[])
+            rethrow()
+        end
+        _stream[] = C_NULL
+        rc = ccall((:lmh_graph_capture_end, libluminal_hip), Cint, (Ptr{Cvoid}, Ref{Ptr{Cvoid}}), sref[], gref)
+        if rc != 0
+            ccall((:lmh_stream_destroy, libluminal_hip), Cint, (Ptr{Cvoid},), sref[])
+            check(rc)
+        end
+        cache[:hip_exec] = gref[]
+        cache[:hip_stream] = sref[]
+        cache[:hip_workspace] = _workspace[]   # keeps the recorded scratch alive if the module's one is replaced by a larger one
+    end
+    # the recording's stream is blocking: work enqueued on the null stream before this call is waited for
+    check(ccall((:lmh_graph_launch, libluminal_hip), Cint, (Ptr{Cvoid}, Ptr{Cvoid}), cache[:hip_exec], cache[:hip_stream]))
+    return nothing
+end
+
+"Drop the recording execute_with_capture keeps in `cache` (the buffers it works on are untouched)."
+function release_capture!(cache::Dict)
+    if haskey(cache, :hip_exec)
+        check(ccall((:lmh_sync, libluminal_hip), Cint, (Ptr{Cvoid},), cache[:hip_stream]))
+        check(ccall((:lmh_graph_destroy, libluminal_hip), Cint, (Ptr{Cvoid},), pop!(cache, :hip_exec)))
+        check(ccall((:lmh_stream_destroy, libluminal_hip), Cint, (Ptr{Cvoid},), pop!(cache, :hip_stream)))
+    end
+    delete!(cache, :hip_warm)
+    delete!(cache, :hip_workspace)
+    return nothing
+end
+
+export HIPDevice, HipArray, release_capture!, DecodeAttentionOp, decode_attention, get_device, functional, rope!, kv_append!,
        self_attention_core!, cached_self_attention_core!
 
 end # module
