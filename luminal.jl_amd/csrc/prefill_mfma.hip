@@ -2,11 +2,12 @@
 //
 // Same mathematics as flash_attn_cpu (reference src/Execution.jl:453-479) — online softmax with a
 // running max m, running sum l and an un-normalised output row — evaluated 64 keys at a time for
-// 128 query rows per workgroup instead of one (i, j) pair at a time.
+// 128 or 256 query rows per workgroup instead of one (i, j) pair at a time.
 //
 // Tiling (wave64, v_mfma_f32_32x32x16):
-//   * workgroup = 4 waves = 128 query rows of one (b, hq); each wave owns 32 query rows and keeps
-//     their Q fragments in registers for the whole kernel;
+//   * workgroup = 4 waves = 128 query rows of one (b, hq) (8 waves = 256 rows in launches large
+//     enough to stay balanced with them); each wave owns 32 query rows and keeps their Q
+//     fragments in registers for the whole kernel;
 //   * the scores are computed TRANSPOSED, S^T = K Q^T (M = keys, N = queries). In the MFMA
 //     accumulator layout a lane then holds one query column (n = lane % 32) and 16 of the 32 keys
 //     of a block, so the softmax statistics (max, sum, rescale factor) are per-lane scalars and
@@ -92,17 +93,21 @@ struct MfmaBF16 {
   }
 };
 
-// KSPLIT = 1: the four waves own 4 x 32 query rows and walk the same 64-key tiles.
+// NW waves per workgroup, 32 query rows each, walking the same 64-key tiles (KSPLIT = 1).
+// NW = 8 (256 query rows, two workgroups = 4 waves per SIMD on a CU, at most 128 registers) stages every
+// K/V tile once per 256 rows instead of once per 128: 3-6 % faster wherever there are enough
+// workgroups to keep the balance (measured: non-causal from 512 such workgroups, causal from 1024).
 // KSPLIT = 2: for launches too small to fill the chip. The workgroup owns 64 query rows; waves 0-1
 // take them against the first 32 keys of every tile, waves 2-3 against the second 32, each pair
 // with its own running max / sum / output, merged through LDS at the end. Twice the workgroups,
 // and a wave's share of a tile is half as long.
-template <typename MT, int D, bool CAUSAL, int KSPLIT>
-__global__ __launch_bounds__(256, (D <= 96 ? 3 : 2)) void prefill_mfma_kernel(PrefillArgs a, int n_q_tiles, int n_bh_groups) {
+// The second launch bound is waves per SIMD.
+template <typename MT, int D, bool CAUSAL, int KSPLIT, int NW>
+__global__ __launch_bounds__(64 * NW, (NW == 8 ? 4 : D <= 96 ? 3 : 2)) void prefill_mfma_kernel(PrefillArgs a, int n_q_tiles, int n_bh_groups) {
   using vec8 = typename MT::vec8;
-  constexpr int BM = 128 / KSPLIT;  // query rows per workgroup
+  constexpr int BM = 32 * NW / KSPLIT;  // query rows per workgroup
   constexpr int BT = BN;            // keys per staged tile
-  constexpr int RG = 4 / KSPLIT;    // waves (32-row groups) per key group
+  constexpr int RG = NW / KSPLIT;   // waves (32-row groups) per key group
   constexpr int NKB = 2 / KSPLIT;   // 32-key blocks a wave takes per tile
   constexpr int BW = 32 * NKB;      // ... in keys
   constexpr int KS = D / 16;       // k-steps of the S^T product
@@ -173,7 +178,7 @@ __global__ __launch_bounds__(256, (D <= 96 ? 3 : 2)) void prefill_mfma_kernel(Pr
   // padded row layout needs no register staging and no LDS store instructions. Lanes that fall on
   // a padding chunk fetch out of range. The descriptor's size is the end of the last valid key row:
   // rows past n_keys arrive as zeros without a branch, and the per-lane offsets are loop
-  // invariants. Wave w issues blocks w, w + 4, ...
+  // invariants. Wave w issues blocks w, w + NW, ...
   // The load is written in asm because the compiler, when it knows of an LDS-writing load in
   // flight, waits for it before the next LDS read of the same array — which would serialise the
   // prefetch of tile kt + 1 with the fragment reads of tile kt. The wait that matters (this wave's
@@ -182,9 +187,9 @@ __global__ __launch_bounds__(256, (D <= 96 ? 3 : 2)) void prefill_mfma_kernel(Pr
   typedef __attribute__((address_space(3))) void lds_void_t;
   constexpr int KC = LDK / 8, VC = LDV / 8;            // 16-byte chunks per LDS row
   constexpr int KI = KC * BT / 64, VI = VC * BT / 64;  // 1 KB blocks per tile
-  constexpr int KJ = (KI + 3) / 4, VJ = (VI + 3) / 4;  // blocks per wave (rounded up)
+  constexpr int KJ = (KI + NW - 1) / NW, VJ = (VI + NW - 1) / NW;  // blocks per wave (rounded up)
   const int wave_u = __builtin_amdgcn_readfirstlane(wave);
-  __builtin_assume(wave_u >= 0 && wave_u < 4);
+  __builtin_assume(wave_u >= 0 && wave_u < NW);
   auto make_desc = [](const uint16_t *base, int bytes) {
     const uint64_t p = (uint64_t)base;
     i32x4_t d;
@@ -199,13 +204,13 @@ __global__ __launch_bounds__(256, (D <= 96 ? 3 : 2)) void prefill_mfma_kernel(Pr
   int k_voff[KJ], v_voff[VJ];
 #pragma unroll
   for (int j = 0; j < KJ; j++) {
-    const int ch = (wave + 4 * j) * 64 + lane;
+    const int ch = (wave + NW * j) * 64 + lane;
     const int row = ch / KC, col = ch % KC;
     k_voff[j] = col < cpr ? (int)((row * a.ks[2] + col * 8) * 2) : kOutOfRange;
   }
 #pragma unroll
   for (int j = 0; j < VJ; j++) {
-    const int ch = (wave + 4 * j) * 64 + lane;
+    const int ch = (wave + NW * j) * 64 + lane;
     const int row = ch / VC, col = ch % VC;
     v_voff[j] = col < cpr ? (int)((row * a.vs[2] + col * 8) * 2) : kOutOfRange;
   }
@@ -222,12 +227,12 @@ __global__ __launch_bounds__(256, (D <= 96 ? 3 : 2)) void prefill_mfma_kernel(Pr
   auto load_tile = [&](int kt, int buf) {
 #pragma unroll
     for (int j = 0; j < KJ; j++)
-      if (wave_u + 4 * j < KI)
-        load_block(k_desc, k_lds0 + buf * (BT * LDK * 2) + j * 4096, k_voff[j], kt * k_tile_bytes);
+      if (wave_u + NW * j < KI)
+        load_block(k_desc, k_lds0 + buf * (BT * LDK * 2) + j * (NW * 1024), k_voff[j], kt * k_tile_bytes);
 #pragma unroll
     for (int j = 0; j < VJ; j++)
-      if (wave_u + 4 * j < VI)
-        load_block(v_desc, v_lds0 + buf * (BT * LDV * 2) + j * 4096, v_voff[j], kt * v_tile_bytes);
+      if (wave_u + NW * j < VI)
+        load_block(v_desc, v_lds0 + buf * (BT * LDV * 2) + j * (NW * 1024), v_voff[j], kt * v_tile_bytes);
   };
 
   // lane-constant pieces of the LDS addresses
@@ -397,15 +402,16 @@ __global__ __launch_bounds__(256, (D <= 96 ? 3 : 2)) void prefill_mfma_kernel(Pr
   }
 }
 
-template <typename MT, int D, int KSPLIT>
+template <typename MT, int D, int KSPLIT, int NW>
 int launch_split(const PrefillArgs &a, hipStream_t stream) {
-  const int n_q_tiles = (a.Sq + 128 / KSPLIT - 1) / (128 / KSPLIT);
+  constexpr int BM = 32 * NW / KSPLIT;
+  const int n_q_tiles = (a.Sq + BM - 1) / BM;
   const int n_bh_groups = (a.B * a.Hq + 7) / 8;
-  dim3 grid(8 * n_bh_groups * n_q_tiles), block(256);
+  dim3 grid(8 * n_bh_groups * n_q_tiles), block(64 * NW);
   if (a.causal)
-    hipLaunchKernelGGL((prefill_mfma_kernel<MT, D, true, KSPLIT>), grid, block, 0, stream, a, n_q_tiles, n_bh_groups);
+    hipLaunchKernelGGL((prefill_mfma_kernel<MT, D, true, KSPLIT, NW>), grid, block, 0, stream, a, n_q_tiles, n_bh_groups);
   else
-    hipLaunchKernelGGL((prefill_mfma_kernel<MT, D, false, KSPLIT>), grid, block, 0, stream, a, n_q_tiles, n_bh_groups);
+    hipLaunchKernelGGL((prefill_mfma_kernel<MT, D, false, KSPLIT, NW>), grid, block, 0, stream, a, n_q_tiles, n_bh_groups);
   LMH_HIP_TRY(hipGetLastError());
   return LMH_OK;
 }
@@ -419,8 +425,16 @@ int launch_for_d(const PrefillArgs &a, hipStream_t stream) {
   // CU it loses for both.
   const int64_t wgs = (int64_t)((a.B * a.Hq + 7) / 8) * 8 * ((a.Sq + 127) / 128);
   const int64_t limit = a.causal ? 2 * kNumCUs : 2 * kNumCUs - 1;
-  if (wgs <= limit && a.Sk >= 4 * BN) return launch_split<MT, D, 2>(a, stream);
-  return launch_split<MT, D, 1>(a, stream);
+  if (wgs <= limit && a.Sk >= 4 * BN) return launch_split<MT, D, 2, 4>(a, stream);
+  // Large launches: 256-row workgroups of eight waves. Measured against the 128-row ones at D = 96, fp16:
+  // non-causal 512 / 768 / 1024 / 1536 / 2048 workgroups +3 / +2 / +2 / +6 / +5 %, causal 512 -7 %
+  // (too few to balance their unequal lengths), 1024 +3 %, 1536 +4..7 %, 2048 +5 %. D = 128 does not fit
+  // the 128 registers that four waves per SIMD leave.
+  if constexpr (D <= 96) {
+    const int64_t wgs256 = (int64_t)((a.B * a.Hq + 7) / 8) * 8 * ((a.Sq + 255) / 256);
+    if (wgs256 >= (a.causal ? 4 * kNumCUs : 2 * kNumCUs)) return launch_split<MT, D, 1, 8>(a, stream);
+  }
+  return launch_split<MT, D, 1, 4>(a, stream);
 }
 
 template <typename MT>

@@ -278,6 +278,30 @@ def test_prefill_small_and_large_launches_agree(lm, hip, oracle, causal):
     assert rel_err(small, large[:, :2]) <= TOL["f16"]
 
 
+@pytest.mark.parametrize("dtype,D,causal", [("f16", 96, False), ("f16", 96, True), ("bf16", 64, True), ("f16", 64, False),
+                                            ("bf16", 96, False), ("f16", 80, True), ("bf16", 40, False)])
+def test_prefill_large_launch_runs_256_row_workgroups(lm, hip, oracle, dtype, D, causal):
+    """From 512 (non-causal) / 1024 (causal) workgroups of 256 query rows on, eight waves share every staged K/V tile
+    (head dims up to 96). GQA, ragged kv_len with a poisoned tail, a query count that is no multiple of 256; every
+    eighth head is checked against the oracle, and two heads against the same heads launched alone (key-split
+    128-row workgroups)."""
+    B, Hq, Hkv = (4, 32, 16) if causal else (2, 32, 8)
+    Sq, Sk = (2048 - 37, 2048 - 37) if causal else (2048 - 200, 1500)
+    q, k, v = inputs(oracle, (B, Hq, Sq, D), (B, Hkv, Sk, D), dtype, 7500 + D, 0.7)
+    lens = np.array([Sk, Sk - 63, 1, Sk - 700][:B], np.int32)
+    kp, vp = k.copy(), v.copy()
+    for b, n in enumerate(lens):
+        kp[b, :, n:] = np.nan
+        vp[b, :, n:] = np.nan
+    got = run_flash(lm, hip, q, kp, vp, dtype, causal, kv_len=lens, out_dtype="f32")
+    assert np.isfinite(got).all()
+    hq = np.arange(0, Hq, 8)
+    want = oracle.flash_attn(q[:, hq], k[:, hq % Hkv], v[:, hq % Hkv], causal=causal, kv_len=lens, nthreads=NT)
+    assert rel_err(got[:, hq], want) <= TOL[dtype]
+    alone = run_flash(lm, hip, q[:1, :2], kp[:1, :2], vp[:1, :2], dtype, causal, kv_len=lens[:1], out_dtype="f32")
+    assert rel_err(alone, got[:1, :2]) <= TOL[dtype]
+
+
 @pytest.mark.parametrize("D", [64, 96, 128])
 @pytest.mark.parametrize("causal", [False, True])
 @pytest.mark.parametrize("B", [1, 9])  # 4 heads: 8 or 72 workgroups of 128 rows -> four-way (D = 64) / two-way key split
