@@ -742,16 +742,23 @@ def _padded(lm, hip, x, dtype, row_pad, rng):
     return lm.to_device(buf, hip, dtype), (H * S * (D + row_pad), S * (D + row_pad), D + row_pad)
 
 
-@pytest.mark.parametrize("seed", range(24))
+@pytest.mark.parametrize("seed", range(32))
 def test_prefill_random_shapes_strides_and_options(lm, hip, oracle, seed):
     """Seeded sweep over what the entry point dispatches on: element type, head dim (matrix-core and vector kernels),
-    GQA group and head map, causal, ragged kv_len, row strides (16-byte aligned and not), fp32 output of half inputs."""
+    GQA group and head map, causal, ragged kv_len, row strides (16-byte aligned and not), fp32 output of half inputs.
+    Seeds from 24 on draw launches of more than a thousand 256-row workgroups (the eight-wave instantiations)."""
     rng = np.random.default_rng(9700 + seed)
     dtype = ["f32", "f16", "bf16"][seed % 3]
     D = int(rng.choice([16, 32, 40, 64, 80, 96, 128]))
-    Hkv = int(rng.integers(1, 4)); G = int(rng.choice([1, 2, 4])); Hq = Hkv * G
-    B = int(rng.integers(1, 4))
-    Sq, Sk = int(rng.integers(1, 260)), int(rng.integers(1, 330))
+    if seed < 24:
+        Hkv = int(rng.integers(1, 4)); G = int(rng.choice([1, 2, 4])); Hq = Hkv * G
+        B = int(rng.integers(1, 4))
+        Sq, Sk = int(rng.integers(1, 260)), int(rng.integers(1, 330))
+    else:
+        dtype = ["f16", "bf16"][seed % 2]
+        Hkv = int(rng.integers(11, 17)); G = int(rng.choice([2, 4])); Hq = Hkv * G
+        B = 352 // Hq + 1
+        Sq, Sk = int(rng.integers(513, 700)), int(rng.integers(260, 800))
     causal = bool(rng.integers(0, 2)); head_map = int(rng.integers(0, 2))
     pad_q, pad_kv = int(rng.choice([0, 8, 3])), int(rng.choice([0, 8, 16, 5]))
     q, k, v = inputs(oracle, (B, Hq, Sq, D), (B, Hkv, Sk, D), dtype, 9800 + seed)
