@@ -94,16 +94,19 @@ struct MfmaBF16 {
 };
 
 // NW waves per workgroup, 32 query rows each, walking the same 64-key tiles (KSPLIT = 1).
-// NW = 8 (256 query rows, two workgroups = 4 waves per SIMD on a CU, at most 128 registers) stages every
-// K/V tile once per 256 rows instead of once per 128: 3-6 % faster wherever there are enough
-// workgroups to keep the balance (measured: non-causal from 512 such workgroups, causal from 1024).
+// NW = 8 (256 query rows) stages every K/V tile once per 256 rows instead of once per 128: 3-8 % faster
+// wherever there are enough workgroups to keep the balance. Head dims up to 96: two such workgroups =
+// 4 waves per SIMD on a CU, at most 128 registers. D = 128: one workgroup per CU, 2 waves per SIMD, as
+// with the 128-row workgroups there.
 // KSPLIT = 2: for launches too small to fill the chip. The workgroup owns 64 query rows; waves 0-1
 // take them against the first 32 keys of every tile, waves 2-3 against the second 32, each pair
 // with its own running max / sum / output, merged through LDS at the end. Twice the workgroups,
 // and a wave's share of a tile is half as long.
 // The second launch bound is waves per SIMD.
-template <typename MT, int D, bool CAUSAL, int KSPLIT, int NW>
-__global__ __launch_bounds__(64 * NW, (NW == 8 ? 4 : D <= 96 ? 3 : 2)) void prefill_mfma_kernel(PrefillArgs a, int n_q_tiles, int n_bh_groups) {
+// WPS: waves per SIMD the register budget is set for (3 x 4 waves, 2 x 8 waves or 1 x 8 waves per CU).
+template <int D, int NW> constexpr int default_wps() { return D > 96 ? 2 : NW == 8 ? 4 : 3; }
+template <typename MT, int D, bool CAUSAL, int KSPLIT, int NW, int WPS>
+__global__ __launch_bounds__(64 * NW, WPS) void prefill_mfma_kernel(PrefillArgs a, int n_q_tiles, int n_bh_groups) {
   using vec8 = typename MT::vec8;
   constexpr int BM = 32 * NW / KSPLIT;  // query rows per workgroup
   constexpr int BT = BN;            // keys per staged tile
@@ -402,16 +405,16 @@ __global__ __launch_bounds__(64 * NW, (NW == 8 ? 4 : D <= 96 ? 3 : 2)) void pref
   }
 }
 
-template <typename MT, int D, int KSPLIT, int NW>
+template <typename MT, int D, int KSPLIT, int NW, int WPS = default_wps<D, NW>()>
 int launch_split(const PrefillArgs &a, hipStream_t stream) {
   constexpr int BM = 32 * NW / KSPLIT;
   const int n_q_tiles = (a.Sq + BM - 1) / BM;
   const int n_bh_groups = (a.B * a.Hq + 7) / 8;
   dim3 grid(8 * n_bh_groups * n_q_tiles), block(64 * NW);
   if (a.causal)
-    hipLaunchKernelGGL((prefill_mfma_kernel<MT, D, true, KSPLIT, NW>), grid, block, 0, stream, a, n_q_tiles, n_bh_groups);
+    hipLaunchKernelGGL((prefill_mfma_kernel<MT, D, true, KSPLIT, NW, WPS>), grid, block, 0, stream, a, n_q_tiles, n_bh_groups);
   else
-    hipLaunchKernelGGL((prefill_mfma_kernel<MT, D, false, KSPLIT, NW>), grid, block, 0, stream, a, n_q_tiles, n_bh_groups);
+    hipLaunchKernelGGL((prefill_mfma_kernel<MT, D, false, KSPLIT, NW, WPS>), grid, block, 0, stream, a, n_q_tiles, n_bh_groups);
   LMH_HIP_TRY(hipGetLastError());
   return LMH_OK;
 }
@@ -428,11 +431,23 @@ int launch_for_d(const PrefillArgs &a, hipStream_t stream) {
   if (wgs <= limit && a.Sk >= 4 * BN) return launch_split<MT, D, 2, 4>(a, stream);
   // Large launches: 256-row workgroups of eight waves. Measured against the 128-row ones at D = 96, fp16:
   // non-causal 512 / 768 / 1024 / 1536 / 2048 workgroups +3 / +2 / +2 / +6 / +5 %, causal 512 -7 %
-  // (too few to balance their unequal lengths), 1024 +3 %, 1536 +4..7 %, 2048 +5 %. D = 128 does not fit
-  // the 128 registers that four waves per SIMD leave.
+  // (too few to balance their unequal lengths), 1024 +3 %, 1536 +4..7 %, 2048 +5 %.
+  // D = 128 does not fit the 128 registers that four waves per SIMD leave: one 256-row workgroup per CU there,
+  // which turns over in rounds and balances earlier. fp16: non-causal 256 / 512 / 2048 workgroups +5 / +3 / +6 %,
+  // causal 256 / 384 -8 / -5 %, 512 / 1024 / 2048 +8 / +3 / +4 %; bf16 (more registers, more MFMAs per staged
+  // tile) 0 / -2 %: stays on 128 rows.
+  const int64_t wgs256 = (int64_t)((a.B * a.Hq + 7) / 8) * 8 * ((a.Sq + 255) / 256);
   if constexpr (D <= 96) {
-    const int64_t wgs256 = (int64_t)((a.B * a.Hq + 7) / 8) * 8 * ((a.Sq + 255) / 256);
     if (wgs256 >= (a.causal ? 4 * kNumCUs : 2 * kNumCUs)) return launch_split<MT, D, 1, 8>(a, stream);
+    // Causal, exactly two rounds of one 256-row workgroup per CU (the Phi-3 prompt: 32 heads x 4096 rows): every
+    // CU takes one long workgroup and then one short one, and K/V tiles are staged once per 256 rows. 120.4 ->
+    // 116.2 us at D = 96 (bf16 164 -> 158 us); at 1.5 or 2.5 rounds it is 1-2 % behind the 128-row workgroups, at
+    // one round 20 %, at D = 64 (less LDS and registers in use per workgroup) 5 %.
+    if constexpr (D == 96)
+      if (a.causal && wgs256 >= 2 * kNumCUs && wgs256 < 2 * kNumCUs + kNumCUs / 4)
+        return launch_split<MT, D, 1, 8, 2>(a, stream);
+  } else if constexpr (!MT::kSplitP) {
+    if (wgs256 >= (a.causal ? 2 * kNumCUs : kNumCUs)) return launch_split<MT, D, 1, 8>(a, stream);
   }
   return launch_split<MT, D, 1, 4>(a, stream);
 }

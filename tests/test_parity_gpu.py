@@ -279,10 +279,11 @@ def test_prefill_small_and_large_launches_agree(lm, hip, oracle, causal):
 
 
 @pytest.mark.parametrize("dtype,D,causal", [("f16", 96, False), ("f16", 96, True), ("bf16", 64, True), ("f16", 64, False),
-                                            ("bf16", 96, False), ("f16", 80, True), ("bf16", 40, False)])
+                                            ("bf16", 96, False), ("f16", 80, True), ("bf16", 40, False),
+                                            ("f16", 128, False), ("f16", 128, True), ("f16", 112, True)])
 def test_prefill_large_launch_runs_256_row_workgroups(lm, hip, oracle, dtype, D, causal):
     """From 512 (non-causal) / 1024 (causal) workgroups of 256 query rows on, eight waves share every staged K/V tile
-    (head dims up to 96). GQA, ragged kv_len with a poisoned tail, a query count that is no multiple of 256; every
+    (fp16 and bf16 at head dims up to 96, fp16 above). GQA, ragged kv_len with a poisoned tail, a query count that is no multiple of 256; every
     eighth head is checked against the oracle, and two heads against the same heads launched alone (key-split
     128-row workgroups)."""
     B, Hq, Hkv = (4, 32, 16) if causal else (2, 32, 8)
