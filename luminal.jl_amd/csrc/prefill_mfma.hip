@@ -30,7 +30,7 @@
 namespace lmh {
 namespace {
 
-constexpr int BN = 64;   // keys a wave takes per tile
+constexpr int BN = 64;   // keys per staged tile (twice that in one instantiation, see BT)
 constexpr int kNumCUs = 256;
 // LDS row paddings in elements. K rows are read 16 bytes per lane, one row per lane: a stride of
 // D + 8 elements spreads 16 consecutive rows over all banks (5 cycles per 1 KB fragment per CU,
@@ -109,9 +109,11 @@ template <typename MT, int D, bool CAUSAL, int KSPLIT, int NW, int WPS>
 __global__ __launch_bounds__(64 * NW, WPS) void prefill_mfma_kernel(PrefillArgs a, int n_q_tiles, int n_bh_groups) {
   using vec8 = typename MT::vec8;
   constexpr int BM = 32 * NW / KSPLIT;  // query rows per workgroup
-  constexpr int BT = BN;            // keys per staged tile
+  // keys per staged tile: 64; 128 where one workgroup has the CU to itself and LDS and registers allow (half the
+  // barriers and per-tile bookkeeping: 114.2 -> 111.9 us on B=1 H=32 S=4096 causal)
+  constexpr int BT = (NW == 8 && WPS == 2 && D <= 96 && KSPLIT == 1) ? 2 * BN : BN;
   constexpr int RG = NW / KSPLIT;   // waves (32-row groups) per key group
-  constexpr int NKB = 2 / KSPLIT;   // 32-key blocks a wave takes per tile
+  constexpr int NKB = BT / 32 / KSPLIT;   // 32-key blocks a wave takes per tile
   constexpr int BW = 32 * NKB;      // ... in keys
   constexpr int KS = D / 16;       // k-steps of the S^T product
   constexpr int DB = D / 32;       // 32-row blocks of O^T
@@ -266,23 +268,27 @@ __global__ __launch_bounds__(64 * NW, WPS) void prefill_mfma_kernel(PrefillArgs 
     if (CAUSAL && k0 > wave_q_hi) continue;   // all of it above this wave's diagonal
     if (KSPLIT > 1 && k0 >= k_end) continue;  // ... or past the last key (second half of the last tile)
 
-    // ---- S^T = K Q^T for the wave's 32-key blocks: all fragments are fetched first, then the
-    // accumulator chains alternate so that neither waits on LDS or on its own previous MFMA ----
-    vec8 kf[NKB][KS];
-#pragma unroll
-    for (int ks = 0; ks < KS; ks++)
-#pragma unroll
-      for (int kb = 0; kb < NKB; kb++)
-        kf[kb][ks] = *reinterpret_cast<const vec8 *>(&Ks[k_frag_off + kb * 32 * LDK + 16 * ks]);
+    // ---- S^T = K Q^T for the wave's 32-key blocks, two at a time: their fragments are fetched first, then
+    // the two accumulator chains alternate so that neither waits on LDS or on its own previous MFMA ----
     floatx16_t sacc[NKB];
 #pragma unroll
     for (int kb = 0; kb < NKB; kb++)
 #pragma unroll
       for (int i = 0; i < 16; i++) sacc[kb][i] = 0.f;
+    constexpr int KBG = NKB < 2 ? NKB : 2;  // key blocks whose fragments are fetched together
 #pragma unroll
-    for (int ks = 0; ks < KS; ks++)
+    for (int kb0 = 0; kb0 < NKB; kb0 += KBG) {
+      vec8 kf[KBG][KS];
 #pragma unroll
-      for (int kb = 0; kb < NKB; kb++) sacc[kb] = MT::mfma(kf[kb][ks], qreg[ks], sacc[kb]);
+      for (int ks = 0; ks < KS; ks++)
+#pragma unroll
+        for (int kb = 0; kb < KBG; kb++)
+          kf[kb][ks] = *reinterpret_cast<const vec8 *>(&Ks[k_frag_off + (kb0 + kb) * 32 * LDK + 16 * ks]);
+#pragma unroll
+      for (int ks = 0; ks < KS; ks++)
+#pragma unroll
+        for (int kb = 0; kb < KBG; kb++) sacc[kb0 + kb] = MT::mfma(kf[kb][ks], qreg[ks], sacc[kb0 + kb]);
+    }
 
     // ---- masking (diagonal tiles and the ragged last tile only) ----
     const bool need_mask = (k0 + BW > n_keys) || (CAUSAL && k0 + BW - 1 > wave_q_lo);

@@ -278,15 +278,18 @@ def test_prefill_small_and_large_launches_agree(lm, hip, oracle, causal):
     assert rel_err(small, large[:, :2]) <= TOL["f16"]
 
 
-@pytest.mark.parametrize("dtype,D,causal", [("f16", 96, False), ("f16", 96, True), ("bf16", 64, True), ("f16", 64, False),
-                                            ("bf16", 96, False), ("f16", 80, True), ("bf16", 40, False),
-                                            ("f16", 128, False), ("f16", 128, True), ("f16", 112, True)])
-def test_prefill_large_launch_runs_256_row_workgroups(lm, hip, oracle, dtype, D, causal):
+@pytest.mark.parametrize("dtype,D,causal,B", [("f16", 96, False, 2), ("f16", 96, True, 4), ("bf16", 64, True, 4),
+                                              ("f16", 64, False, 2), ("bf16", 96, False, 2), ("f16", 80, True, 4),
+                                              ("bf16", 40, False, 2), ("f16", 128, False, 2), ("f16", 128, True, 4),
+                                              ("f16", 112, True, 4),
+                                              # causal, 512 workgroups = two rounds of one per CU: 128-key tiles at D = 96
+                                              ("f16", 96, True, 2), ("bf16", 96, True, 2), ("f16", 88, True, 2)])
+def test_prefill_large_launch_runs_256_row_workgroups(lm, hip, oracle, dtype, D, causal, B):
     """From 512 (non-causal) / 1024 (causal) workgroups of 256 query rows on, eight waves share every staged K/V tile
     (fp16 and bf16 at head dims up to 96, fp16 above). GQA, ragged kv_len with a poisoned tail, a query count that is no multiple of 256; every
     eighth head is checked against the oracle, and two heads against the same heads launched alone (key-split
     128-row workgroups)."""
-    B, Hq, Hkv = (4, 32, 16) if causal else (2, 32, 8)
+    Hq, Hkv = (32, 16) if causal else (32, 8)
     Sq, Sk = (2048 - 37, 2048 - 37) if causal else (2048 - 200, 1500)
     q, k, v = inputs(oracle, (B, Hq, Sq, D), (B, Hkv, Sk, D), dtype, 7500 + D, 0.7)
     lens = np.array([Sk, Sk - 63, 1, Sk - 700][:B], np.int32)
