@@ -445,12 +445,13 @@ int launch_for_d(const PrefillArgs &a, hipStream_t stream) {
   const int64_t wgs256 = (int64_t)((a.B * a.Hq + 7) / 8) * 8 * ((a.Sq + 255) / 256);
   if constexpr (D <= 96) {
     if (wgs256 >= (a.causal ? 4 * kNumCUs : 2 * kNumCUs)) return launch_split<MT, D, 1, 8>(a, stream);
-    // Causal, exactly two rounds of one 256-row workgroup per CU (the Phi-3 prompt: 32 heads x 4096 rows): every
-    // CU takes one long workgroup and then one short one, and K/V tiles are staged once per 256 rows. 120.4 ->
-    // 116.2 us at D = 96 (bf16 164 -> 158 us); at 1.5 or 2.5 rounds it is 1-2 % behind the 128-row workgroups, at
-    // one round 20 %, at D = 64 (less LDS and registers in use per workgroup) 5 %.
+    // Causal launches of 1.5 to 3 rounds of one 256-row workgroup per CU (the Phi-3 prompt, 32 heads x 4096 rows,
+    // is exactly two): the workgroups turn over heaviest first, so every CU ends up with about the same number
+    // of key tiles; K/V tiles are staged once per 256 rows, and with the CU to itself the workgroup stages 128
+    // keys at a time. Against the 128-row workgroups at D = 96: 1.5 rounds +2 %, 2 rounds +6 % (120.4 -> 112 us;
+    // bf16 164 -> 153 us), 2.25 / 2.5 rounds +1 %, 3 and 3.5 rounds +-0; one round -20 %; D = 64 (2 rounds) -5 %.
     if constexpr (D == 96)
-      if (a.causal && wgs256 >= 2 * kNumCUs && wgs256 < 2 * kNumCUs + kNumCUs / 4)
+      if (a.causal && 2 * wgs256 >= 3 * kNumCUs && wgs256 < 3 * kNumCUs)
         return launch_split<MT, D, 1, 8, 2>(a, stream);
   } else if constexpr (!MT::kSplitP) {
     if (wgs256 >= (a.causal ? 2 * kNumCUs : kNumCUs)) return launch_split<MT, D, 1, 8>(a, stream);
