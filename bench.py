@@ -381,7 +381,7 @@ def other_configs(lm, dev, check=False):
         ap.dtype, ap.rope_k, ap.pairing, ap.base, ap.stream = lm.binding.DTYPE_CODES["bf16"], 1, lm.binding.ROPE_HALF_SPLIT, 10000.0, None
         hbm_line("cache append + rotary K bf16 B=16 Hkv=8 D=128, %s" % label, lambda: lm.binding.kv_append(ap), 4.0 * B * Hkv * T * D * 2)
 
-    # one whole decode step of an attention layer (rotary q, append with rotary K, split-KV attention, merge: 4
+    # one whole decode step of an attention layer (append with rotary q and K, split-KV attention, merge: 3
     # kernels), driven from the host step by step and as one recorded HIP graph; wall clock per step. On the C4
     # shape the GPU is the bottleneck either way; a single short sequence is bound by the host's launches.
     for B, L in ((16, 4096), (1, 512)):
@@ -409,9 +409,9 @@ def other_configs(lm, dev, check=False):
         cg.capture()
         replay = wall_us()
         cg.release()
-        res["decode step of a layer bf16 B=%d Hq=32 Hkv=8 L=%d D=128 (rotary q + append + attention), wall clock" % (B, L)] = {
-            "us_per_step_4_launches_from_the_host": eager, "us_per_step_one_hip_graph": replay}
-        log("[other] decode step B=%d L=%d, wall clock: %.1f us as 4 host launches, %.1f us as one HIP graph" % (B, L, eager, replay))
+        res["decode step of a layer bf16 B=%d Hq=32 Hkv=8 L=%d D=128 (append with rotary q and K + attention), wall clock" % (B, L)] = {
+            "us_per_step_3_launches_from_the_host": eager, "us_per_step_one_hip_graph": replay}
+        log("[other] decode step B=%d L=%d, wall clock: %.1f us as 3 host launches, %.1f us as one HIP graph" % (B, L, eager, replay))
     return res
 
 

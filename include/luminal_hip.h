@@ -23,7 +23,7 @@
 extern "C" {
 #endif
 
-#define LMH_VERSION 100 /* major*10000 + minor*100 + patch */
+#define LMH_VERSION 101 /* major*10000 + minor*100 + patch */
 
 /* status codes */
 #define LMH_OK 0
@@ -217,6 +217,12 @@ typedef struct lmh_kv_append_params {
   int32_t pairing;      /* LMH_ROPE_*, used when rope_k != 0 */
   float base;
   void *stream;
+  /* Optional, for a decode step: this step's queries [B,Hq,T,D] (device, contiguous), rotated in place at the same
+   * positions pos + t with `pairing` and `base` (whatever rope_k says) — saves the separate lmh_rope launch of
+   * apply_rotary_embeddings on q (reference src/NN.jl:253-303, called on the queries at :356). Null = none. Last in the struct
+   * so that zero-initialised params of earlier callers keep their meaning. */
+  void *q_rope;
+  int32_t Hq;
 } lmh_kv_append_params;
 int lmh_kv_append(const lmh_kv_append_params *p);
 

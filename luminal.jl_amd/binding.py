@@ -80,6 +80,7 @@ class KvAppendParams(ctypes.Structure):
         ("k_stride", ctypes.c_int64 * 3), ("v_stride", ctypes.c_int64 * 3),
         ("dtype", ctypes.c_int32), ("rope_k", ctypes.c_int32), ("pairing", ctypes.c_int32), ("base", ctypes.c_float),
         ("stream", ctypes.c_void_p),
+        ("q_rope", ctypes.c_void_p), ("Hq", ctypes.c_int32),
     ]
 
 

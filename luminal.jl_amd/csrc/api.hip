@@ -393,7 +393,8 @@ int lmh_kv_append(const lmh_kv_append_params *p) {
                 p->D, p->Lmax);
   if (p->dtype != LMH_F32 && p->dtype != LMH_F16 && p->dtype != LMH_BF16)
     return fail(LMH_E_UNSUPPORTED, "lmh_kv_append: unknown dtype %d", p->dtype);
-  if (p->rope_k) {
+  if (p->q_rope && p->Hq <= 0) return fail(LMH_E_SHAPE, "lmh_kv_append: q_rope given with Hq=%d", p->Hq);
+  if (p->rope_k || p->q_rope) {
     if (p->D % 2 != 0) return fail(LMH_E_SHAPE, "lmh_kv_append: head dim %d must be even for the rotary embedding", p->D);
     if (p->pairing != LMH_ROPE_HALF_SPLIT && p->pairing != LMH_ROPE_INTERLEAVED)
       return fail(LMH_E_UNSUPPORTED, "lmh_kv_append: unknown pairing %d", p->pairing);
@@ -414,7 +415,9 @@ int lmh_kv_append(const lmh_kv_append_params *p) {
   if (a.ks[2] < p->D || a.vs[2] < p->D) return fail(LMH_E_SHAPE, "lmh_kv_append: cache row stride smaller than head dim");
   a.rope_k = p->rope_k ? 1 : 0;
   a.interleaved = p->pairing == LMH_ROPE_INTERLEAVED;
-  a.log2_base = p->rope_k ? log2f(p->base) : 0.f;
+  a.log2_base = (p->rope_k || p->q_rope) ? log2f(p->base) : 0.f;
+  a.q = p->q_rope;
+  a.Hq = p->q_rope ? p->Hq : 0;
   return launch_kv_append(a, p->dtype, (hipStream_t)p->stream);
 }
 

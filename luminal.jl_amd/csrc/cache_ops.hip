@@ -59,7 +59,23 @@ __global__ __launch_bounds__(256) void kv_append_kernel(KvAppendArgs a) {
   using raw = typename E::raw;
   const int64_t total = (int64_t)a.B * a.Hkv * a.T * a.D;
   const int half = a.D / 2;
-  for (int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += (int64_t)gridDim.x * blockDim.x) {
+  const int64_t total_q = a.q ? (int64_t)a.B * a.Hq * a.T * half : 0;  // pairs of this step's queries to rotate in place
+  for (int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total + total_q; idx += (int64_t)gridDim.x * blockDim.x) {
+    if (idx >= total) {
+      const int64_t r = idx - total;
+      const int j = (int)(r % half);
+      const int t = (int)((r / half) % a.T);
+      const int64_t bh = r / ((int64_t)half * a.T);  // b * Hq + h
+      const int b = (int)(bh / a.Hq);
+      const int d0 = a.interleaved ? 2 * j : j;
+      const int d1 = a.interleaved ? 2 * j + 1 : j + half;
+      raw *qp = reinterpret_cast<raw *>(a.q) + (bh * a.T + t) * a.D;
+      float o0, o1;
+      rope_pair<E>(E::ld(qp[d0]), E::ld(qp[d1]), (float)((a.pos ? a.pos[b] : a.pos_all) + t), j, a.D, a.log2_base, &o0, &o1);
+      qp[d0] = E::st(o0);
+      qp[d1] = E::st(o1);
+      continue;
+    }
     const int d = (int)(idx % a.D);
     const int t = (int)((idx / a.D) % a.T);
     const int h = (int)((idx / ((int64_t)a.D * a.T)) % a.Hkv);
@@ -293,9 +309,16 @@ int launch_kv_append(const KvAppendArgs &a, int dtype, hipStream_t stream) {
       default: return fail(LMH_E_UNSUPPORTED, "kv append: unknown dtype %d", dtype);
     }
     LMH_HIP_TRY(hipGetLastError());
-    return LMH_OK;
+    if (!a.q) return LMH_OK;
+    // prompt-sized: the queries take the rotary kernel of their own
+    RopeArgs r;
+    r.out = a.q; r.x = a.q; r.pos0 = a.pos; r.prev_seq = a.pos_all;
+    r.B = a.B; r.H = a.Hq; r.S = a.T; r.D = a.D;
+    r.xs[0] = r.os[0] = (int64_t)a.Hq * a.T * a.D; r.xs[1] = r.os[1] = (int64_t)a.T * a.D; r.xs[2] = r.os[2] = a.D;
+    r.log2_base = a.log2_base; r.interleaved = a.interleaved;
+    return launch_rope(r, dtype, stream);
   }
-  const int64_t total = (int64_t)a.B * a.Hkv * a.T * a.D;
+  const int64_t total = (int64_t)a.B * a.Hkv * a.T * a.D + (a.q ? (int64_t)a.B * a.Hq * a.T * (a.D / 2) : 0);
   dim3 grid(grid_for(total)), block(256);
   switch (dtype) {
     case LMH_F32: hipLaunchKernelGGL(kv_append_kernel<F32>, grid, block, 0, stream, a); break;

@@ -73,6 +73,8 @@ struct KvAppendArgs {
   int32_t rope_k;  // rotate K by its row position while writing it
   int32_t interleaved;
   float log2_base;
+  void *q;         // optional [B, Hq, T, D], contiguous: rotated in place at the same positions
+  int32_t Hq;
 };
 
 __host__ __device__ inline int kv_head_of(int hq, int Hq, int Hkv, int head_map) {

@@ -248,12 +248,15 @@ class RotaryEmbeddingOp(Op):
 
 class KVAppendOp(Op):
     """In-place cache update (the reference rebuilds the cache with _kv_scatter, src/Whisper.jl:552-570); inputs
-    (k_cache, v_cache, k_new, v_new, pos); outputs 0 and 1 are the two caches themselves (same buffers)."""
+    (k_cache, v_cache, k_new, v_new, pos); outputs 0 and 1 are the two caches themselves (same buffers).
+    With rope_q a sixth input, this step's queries (B,Hq,T,D), is rotated in place by the same launch and is
+    output 2 (the rotary embedding of the queries, reference src/NN.jl:356, without a launch of its own)."""
 
-    def __init__(self, rope_k=False, base=10000.0, interleaved=False):
+    def __init__(self, rope_k=False, base=10000.0, interleaved=False, rope_q=False):
         self.rope_k = bool(rope_k)
         self.base = float(base)
         self.interleaved = bool(interleaved)
+        self.rope_q = bool(rope_q)
 
 
 class Node:
@@ -323,13 +326,20 @@ def rotary_embedding(x, prev_seq=0, base=10000.0, pos0=None, interleaved=False):
     return add_op(g, RotaryEmbeddingOp(prev_seq, base, interleaved), inputs, x.shape, g.dtypes[x.id])
 
 
-def kv_cache_append(k_cache, v_cache, k_new, v_new, pos, rope_k=False, base=10000.0, interleaved=False):
+def kv_cache_append(k_cache, v_cache, k_new, v_new, pos, rope_k=False, base=10000.0, interleaved=False, q=None):
     """Graph form of the cache update: returns the (k, v) cache tensors after rows pos[b] .. pos[b]+T-1 of sequence
-    b were overwritten by k_new / v_new (K optionally rotated by its position on the way in)."""
+    b were overwritten by k_new / v_new (K optionally rotated by its position on the way in). With `q`, this
+    step's queries (B,Hq,T,D), the same node rotates them in place at the same positions and a third tensor, the
+    rotated queries (q's own buffer: the unrotated values are gone), is returned as well."""
     g = k_cache.graph_ref
-    inputs = [(t.id, t.index, t.shape) for t in (k_cache, v_cache, k_new, v_new, pos)]
-    k_out = add_op(g, KVAppendOp(rope_k, base, interleaved), inputs, k_cache.shape, g.dtypes[k_cache.id])
-    return k_out, GraphTensor(k_out.id, v_cache.shape, g, index=1)
+    tensors = (k_cache, v_cache, k_new, v_new, pos) + (() if q is None else (q,))
+    inputs = [(t.id, t.index, t.shape) for t in tensors]
+    k_out = add_op(g, KVAppendOp(rope_k, base, interleaved, rope_q=q is not None), inputs, k_cache.shape,
+                   g.dtypes[k_cache.id])
+    v_out = GraphTensor(k_out.id, v_cache.shape, g, index=1)
+    if q is None:
+        return k_out, v_out
+    return k_out, v_out, GraphTensor(k_out.id, q.shape, g, index=2)
 
 
 def self_attention_core(q, k, v, causal=True, prev_seq=0, rope_base=None, scale=None, head_map=HEADMAP_INTERLEAVED,
@@ -347,16 +357,16 @@ def self_attention_core(q, k, v, causal=True, prev_seq=0, rope_base=None, scale=
 
 def cached_self_attention_core(q, k_new, v_new, k_cache, v_cache, pos, kv_len, rope_base=None, scale=None,
                                head_map=HEADMAP_INTERLEAVED, num_splits=0, out_dtype=None):
-    """One decode step of a cached attention layer (reference src/Whisper.jl:584-620) as three fused nodes:
+    """One decode step of a cached attention layer (reference src/Whisper.jl:584-620) as two fused nodes:
     q (B,Hq,1,D), k_new / v_new (B,Hkv,1,D) are this step's projections, pos int32[B] the row each sequence
     writes, kv_len = pos + 1 the rows it then attends over. Positions are tensors, so one compiled graph serves
     every step (the reference compiles one graph per position, src/Decoding.jl:98-106). Returns (out (B,Hq,D),
     k_cache, v_cache)."""
     g = q.graph_ref
-    if rope_base is not None:
-        q = rotary_embedding(q, 0, rope_base, pos0=pos)
-    k_cache, v_cache = kv_cache_append(k_cache, v_cache, k_new, v_new, pos, rope_k=rope_base is not None,
-                                       base=rope_base or 10000.0)
+    if rope_base is not None:  # one launch: rotate q in place, write the new rows with K rotated on the way in
+        k_cache, v_cache, q = kv_cache_append(k_cache, v_cache, k_new, v_new, pos, rope_k=True, base=rope_base, q=q)
+    else:
+        k_cache, v_cache = kv_cache_append(k_cache, v_cache, k_new, v_new, pos)
     B, Hq, one, D = q.shape
     if one != 1:
         raise ValueError("cached attention takes one query token per sequence; got q %s" % (q.shape,))
@@ -454,11 +464,16 @@ def execute_op_inplace(out, op, *inputs, stream=None, workspaces=None):
         return apply_rotary_embeddings(x, op.prev_seq, op.base, pos0=pos0, out=out, interleaved=op.interleaved,
                                        stream=stream)
     if isinstance(op, KVAppendOp):
-        kc, vc, k_new, v_new, pos = inputs
-        if out is not None and not (isinstance(out, tuple) and out[0] is kc and out[1] is vc):
-            raise ValueError("KVAppendOp works in place: its outputs are its cache inputs")
-        kv_append(kc, vc, k_new, v_new, pos, rope_k=op.rope_k, base=op.base, interleaved=op.interleaved, stream=stream)
-        return (kc, vc)
+        if len(inputs) != (6 if op.rope_q else 5):
+            raise ValueError("KVAppendOp takes (k_cache, v_cache, k_new, v_new, pos%s)" % (", q" if op.rope_q else ""))
+        kc, vc, k_new, v_new, pos = inputs[:5]
+        q = inputs[5] if op.rope_q else None
+        if out is not None and not (isinstance(out, tuple) and out[0] is kc and out[1] is vc and
+                                    (q is None or out[2] is q)):
+            raise ValueError("KVAppendOp works in place: its outputs are its cache (and query) inputs")
+        kv_append(kc, vc, k_new, v_new, pos, rope_k=op.rope_k, base=op.base, interleaved=op.interleaved, q=q,
+                  stream=stream)
+        return (kc, vc) if q is None else (kc, vc, q)
     raise TypeError("no HIP kernel for op %s" % type(op).__name__)
 
 
@@ -603,8 +618,9 @@ def compile(graph, device=None):
         raise RuntimeError("compile: no HIP device available and this backend has no CPU path")
     results = []
     for node_id, node in enumerate(graph.nodes):
-        if isinstance(node.op, KVAppendOp):  # in place: the node's outputs are its cache inputs
-            results.append((_pick(results, node.inputs[0]), _pick(results, node.inputs[1])))
+        if isinstance(node.op, KVAppendOp):  # in place: the node's outputs are its cache (and query) inputs
+            refs = [node.inputs[0], node.inputs[1]] + ([node.inputs[5]] if node.op.rope_q else [])
+            results.append(tuple(_pick(results, r) for r in refs))
             continue
         results.append(HipArray(graph.shapes[node_id], graph.dtypes[node_id], device).fill_bytes(0))
     steps = []
@@ -644,9 +660,11 @@ def apply_rotary_embeddings(x, prev_seq=0, base=10000.0, pos0=None, out=None, in
     return out
 
 
-def kv_append(k_cache, v_cache, k_new, v_new, pos, rope_k=False, base=10000.0, interleaved=False, stream=None):
+def kv_append(k_cache, v_cache, k_new, v_new, pos, rope_k=False, base=10000.0, interleaved=False, q=None,
+              stream=None):
     """In-place cache update cache[b,h,pos[b]+t,:] = new[b,h,t,:] (the reference rebuilds the whole cache
-    with _kv_scatter, reference src/Whisper.jl:552-570). `pos` is a HipArray int32[B] or an int."""
+    with _kv_scatter, reference src/Whisper.jl:552-570). `pos` is a HipArray int32[B] or an int. `q`
+    (B,Hq,T,D), if given, is rotated in place at the same positions by the same launch."""
     _require_hip(k_cache, v_cache, k_new, v_new)
     if k_cache.shape != v_cache.shape or k_new.shape != v_new.shape or len(k_cache.shape) != 4:
         raise ValueError("kv_append expects caches (B,Hkv,Lmax,D) and new rows (B,Hkv,T,D)")
@@ -667,6 +685,12 @@ def kv_append(k_cache, v_cache, k_new, v_new, pos, rope_k=False, base=10000.0, i
     p.pairing = binding.ROPE_INTERLEAVED if interleaved else binding.ROPE_HALF_SPLIT
     p.base = float(base)
     p.stream = stream
+    if q is not None:
+        _require_hip(q)
+        if len(q.shape) != 4 or q.shape[0] != B or q.shape[2:] != (k_new.shape[2], D) or q.dtype != k_cache.dtype:
+            raise ValueError("kv_append: q %s (%s) does not match new rows %s (%s)" %
+                             (q.shape, q.dtype, k_new.shape, k_cache.dtype))
+        p.q_rope, p.Hq = q.ptr, q.shape[1]
     binding.kv_append(p)
 
 

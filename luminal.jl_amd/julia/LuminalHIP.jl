@@ -213,14 +213,21 @@ struct KvAppendParams
     k_stride::NTuple{3,Int64}; v_stride::NTuple{3,Int64}
     dtype::Int32; rope_k::Int32; pairing::Int32; base::Float32
     stream::Ptr{Cvoid}
+    q_rope::Ptr{Cvoid}; Hq::Int32
 end
 
-"cache[b,h,pos[b]+t,:] = new[b,h,t,:] in place (the reference rebuilds the cache with _kv_scatter, src/Whisper.jl:552-570)."
+"""
+cache[b,h,pos[b]+t,:] = new[b,h,t,:] in place (the reference rebuilds the cache with _kv_scatter,
+src/Whisper.jl:552-570). With `q` (B,Hq,T,D) the same launch rotates this step's queries in place at the same
+positions (apply_rotary_embeddings on the queries, src/NN.jl:356).
+"""
 function kv_append!(kc::HipArray{T,4}, vc::HipArray{T,4}, k_new::HipArray{T,4}, v_new::HipArray{T,4},
-                    pos::HipArray{Int32,1}; rope_k::Bool=false, base::Real=10000.0f0) where {T}
+                    pos::HipArray{Int32,1}; rope_k::Bool=false, base::Real=10000.0f0,
+                    q::Union{Nothing,HipArray{T,4}}=nothing) where {T}
     B, Hkv, Lmax, D = size(kc)
     p = Ref(KvAppendParams(kc.ptr, vc.ptr, k_new.ptr, v_new.ptr, Ptr{Int32}(pos.ptr), 0, B, Hkv, size(k_new, 3), D, Lmax,
-                           Z3, Z3, dtype_code(T), Int32(rope_k), Int32(0), Float32(base), current_stream()))
+                           Z3, Z3, dtype_code(T), Int32(rope_k), Int32(0), Float32(base), current_stream(),
+                           q === nothing ? C_NULL : q.ptr, q === nothing ? Int32(0) : Int32(size(q, 2))))
     check(ccall((:lmh_kv_append, libluminal_hip), Cint, (Ref{KvAppendParams},), p))
     return kc, vc
 end
@@ -254,8 +261,9 @@ function cached_self_attention_core!(out::HipArray{TO,3}, q::HipArray{T,4}, k_ne
                                      kv_len::HipArray{Int32,1}; rope_base=nothing, scale=nothing,
                                      head_map::Int32=HEADMAP_INTERLEAVED) where {TO,T}
     size(q, 3) == 1 || error("cached attention takes one query token per sequence")
-    rope_base !== nothing && rope!(q; pos0=pos, base=rope_base)
-    kv_append!(kc, vc, k_new, v_new, pos; rope_k=(rope_base !== nothing), base=something(rope_base, 10000.0f0))
+    # one launch: the new rows go into the caches (K rotated on the way in) and q is rotated in place
+    kv_append!(kc, vc, k_new, v_new, pos; rope_k=(rope_base !== nothing), base=something(rope_base, 10000.0f0),
+               q=(rope_base !== nothing ? q : nothing))
     s = isnothing(scale) ? 1.0f0 / sqrt(Float32(size(q, 4))) : Float32(scale)
     q3 = HipArray{T,3}(q.ptr, (size(q, 1), size(q, 2), size(q, 4)), q)   # same memory, (B,Hq,D); keeps q alive
     return execute_op!(out, DecodeAttentionOp(s, head_map), q3, kc, vc, kv_len)

@@ -23,7 +23,7 @@ def test_library_exports_every_declared_symbol(lm):
     lib = lm.binding.load()
     for name in header_functions():
         assert hasattr(lib, name), name
-    assert lib.lmh_version() == 100
+    assert lib.lmh_version() == 101
 
 
 def test_struct_layout_matches_header(lm):
@@ -139,6 +139,19 @@ def test_rope_and_kv_append_argument_errors(lm):
         b.kv_append(a)
     assert e.value.code == b.LMH_E_NULL and "lmh_kv_append" in str(e.value)
     a.v_new, a.Lmax = 0x4000, 0
+    with pytest.raises(lm.LuminalHipError) as e:
+        b.kv_append(a)
+    assert e.value.code == b.LMH_E_SHAPE
+    # queries to rotate along: a head count is needed, and the rotary arguments are checked although rope_k is off
+    a.Lmax, a.q_rope, a.Hq = 16, 0x5000, 0
+    with pytest.raises(lm.LuminalHipError) as e:
+        b.kv_append(a)
+    assert e.value.code == b.LMH_E_SHAPE and "Hq" in str(e.value)
+    a.Hq, a.rope_k, a.pairing, a.base = 4, 0, 7, 10000.0
+    with pytest.raises(lm.LuminalHipError) as e:
+        b.kv_append(a)
+    assert e.value.code == b.LMH_E_UNSUPPORTED
+    a.pairing, a.D = 0, 7
     with pytest.raises(lm.LuminalHipError) as e:
         b.kv_append(a)
     assert e.value.code == b.LMH_E_SHAPE

@@ -69,8 +69,8 @@ def test_execute_needs_values_for_inputs(lm):
         lm.execute(g, out.id, {}, lm.CPUDevice())
 
 
-def test_cached_attention_core_emits_three_fused_nodes(lm):
-    # rotary on q, in-place append (K rotated on the way in), fused cached attention; positions are tensors
+def test_cached_attention_core_emits_two_fused_nodes(lm):
+    # in-place append that also rotates q (K rotated on the way in), then fused cached attention; positions are tensors
     B, Hq, Hkv, D, Lmax = 2, 8, 2, 64, 32
     g = lm.Graph()
     q, kn, vn = lm.tensor(g, (B, Hq, 1, D)), lm.tensor(g, (B, Hkv, 1, D)), lm.tensor(g, (B, Hkv, 1, D))
@@ -79,16 +79,25 @@ def test_cached_attention_core_emits_three_fused_nodes(lm):
     n_inputs = len(g.nodes)
     out, kc2, vc2 = lm.cached_self_attention_core(q, kn, vn, kc, vc, pos, kv_len, rope_base=10000.0)
     ops = [type(n.op).__name__ for n in g.nodes[n_inputs:]]
-    assert ops == ["RotaryEmbeddingOp", "KVAppendOp", "DecodeAttentionOp"]
-    rot, app, att = g.nodes[n_inputs:]
-    assert [i[0] for i in rot.inputs] == [q.id, pos.id]
-    assert app.op.rope_k is True and [i[0] for i in app.inputs] == [kc.id, vc.id, kn.id, vn.id, pos.id]
-    # attention reads outputs 0 and 1 of the append node (the caches after the update) and q as (B, Hq, D)
-    assert [(i[0], i[1]) for i in att.inputs] == [(n_inputs, 0), (kc2.id, 0), (vc2.id, 1), (kv_len.id, 0)]
+    assert ops == ["KVAppendOp", "DecodeAttentionOp"]
+    app, att = g.nodes[n_inputs:]
+    assert app.op.rope_k is True and app.op.rope_q is True
+    assert [i[0] for i in app.inputs] == [kc.id, vc.id, kn.id, vn.id, pos.id, q.id]
+    # attention reads outputs 2 (the rotated q, as (B, Hq, D)), 0 and 1 (the caches after the update) of the append node
+    assert [(i[0], i[1]) for i in att.inputs] == [(n_inputs, 2), (kc2.id, 0), (vc2.id, 1), (kv_len.id, 0)]
     assert att.inputs[0][2] == (B, Hq, D) and out.shape == (B, Hq, D)
-    assert kc2.id == vc2.id and (kc2.index, vc2.index) == (0, 1)
+    assert kc2.id == vc2.id == n_inputs and (kc2.index, vc2.index) == (0, 1)
     with pytest.raises(ValueError):
         lm.cached_self_attention_core(lm.tensor(g, (B, Hq, 2, D)), kn, vn, kc, vc, pos, kv_len)
+    # without a rotary embedding the append node takes no q
+    g2 = lm.Graph()
+    q, kn, vn = lm.tensor(g2, (B, Hq, 1, D)), lm.tensor(g2, (B, Hkv, 1, D)), lm.tensor(g2, (B, Hkv, 1, D))
+    kc, vc = lm.tensor(g2, (B, Hkv, Lmax, D)), lm.tensor(g2, (B, Hkv, Lmax, D))
+    pos, kv_len = lm.tensor(g2, (B,), "i32"), lm.tensor(g2, (B,), "i32")
+    n_inputs = len(g2.nodes)
+    lm.cached_self_attention_core(q, kn, vn, kc, vc, pos, kv_len)
+    app, att = g2.nodes[n_inputs:]
+    assert app.op.rope_q is False and len(app.inputs) == 5 and att.inputs[0][0] == q.id
 
 
 def test_self_attention_core_without_rope_is_one_flash_node(lm):

@@ -539,6 +539,36 @@ def test_kv_append_in_place(lm, hip, oracle, dtype, D, interleaved):
 
 @pytest.mark.parametrize("dtype", ["f32", "f16", "bf16"])
 @pytest.mark.parametrize("interleaved", [False, True])
+@pytest.mark.parametrize("T,D,rope_k", [(1, 128, True), (1, 20, False), (3, 64, True), (250, 64, True)])
+def test_kv_append_rotates_the_queries_in_the_same_call(lm, hip, oracle, dtype, interleaved, T, D, rope_k):
+    """The decode step's q rides along with the cache append: rotated in place at pos[b] + t, what the rotary kernel
+    alone produces (to an ulp) and within tolerance of the oracle; the caches come out as without q."""
+    B, Hq, Hkv, Lmax = 3, 8, 2, 400
+    kc = oracle.round_to(oracle.gen_normal((B, Hkv, Lmax, D), 9270), dtype)
+    vc = oracle.round_to(oracle.gen_normal((B, Hkv, Lmax, D), 9271), dtype)
+    kn = oracle.round_to(oracle.gen_normal((B, Hkv, T, D), 9272), dtype)
+    vn = oracle.round_to(oracle.gen_normal((B, Hkv, T, D), 9273), dtype)
+    q = oracle.round_to(oracle.gen_normal((B, Hq, T, D), 9274), dtype)
+    pos = np.array([0, 17, 149], np.int32)
+    dpos = lm.to_device(pos, hip)
+    dk, dv, dkn, dvn, dq = (lm.to_device(a, hip, dtype) for a in (kc, vc, kn, vn, q))
+    lm.kv_append(dk, dv, dkn, dvn, dpos, rope_k=rope_k, interleaved=interleaved, q=dq)
+    dk2, dv2, dq2 = (lm.to_device(a, hip, dtype) for a in (kc, vc, q))
+    lm.kv_append(dk2, dv2, dkn, dvn, dpos, rope_k=rope_k, interleaved=interleaved)
+    lm.apply_rotary_embeddings(dq2, pos0=dpos, out=dq2, interleaved=interleaved)
+    np.testing.assert_array_equal(dk.to_host(), dk2.to_host())
+    np.testing.assert_array_equal(dv.to_host(), dv2.to_host())
+    # the two kernels contract x0*cos - x1*sin differently: equal to an ulp of the element type
+    assert rel_err(dq.to_host(), dq2.to_host()) <= {"f32": 1e-6, "f16": 1e-3, "bf16": 8e-3}[dtype]
+    tol = {"f32": 1e-4, "f16": 2e-3, "bf16": 8e-3}[dtype]
+    assert rel_err(dq.to_host(), oracle.rope(q, pos0=pos, interleaved=interleaved)) <= tol
+    assert rel_err(dq.to_host(), q) > 1e-2  # it did rotate
+    with pytest.raises(ValueError):
+        lm.kv_append(dk, dv, dkn, dvn, dpos, q=lm.to_device(q[:, :, :, : D // 2], hip, dtype))
+
+
+@pytest.mark.parametrize("dtype", ["f32", "f16", "bf16"])
+@pytest.mark.parametrize("interleaved", [False, True])
 def test_kv_append_whole_prompt(lm, hip, oracle, dtype, interleaved):
     # enough rows for the 16-byte-chunk kernel; the last sequence runs into the end of the cache
     B, Hkv, Lmax, D, T = 3, 4, 400, 64, 250
@@ -593,8 +623,8 @@ def test_calibration_kernels(lm, hip):
 
 
 def test_compiled_decode_step_graph_serves_every_position(lm, hip, oracle):
-    """One compiled graph — rotary embedding of q, in-place cache append with K rotated on the way in, fused
-    cached attention — is built once and stepped through all positions with `pos` / `kv_len` as device tensors
+    """One compiled graph — in-place cache append that rotates q and, on the way in, K; fused cached
+    attention — is built once and stepped through all positions with `pos` / `kv_len` as device tensors
     (the reference compiles one graph per position, src/Decoding.jl:98-106). Every step must equal the matching
     row of causal attention over the rotated sequence (reference src/NN.jl:352-382 as a whole)."""
     B, Hq, Hkv, S, D, Lmax = 2, 8, 2, 24, 64, 32
@@ -613,7 +643,7 @@ def test_compiled_decode_step_graph_serves_every_position(lm, hip, oracle):
                   tlen.id: np.full(B, t + 1, np.int32)})
         got = res[out.id].to_host()
         assert rel_err(got, want[:, :, t]) <= 2e-5, t
-    assert len(cg.steps) == n_steps_built == 3  # rotary, append, attention: nothing was rebuilt per position
+    assert len(cg.steps) == n_steps_built == 2  # append with the rotations, attention: nothing was rebuilt per position
     # the cache the graph holds is the rotated K and the raw V of all steps
     kc_host = res[kc2.id][0].to_host()
     assert rel_err(kc_host[:, :, :S], oracle.rope(k)) <= 2e-5
