@@ -444,15 +444,17 @@ int launch_for_d(const PrefillArgs &a, hipStream_t stream) {
   // tile) 0 / -2 %: stays on 128 rows.
   const int64_t wgs256 = (int64_t)((a.B * a.Hq + 7) / 8) * 8 * ((a.Sq + 255) / 256);
   if constexpr (D <= 96) {
-    if (wgs256 >= (a.causal ? 4 * kNumCUs : 2 * kNumCUs)) return launch_split<MT, D, 1, 8>(a, stream);
     // Causal launches of 1.5 to 3 rounds of one 256-row workgroup per CU (the Phi-3 prompt, 32 heads x 4096 rows,
     // is exactly two): the workgroups turn over heaviest first, so every CU ends up with about the same number
     // of key tiles; K/V tiles are staged once per 256 rows, and with the CU to itself the workgroup stages 128
     // keys at a time. Against the 128-row workgroups at D = 96: 1.5 rounds +2 %, 2 rounds +6 % (120.4 -> 112 us;
     // bf16 164 -> 153 us), 2.25 / 2.5 rounds +1 %, 3 and 3.5 rounds +-0; one round -20 %; D = 64 (2 rounds) -5 %.
+    // Non-causal workgroups are all equally long and a part-filled round is lost time: from two rounds on only
+    // (2 rounds +1 %, bf16 +4 %; 2.5 rounds +3 %; 1.5 rounds -11 %).
     if constexpr (D == 96)
-      if (a.causal && 2 * wgs256 >= 3 * kNumCUs && wgs256 < 3 * kNumCUs)
+      if (wgs256 < 3 * kNumCUs && (a.causal ? 2 * wgs256 >= 3 * kNumCUs : wgs256 >= 2 * kNumCUs))
         return launch_split<MT, D, 1, 8, 2>(a, stream);
+    if (wgs256 >= (a.causal ? 4 * kNumCUs : 2 * kNumCUs)) return launch_split<MT, D, 1, 8>(a, stream);
   } else if constexpr (!MT::kSplitP) {
     if (wgs256 >= (a.causal ? 2 * kNumCUs : kNumCUs)) return launch_split<MT, D, 1, 8>(a, stream);
   }
