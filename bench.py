@@ -37,7 +37,7 @@ PEAK_HBM_GBS = 8000.0      # MI355X HBM3E
 # WRITE_SIZE runs of this script (--only prefill / --only decode), each scaled by what the same
 # counter reads for the calibration copy kernel (--only copy: factor 2.0 for FETCH_SIZE, 1.0 for
 # WRITE_SIZE). Counters cannot be read from inside a timed run, so the figures are recorded here.
-PREFILL_TRAFFIC_BYTES = 104.8e6 + 25.2e6           # vs 75.5 MB + 25.2 MB compulsory
+PREFILL_TRAFFIC_BYTES = 105.2e6 + 25.2e6           # vs 75.5 MB + 25.2 MB compulsory
 DECODE_TRAFFIC_BYTES = 5.2718e9 + 2.8e6 + 4.7e6    # split kernel read + partials + merge kernel
 
 
