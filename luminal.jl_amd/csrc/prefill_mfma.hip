@@ -443,6 +443,7 @@ int launch_for_d(const PrefillArgs &a, hipStream_t stream) {
   // causal 256 / 384 -8 / -5 %, 512 / 1024 / 2048 +8 / +3 / +4 %; bf16 (more registers, more MFMAs per staged
   // tile) 0 / -2 %: stays on 128 rows.
   const int64_t wgs256 = (int64_t)((a.B * a.Hq + 7) / 8) * 8 * ((a.Sq + 255) / 256);
+  if (a.Sq <= 128) return launch_split<MT, D, 1, 4>(a, stream);  // nothing for waves 4-7 to own
   if constexpr (D <= 96) {
     // Causal launches of 1.5 to 3 rounds of one 256-row workgroup per CU (the Phi-3 prompt, 32 heads x 4096 rows,
     // is exactly two): the workgroups turn over heaviest first, so every CU ends up with about the same number

@@ -309,9 +309,9 @@ def test_prefill_large_launch_runs_256_row_workgroups(lm, hip, oracle, dtype, D,
 @pytest.mark.parametrize("dtype,D", [("f16", 96), ("bf16", 96), ("f16", 64), ("f16", 128)])
 @pytest.mark.parametrize("causal", [False, True])
 def test_prefill_many_heads_few_queries_on_256_row_workgroups(lm, hip, oracle, dtype, D, causal):
-    """512 (b, head) pairs with 100 queries each: the launch is large enough for the eight-wave workgroups, whose
-    upper waves then own no query at all (they still stage tiles and meet the barriers); keys end inside a tile."""
-    B, H, Sq, Sk = 8, 64, 100, 300
+    """512 (b, head) pairs with 150 queries each: the launch is large enough for the eight-wave workgroups, three of
+    whose waves then own no query at all (they still stage tiles and meet the barriers); keys end inside a tile."""
+    B, H, Sq, Sk = 8, 64, 150, 300
     q, k, v = inputs(oracle, (B, H, Sq, D), (B, H, Sk, D), dtype, 7600 + D, 0.8)
     got = run_flash(lm, hip, q, k, v, dtype, causal, out_dtype="f32")
     assert np.isfinite(got).all()
