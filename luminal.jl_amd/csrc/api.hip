@@ -12,6 +12,19 @@ namespace lmh {
 
 static thread_local char g_last_error[512] = "";
 
+int device_cu_count() {
+  static const int n = [] {  // one device kind per process (gfx950); initialised once, thread-safely
+    int dev = 0;
+    hipDeviceProp_t prop;
+    if (hipGetDevice(&dev) != hipSuccess || hipGetDeviceProperties(&prop, dev) != hipSuccess || prop.multiProcessorCount < 1) {
+      (void)hipGetLastError();
+      return 256;
+    }
+    return prop.multiProcessorCount;
+  }();
+  return n;
+}
+
 int fail(int code, const char *fmt, ...) {
   va_list ap;
   va_start(ap, fmt);

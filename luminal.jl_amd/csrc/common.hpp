@@ -12,6 +12,9 @@ namespace lmh {
 // Records a message for lmh_last_error() and returns `code`, so call sites read
 // `return fail(LMH_E_SHAPE, "...")`.
 int fail(int code, const char *fmt, ...) __attribute__((format(printf, 2, 3)));
+// Compute units of the current device (256 on an MI355X in its default partition mode; 256 as well if the query
+// fails). The launchers size their workgroups by it; any value gives correct results.
+int device_cu_count();
 int hip_fail(hipError_t e, const char *what);
 
 #define LMH_HIP_TRY(expr)                                \

@@ -24,7 +24,6 @@ namespace lmh {
 namespace {
 
 constexpr int BN = 32;   // keys a wave takes per tile
-constexpr int kNumCUs = 256;
 constexpr int kPadK = 4;  // floats: a row stride of D + 4 puts 16 consecutive rows' 16-byte reads on distinct banks
 constexpr int kPadV = 8;  // floats: rows key and key + 4 (the two halves of a wave) land 32 banks apart
 constexpr float kLog2e = 1.4426950408889634f;
@@ -304,9 +303,10 @@ template <int D>
 int launch_for_d(const PrefillArgs &a, hipStream_t stream) {
   // The key-split workgroups hold tiles of 64 or 128 keys in LDS, one workgroup per CU: use them only while
   // every workgroup still gets a CU of its own. (Four-way needs 143 KB at D = 64 and does not fit beyond.)
+  const int n_cus = device_cu_count();
   const int64_t wgs = (int64_t)((a.B * a.Hq + 7) / 8) * 8 * ((a.Sq + 127) / 128);
-  if (D == 64 && 4 * wgs <= kNumCUs && a.Sk >= 4 * BN) return launch_split<D, (D == 64 ? 4 : 1)>(a, stream);
-  if (2 * wgs <= kNumCUs && a.Sk >= 2 * BN) return launch_split<D, 2>(a, stream);
+  if (D == 64 && 4 * wgs <= n_cus && a.Sk >= 4 * BN) return launch_split<D, (D == 64 ? 4 : 1)>(a, stream);
+  if (2 * wgs <= n_cus && a.Sk >= 2 * BN) return launch_split<D, 2>(a, stream);
   return launch_split<D, 1>(a, stream);
 }
 

@@ -31,7 +31,6 @@ namespace lmh {
 namespace {
 
 constexpr int BN = 64;   // keys per staged tile (twice that in one instantiation, see BT)
-constexpr int kNumCUs = 256;
 // LDS row paddings in elements. K rows are read 16 bytes per lane, one row per lane: a stride of
 // D + 8 elements spreads 16 consecutive rows over all banks (5 cycles per 1 KB fragment per CU,
 // against 16 unpadded). V rows go through the transposing read (4 rows x 32 bytes per 16 lanes); in
@@ -432,8 +431,9 @@ int launch_for_d(const PrefillArgs &a, hipStream_t stream) {
   // Measured on 256 CUs: at exactly two per CU the split still wins for causal launches (41.8 vs
   // 46.7 us at B=1 H=32 S=2048 D=96) and loses for non-causal ones (79.8 vs 66.6 us); at three per
   // CU it loses for both.
+  const int n_cus = device_cu_count();
   const int64_t wgs = (int64_t)((a.B * a.Hq + 7) / 8) * 8 * ((a.Sq + 127) / 128);
-  const int64_t limit = a.causal ? 2 * kNumCUs : 2 * kNumCUs - 1;
+  const int64_t limit = a.causal ? 2 * n_cus : 2 * n_cus - 1;
   if (wgs <= limit && a.Sk >= 4 * BN) return launch_split<MT, D, 2, 4>(a, stream);
   // Large launches: 256-row workgroups of eight waves. Measured against the 128-row ones at D = 96, fp16:
   // non-causal 512 / 768 / 1024 / 1536 / 2048 workgroups +3 / +2 / +2 / +6 / +5 %, causal 512 -7 %
@@ -453,11 +453,11 @@ int launch_for_d(const PrefillArgs &a, hipStream_t stream) {
     // Non-causal workgroups are all equally long and a part-filled round is lost time: from two rounds on only
     // (2 rounds +1 %, bf16 +4 %; 2.5 rounds +3 %; 1.5 rounds -11 %).
     if constexpr (D == 96)
-      if (wgs256 < 3 * kNumCUs && (a.causal ? 2 * wgs256 >= 3 * kNumCUs : wgs256 >= 2 * kNumCUs))
+      if (wgs256 < 3 * n_cus && (a.causal ? 2 * wgs256 >= 3 * n_cus : wgs256 >= 2 * n_cus))
         return launch_split<MT, D, 1, 8, 2>(a, stream);
-    if (wgs256 >= (a.causal ? 4 * kNumCUs : 2 * kNumCUs)) return launch_split<MT, D, 1, 8>(a, stream);
+    if (wgs256 >= (a.causal ? 4 * n_cus : 2 * n_cus)) return launch_split<MT, D, 1, 8>(a, stream);
   } else if constexpr (!MT::kSplitP) {
-    if (wgs256 >= (a.causal ? 2 * kNumCUs : kNumCUs)) return launch_split<MT, D, 1, 8>(a, stream);
+    if (wgs256 >= (a.causal ? 2 * n_cus : n_cus)) return launch_split<MT, D, 1, 8>(a, stream);
   }
   return launch_split<MT, D, 1, 4>(a, stream);
 }
