@@ -214,13 +214,13 @@ typedef struct lmh_kv_append_params {
   int64_t v_stride[3];
   int32_t dtype;
   int32_t rope_k;       /* 0 / 1 */
-  int32_t pairing;      /* LMH_ROPE_*, used when rope_k != 0 */
+  int32_t pairing;      /* LMH_ROPE_*, used when rope_k != 0 or q_rope is given */
   float base;
   void *stream;
-  /* Optional, for a decode step: this step's queries [B,Hq,T,D] (device, contiguous), rotated in place at the same
-   * positions pos + t with `pairing` and `base` (whatever rope_k says) — saves the separate lmh_rope launch of
-   * apply_rotary_embeddings on q (reference src/NN.jl:253-303, called on the queries at :356). Null = none. Last in the struct
-   * so that zero-initialised params of earlier callers keep their meaning. */
+  /* Optional, for a decode step: this step's queries [B,Hq,T,D] (device, contiguous), rotated in place at the
+   * same positions pos + t with `pairing` and `base` (whatever rope_k says) — saves the separate lmh_rope
+   * launch of apply_rotary_embeddings on q (reference src/NN.jl:253-303, called on the queries at :356).
+   * Null = none. Last in the struct so that zero-initialised params of earlier callers keep their meaning. */
   void *q_rope;
   int32_t Hq;
 } lmh_kv_append_params;
