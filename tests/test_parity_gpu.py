@@ -603,6 +603,32 @@ def test_kv_append_whole_prompt(lm, hip, oracle, dtype, interleaved):
     np.testing.assert_array_equal(dv2.to_host(), oracle.kv_append(vc, vn, pos))
 
 
+def test_kv_cache_state_allocation_and_row_placement(lm, hip):
+    """The reference's own cache tests (tests/test_kv_cache.jl:13-29 "KVCacheState allocation", :54-70 "_kv_scatter
+    places token at correct position") on the in-place form: a fresh cache is zero with step_pos 0 and the shape
+    (batch, heads, max_seq, head_dim); a row written at position 0, 1 or the last slot lands there and nowhere else,
+    the cache keeps its shape; appending to a full cache is refused."""
+    cache = lm.KVCacheState(1, 6, 64, max_seq=10, dtype="f32", device=hip)
+    assert cache.step_pos == 0 and cache.max_seq == 10
+    assert cache.k.shape == cache.v.shape == (1, 6, 10, 64)
+    assert not cache.k.to_host().any() and not cache.v.to_host().any()
+    for pos in (0, 1, 3):  # the reference's minimal dims: (batch=1, heads=1, max_seq=4, head_dim=2)
+        past = lm.to_device(np.zeros((1, 1, 4, 2), np.float32), hip)
+        past_v = lm.to_device(np.zeros((1, 1, 4, 2), np.float32), hip)
+        new = lm.to_device(np.array([[[[1.5, -2.5]]]], np.float32), hip)
+        lm.kv_append(past, past_v, new, new, pos)
+        want = np.zeros((1, 1, 4, 2), np.float32)
+        want[0, 0, pos] = [1.5, -2.5]
+        assert past.shape == (1, 1, 4, 2)
+        np.testing.assert_array_equal(past.to_host(), want)
+        np.testing.assert_array_equal(past_v.to_host(), want)
+    for _ in range(10):
+        cache.append(lm.to_device(np.ones((1, 6, 1, 64), np.float32), hip), lm.to_device(np.ones((1, 6, 1, 64), np.float32), hip))
+    assert cache.step_pos == 10
+    with pytest.raises(ValueError, match="full"):
+        cache.append(lm.to_device(np.ones((1, 6, 1, 64), np.float32), hip), lm.to_device(np.ones((1, 6, 1, 64), np.float32), hip))
+
+
 def test_incremental_decode_equals_causal_prefill(lm, hip, oracle):
     """Token-by-token decode through KVCacheState (append + fused cached attention) reproduces causal
     prefill row by row — the end-to-end property the reference's cached path is built on
