@@ -23,7 +23,7 @@
 extern "C" {
 #endif
 
-#define LMH_VERSION 101 /* major*10000 + minor*100 + patch */
+#define LMH_VERSION 102 /* major*10000 + minor*100 + patch */
 
 /* status codes */
 #define LMH_OK 0
@@ -172,6 +172,26 @@ size_t lmh_decode_workspace_bytes(int32_t B, int32_t Hq, int32_t Hkv, int32_t Lm
 /* the split count lmh_decode_attn uses when num_splits == 0 */
 int32_t lmh_decode_auto_splits(int32_t B, int32_t Hkv, int32_t Lmax);
 int lmh_decode_attn(const lmh_decode_params *p);
+
+/* ---- decode attention that allocates nothing and takes no workspace. No counterpart in the reference: it
+ * is lmh_decode_attn for callers that cannot call hipMalloc (code under HIP graph capture, tight serving
+ * loops, harnesses that forbid allocation). Same parameter block, same kernels, same results; `workspace`
+ * and `workspace_bytes` are ignored. The split-KV partials go to a static device array of
+ * LMH_STATIC_SCRATCH_BYTES that each GPU the library runs on holds until the process ends.
+ *   - num_splits == 0 takes lmh_decode_static_splits(): the split count of lmh_decode_attn, halved until
+ *     the partials fit. An explicit num_splits whose partials (lmh_decode_workspace_bytes) exceed the
+ *     array is rejected with LMH_E_WORKSPACE.
+ *   - Every call on one GPU shares that GPU's array, which keeps the last call's contents. Nothing in it
+ *     has to start at zero (each call writes every slot it later reads), so none is cleared; calls that
+ *     overlap in time on one GPU (two streams, two host threads) race on it and must be serialised by the
+ *     caller.
+ *   - lmh_init(device) resolves the array's address on that device; a device that was never passed to
+ *     lmh_init resolves it on its first call here, which may load the code object (do that before a capture).
+ * No hipMalloc, hipFree or other allocating call is made. ---- */
+#define LMH_STATIC_SCRATCH_BYTES ((size_t)32 << 20)
+size_t lmh_static_scratch_bytes(void);
+int32_t lmh_decode_static_splits(int32_t B, int32_t Hq, int32_t Hkv, int32_t Lmax, int32_t D);
+int lmh_decode_attn_static(const lmh_decode_params *p);
 
 /* ---- rotary position embedding: replaces the ~25-node subgraph of
  *   apply_rotary_embeddings(input, prev_seq; base)    reference src/NN.jl:253-303

@@ -25,7 +25,8 @@ EXPORTS = [
     "lmh_event_destroy", "lmh_event_record", "lmh_event_elapsed_ms", "lmh_flash_attn_fwd",
     "lmh_decode_workspace_bytes", "lmh_decode_auto_splits", "lmh_decode_attn", "lmh_calib_copy", "lmh_calib_mfma", "lmh_rope",
     "lmh_kv_append", "lmh_stream_create", "lmh_stream_destroy", "lmh_graph_capture_begin", "lmh_graph_capture_end",
-    "lmh_graph_launch", "lmh_graph_destroy",
+    "lmh_graph_launch", "lmh_graph_destroy", "lmh_static_scratch_bytes", "lmh_decode_static_splits",
+    "lmh_decode_attn_static",
 ]
 
 
@@ -122,6 +123,11 @@ def load():
     L.lmh_decode_workspace_bytes.argtypes = [ctypes.c_int32] * 6
     L.lmh_decode_auto_splits.restype = ctypes.c_int32
     L.lmh_decode_auto_splits.argtypes = [ctypes.c_int32] * 3
+    L.lmh_decode_attn_static.argtypes = [ctypes.POINTER(DecodeParams)]
+    L.lmh_decode_attn_static.restype = ctypes.c_int
+    L.lmh_static_scratch_bytes.restype = ctypes.c_size_t
+    L.lmh_decode_static_splits.restype = ctypes.c_int32
+    L.lmh_decode_static_splits.argtypes = [ctypes.c_int32] * 5
     L.lmh_calib_copy.argtypes = [vp, vp, ctypes.c_size_t, vp]
     L.lmh_calib_mfma.argtypes = [vp, vp, ctypes.c_size_t, ctypes.c_int, ctypes.POINTER(ctypes.c_double), vp]
     L.lmh_rope.argtypes = [ctypes.POINTER(RopeParams)]
@@ -217,6 +223,19 @@ def flash_attn_fwd(params):
 
 def decode_attn(params):
     check(load().lmh_decode_attn(ctypes.byref(params)))
+
+
+def decode_attn_static(params):
+    """lmh_decode_attn without a workspace: partials go to the library's static device scratch."""
+    check(load().lmh_decode_attn_static(ctypes.byref(params)))
+
+
+def static_scratch_bytes():
+    return int(load().lmh_static_scratch_bytes())
+
+
+def decode_static_splits(B, Hq, Hkv, Lmax, D):
+    return int(load().lmh_decode_static_splits(B, Hq, Hkv, Lmax, D))
 
 
 def rope(params):

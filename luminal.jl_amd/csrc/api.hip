@@ -6,7 +6,13 @@
 #include <stdio.h>
 #include <string.h>
 
+#include <mutex>
+
 #include "common.hpp"
+
+// Split-KV partial storage of lmh_decode_attn_static, for callers that cannot allocate device memory.
+// One copy per GPU, held from the moment the code object is loaded on that GPU until the process ends.
+static __device__ __align__(256) unsigned char scratch[LMH_STATIC_SCRATCH_BYTES];
 
 namespace lmh {
 
@@ -49,6 +55,32 @@ size_t elem_bytes(int dtype) { return dtype == LMH_F32 ? 4 : 2; }
 
 bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
+constexpr int kMaxDevices = 64;
+// Device address of `scratch` on each GPU. In host code the array's name is only a handle for
+// hipGetSymbolAddress, never an address a kernel can use.
+void *g_scratch_ptr[kMaxDevices];
+std::mutex g_scratch_mutex;
+
+// Looks the address up once per device, with that device current, and returns it in *out.
+int static_scratch_for_current_device(void **out) {
+  *out = nullptr;
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) {
+    (void)hipGetLastError();
+    return fail(LMH_E_NODEVICE, "static scratch: no current HIP device (or its index is >= %d)", kMaxDevices);
+  }
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (!g_scratch_ptr[dev]) {
+    void *ptr = nullptr;
+    const hipError_t e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+    if (e != hipSuccess) return hip_fail(e, "hipGetSymbolAddress(scratch)");
+    if (!ptr) return fail(LMH_E_HIP, "static scratch: hipGetSymbolAddress returned a null address");
+    g_scratch_ptr[dev] = ptr;
+  }
+  *out = g_scratch_ptr[dev];
+  return LMH_OK;
+}
+
 }  // namespace
 }  // namespace lmh
 
@@ -89,6 +121,10 @@ int lmh_init(int device) {
   void *probe = nullptr;  // same health check as get_device(): a tiny allocation
   LMH_HIP_TRY(hipMalloc(&probe, 4));
   LMH_HIP_TRY(hipFree(probe));
+  // set-up for lmh_decode_attn_static: resolve this device's copy of the static scratch now, so that the
+  // entry point itself never has to (a failure here is reported by that entry point, not by init)
+  void *unused = nullptr;
+  (void)static_scratch_for_current_device(&unused);
   return LMH_OK;
 }
 
@@ -305,23 +341,9 @@ size_t lmh_decode_workspace_bytes(int32_t B, int32_t Hq, int32_t Hkv, int32_t Lm
   return (size_t)B * Hq * num_splits * (size_t)(D + 2) * sizeof(float);
 }
 
-int lmh_decode_attn(const lmh_decode_params *p) {
-  if (!p) return fail(LMH_E_NULL, "lmh_decode_attn: null params");
-  if (!p->out || !p->q || !p->k_cache || !p->v_cache) return fail(LMH_E_NULL, "lmh_decode_attn: null tensor pointer");
-  if (p->B <= 0 || p->Hq <= 0 || p->Hkv <= 0 || p->Lmax <= 0 || p->D <= 0)
-    return fail(LMH_E_SHAPE, "lmh_decode_attn: non-positive dimension (B=%d Hq=%d Hkv=%d Lmax=%d D=%d)", p->B, p->Hq,
-                p->Hkv, p->Lmax, p->D);
-  if (p->Hq % p->Hkv != 0) return fail(LMH_E_SHAPE, "lmh_decode_attn: Hq=%d is not a multiple of Hkv=%d", p->Hq, p->Hkv);
-  if (p->dtype != LMH_F32 && p->dtype != LMH_F16 && p->dtype != LMH_BF16)
-    return fail(LMH_E_UNSUPPORTED, "lmh_decode_attn: unknown dtype %d", p->dtype);
-  if (p->head_map != LMH_HEADMAP_INTERLEAVED && p->head_map != LMH_HEADMAP_BLOCKED)
-    return fail(LMH_E_UNSUPPORTED, "lmh_decode_attn: unknown head_map %d", p->head_map);
-  const int vec = p->dtype == LMH_F32 ? 4 : 8;
-  if (p->D % vec != 0 || p->D > 256)
-    return fail(LMH_E_UNSUPPORTED, "lmh_decode_attn: head dim %d must be a multiple of %d and <= 256", p->D, vec);
-  if (p->num_splits < 0) return fail(LMH_E_SHAPE, "lmh_decode_attn: negative num_splits");
-  if (!(p->scale == p->scale)) return fail(LMH_E_SHAPE, "lmh_decode_attn: scale is NaN");
-
+// Validation and launch shared by lmh_decode_attn (caller-owned workspace) and lmh_decode_attn_static (the
+// library's static scratch): `ws` / `ws_bytes` is the split-KV partial storage, `num_splits` already resolved.
+static int decode_launch(const lmh_decode_params *p, const char *fn, int32_t num_splits, void *ws, size_t ws_bytes) {
   DecodeArgs a;
   a.out = p->out; a.q = p->q; a.k = p->k_cache; a.v = p->v_cache; a.kv_len = p->kv_len;
   a.B = p->B; a.Hq = p->Hq; a.Hkv = p->Hkv; a.Lmax = p->Lmax; a.D = p->D;
@@ -343,29 +365,90 @@ int lmh_decode_attn(const lmh_decode_params *p) {
   // 128-bit loads: every row start must be 16-byte aligned
   const int64_t align_elems = 16 / (int64_t)elem_bytes(p->dtype);
   if (!aligned16(p->k_cache) || !aligned16(p->v_cache))
-    return fail(LMH_E_SHAPE, "lmh_decode_attn: cache pointers must be 16-byte aligned");
+    return fail(LMH_E_SHAPE, "%s: cache pointers must be 16-byte aligned", fn);
   for (int i = 0; i < 3; i++)
     if (a.ks[i] < 0 || a.vs[i] < 0 || a.ks[i] % align_elems != 0 || a.vs[i] % align_elems != 0)
-      return fail(LMH_E_SHAPE, "lmh_decode_attn: cache strides must be non-negative multiples of %lld elements",
+      return fail(LMH_E_SHAPE, "%s: cache strides must be non-negative multiples of %lld elements", fn,
                   (long long)align_elems);
-  if (a.ks[2] < p->D || a.vs[2] < p->D) return fail(LMH_E_SHAPE, "lmh_decode_attn: cache row stride smaller than head dim");
-  if (a.qs[0] < 0 || a.qs[1] < 0 || a.os[0] < 0 || a.os[1] < 0) return fail(LMH_E_SHAPE, "lmh_decode_attn: negative stride");
+  if (a.ks[2] < p->D || a.vs[2] < p->D) return fail(LMH_E_SHAPE, "%s: cache row stride smaller than head dim", fn);
+  if (a.qs[0] < 0 || a.qs[1] < 0 || a.os[0] < 0 || a.os[1] < 0) return fail(LMH_E_SHAPE, "%s: negative stride", fn);
 
   a.mfma_ok = (p->scale > 0.f && aligned16(p->q) && a.qs[0] % 8 == 0 && a.qs[1] % 8 == 0) ? 1 : 0;
-  a.num_splits = p->num_splits == 0 ? lmh_decode_auto_splits(p->B, p->Hkv, p->Lmax) : p->num_splits;
+  a.num_splits = num_splits;
   a.chunk = decode_chunk_for(p->Lmax, a.num_splits);
   a.ws_o = nullptr;
   a.ws_ml = nullptr;
   if (a.num_splits > 1) {
     const size_t need = lmh_decode_workspace_bytes(p->B, p->Hq, p->Hkv, p->Lmax, p->D, a.num_splits);
-    if (!p->workspace || p->workspace_bytes < need)
-      return fail(LMH_E_WORKSPACE, "lmh_decode_attn: workspace of %zu bytes needed for %d splits, got %zu", need,
-                  a.num_splits, p->workspace ? p->workspace_bytes : (size_t)0);
-    if (!aligned16(p->workspace)) return fail(LMH_E_WORKSPACE, "lmh_decode_attn: workspace must be 16-byte aligned");
-    a.ws_o = reinterpret_cast<float *>(p->workspace);
+    if (!ws || ws_bytes < need)
+      return fail(LMH_E_WORKSPACE, "%s: workspace of %zu bytes needed for %d splits, got %zu", fn, need,
+                  a.num_splits, ws ? ws_bytes : (size_t)0);
+    if (!aligned16(ws)) return fail(LMH_E_WORKSPACE, "%s: workspace must be 16-byte aligned", fn);
+    a.ws_o = reinterpret_cast<float *>(ws);
     a.ws_ml = a.ws_o + (size_t)p->B * p->Hq * a.num_splits * p->D;
   }
   return launch_decode(a, p->dtype, (hipStream_t)p->stream);
+}
+
+static int decode_check(const lmh_decode_params *p, const char *fn) {
+  if (!p) return fail(LMH_E_NULL, "%s: null params", fn);
+  if (!p->out || !p->q || !p->k_cache || !p->v_cache) return fail(LMH_E_NULL, "%s: null tensor pointer", fn);
+  if (p->B <= 0 || p->Hq <= 0 || p->Hkv <= 0 || p->Lmax <= 0 || p->D <= 0)
+    return fail(LMH_E_SHAPE, "%s: non-positive dimension (B=%d Hq=%d Hkv=%d Lmax=%d D=%d)", fn, p->B, p->Hq,
+                p->Hkv, p->Lmax, p->D);
+  if (p->Hq % p->Hkv != 0) return fail(LMH_E_SHAPE, "%s: Hq=%d is not a multiple of Hkv=%d", fn, p->Hq, p->Hkv);
+  if (p->dtype != LMH_F32 && p->dtype != LMH_F16 && p->dtype != LMH_BF16)
+    return fail(LMH_E_UNSUPPORTED, "%s: unknown dtype %d", fn, p->dtype);
+  if (p->head_map != LMH_HEADMAP_INTERLEAVED && p->head_map != LMH_HEADMAP_BLOCKED)
+    return fail(LMH_E_UNSUPPORTED, "%s: unknown head_map %d", fn, p->head_map);
+  const int vec = p->dtype == LMH_F32 ? 4 : 8;
+  if (p->D % vec != 0 || p->D > 256)
+    return fail(LMH_E_UNSUPPORTED, "%s: head dim %d must be a multiple of %d and <= 256", fn, p->D, vec);
+  if (p->num_splits < 0) return fail(LMH_E_SHAPE, "%s: negative num_splits", fn);
+  if (!(p->scale == p->scale)) return fail(LMH_E_SHAPE, "%s: scale is NaN", fn);
+  return LMH_OK;
+}
+
+int lmh_decode_attn(const lmh_decode_params *p) {
+  const int rc = decode_check(p, "lmh_decode_attn");
+  if (rc != LMH_OK) return rc;
+  const int32_t splits = p->num_splits == 0 ? lmh_decode_auto_splits(p->B, p->Hkv, p->Lmax) : p->num_splits;
+  return decode_launch(p, "lmh_decode_attn", splits, p->workspace, p->workspace_bytes);
+}
+
+// --------------------------------------------------------------------------------------------
+// decode attention for callers that cannot allocate: the split-KV partials live in a static device array
+// --------------------------------------------------------------------------------------------
+size_t lmh_static_scratch_bytes(void) { return LMH_STATIC_SCRATCH_BYTES; }
+
+int32_t lmh_decode_static_splits(int32_t B, int32_t Hq, int32_t Hkv, int32_t Lmax, int32_t D) {
+  int32_t splits = lmh_decode_auto_splits(B, Hkv, Lmax);
+  if (splits <= 0 || Hq <= 0 || D <= 0) return 0;
+  // halve the split count (double the keys per split) until the partials fit; one split needs none
+  while (splits > 1 && lmh_decode_workspace_bytes(B, Hq, Hkv, Lmax, D, splits) > LMH_STATIC_SCRATCH_BYTES)
+    splits = (splits + 1) / 2;
+  return splits;
+}
+
+int lmh_decode_attn_static(const lmh_decode_params *p) {
+  const char *fn = "lmh_decode_attn_static";
+  const int rc = decode_check(p, fn);
+  if (rc != LMH_OK) return rc;
+  const int32_t splits = p->num_splits == 0 ? lmh_decode_static_splits(p->B, p->Hq, p->Hkv, p->Lmax, p->D) : p->num_splits;
+  const size_t need = lmh_decode_workspace_bytes(p->B, p->Hq, p->Hkv, p->Lmax, p->D, splits);
+  if (need > LMH_STATIC_SCRATCH_BYTES)
+    return fail(LMH_E_WORKSPACE,
+                "%s: %d splits of B=%d Hq=%d D=%d need %zu bytes of partials, the static scratch holds %zu; "
+                "pass num_splits = 0 or a smaller count, or use lmh_decode_attn with a workspace",
+                fn, splits, p->B, p->Hq, p->D, need, (size_t)LMH_STATIC_SCRATCH_BYTES);
+  void *ws = nullptr;
+  if (splits > 1) {
+    const int rc_ws = static_scratch_for_current_device(&ws);
+    if (rc_ws != LMH_OK) return rc_ws;
+  }
+  // Nothing in the scratch has to start at zero: every partial slot the merge kernel reads was written by
+  // the split kernel of the same call (a result, or the "empty" marker), so no clearing is enqueued.
+  return decode_launch(p, fn, splits, ws, LMH_STATIC_SCRATCH_BYTES);
 }
 
 // --------------------------------------------------------------------------------------------

@@ -169,15 +169,23 @@ function workspace(bytes::Integer)
 end
 
 function execute_op!(out::HipArray{TO,3}, op::DecodeAttentionOp, q::HipArray{T,3}, kc::HipArray{T,4}, vc::HipArray{T,4},
-                     kv_len::HipArray{Int32,1}) where {TO,T}
+                     kv_len::HipArray{Int32,1}; static_scratch::Bool=false) where {TO,T}
     B, Hq, D = size(q)
     _, Hkv, Lmax, _ = size(kc)
+    out_f32 = Int32(TO === Float32 && T !== Float32)
+    if static_scratch
+        # lmh_decode_attn_static: no workspace, nothing allocated (split-KV partials in the library's static device array)
+        p = Ref(DecodeParams(out.ptr, q.ptr, kc.ptr, vc.ptr, Ptr{Int32}(kv_len.ptr), B, Hq, Hkv, Lmax, D, Z2, Z2, Z3, Z3,
+                             dtype_code(T), op.scale, op.head_map, out_f32, Int32(0), C_NULL, Csize_t(0), current_stream()))
+        check(ccall((:lmh_decode_attn_static, libluminal_hip), Cint, (Ref{DecodeParams},), p))
+        return out
+    end
     splits = ccall((:lmh_decode_auto_splits, libluminal_hip), Int32, (Int32, Int32, Int32), B, Hkv, Lmax)
     need = ccall((:lmh_decode_workspace_bytes, libluminal_hip), Csize_t, (Int32, Int32, Int32, Int32, Int32, Int32),
                  B, Hq, Hkv, Lmax, D, splits)
     ws = workspace(need)
     p = Ref(DecodeParams(out.ptr, q.ptr, kc.ptr, vc.ptr, Ptr{Int32}(kv_len.ptr), B, Hq, Hkv, Lmax, D, Z2, Z2, Z3, Z3,
-                         dtype_code(T), op.scale, op.head_map, Int32(TO === Float32 && T !== Float32), splits,
+                         dtype_code(T), op.scale, op.head_map, out_f32, splits,
                          ws === nothing ? C_NULL : ws.ptr, need, current_stream()))
     check(ccall((:lmh_decode_attn, libluminal_hip), Cint, (Ref{DecodeParams},), p))
     return out

@@ -23,7 +23,7 @@ def test_library_exports_every_declared_symbol(lm):
     lib = lm.binding.load()
     for name in header_functions():
         assert hasattr(lib, name), name
-    assert lib.lmh_version() == 101
+    assert lib.lmh_version() == 102
 
 
 def test_struct_layout_matches_header(lm):
@@ -95,6 +95,28 @@ def test_decode_workspace_and_split_heuristic(lm):
         chunk = -(-L // s)
         assert s == 1 or chunk >= 100  # never shreds the cache into tiny splits
         assert b.decode_workspace_bytes(B, 4 * Hkv, Hkv, L, 128, 0) == b.decode_workspace_bytes(B, 4 * Hkv, Hkv, L, 128, s)
+
+
+def test_static_scratch_decode_limits_are_checked_on_the_host(lm):
+    # the entry point without a workspace: its split count always fits the static array, and an explicit count
+    # that does not is refused before anything touches a GPU
+    b = lm.binding
+    cap = b.static_scratch_bytes()
+    assert cap == 32 << 20
+    for (B, Hq, Hkv, L, D) in [(16, 32, 8, 4096, 128), (64, 32, 8, 32768, 128), (64, 64, 1, 4096, 64), (1, 8, 8, 17, 64),
+                               (512, 128, 8, 65536, 256)]:
+        s = b.decode_static_splits(B, Hq, Hkv, L, D)
+        assert 1 <= s <= b.decode_auto_splits(B, Hkv, L)
+        assert b.decode_workspace_bytes(B, Hq, Hkv, L, D, s) <= cap
+    assert b.decode_static_splits(16, 32, 8, 4096, 128) == b.decode_auto_splits(16, 8, 4096)  # fits as it is
+    assert b.decode_static_splits(64, 32, 8, 32768, 128) < b.decode_auto_splits(64, 8, 32768)
+    p = _dec(lm, B=64, Hq=32, Hkv=8, Lmax=32768, D=128, num_splits=64)
+    with pytest.raises(lm.LuminalHipError) as e:
+        b.decode_attn_static(p)
+    assert e.value.code == b.LMH_E_WORKSPACE and "lmh_decode_attn_static" in str(e.value)
+    with pytest.raises(lm.LuminalHipError) as e:
+        b.decode_attn_static(_dec(lm, q=None))
+    assert e.value.code == b.LMH_E_NULL and "lmh_decode_attn_static" in str(e.value)
 
 
 def test_no_device_is_reported_not_fatal(lm):
