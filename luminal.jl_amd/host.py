@@ -525,7 +525,9 @@ def execute_with_capture(device, f, cache):
     recording was invalidated by transient workspaces that were freed); here `f(stream)` must enqueue only on
     the stream it is given and only on buffers that outlive the recording. Every call runs `f`'s work exactly
     once: the first call runs it eagerly (the library's first-use set-up stays outside the recording), the second
-    records and replays, later ones replay."""
+    records and replays, later ones replay. Measured on an MI355X a recording of a decode step's three kernels
+    replays no faster than the three launches (57 vs 52 us at B=16, L=4096), so this is there for parity with the
+    reference's interface and for hosts whose per-op dispatch is slow, not as a speed-up."""
     if not isinstance(device, HIPDevice):
         return f(None)
     if "hip_exec" not in cache:
@@ -539,8 +541,8 @@ def execute_with_capture(device, f, cache):
             try:
                 f(stream)
             except Exception:
-                try:
-                    binding.graph_capture_end(stream)  # leave the stream usable; the recording is dropped
+                try:  # leave the stream usable; a recording that still instantiated is dropped
+                    binding.graph_destroy(binding.graph_capture_end(stream))
                 except binding.LuminalHipError:
                     pass
                 raise

@@ -9,6 +9,12 @@
 #   * an execute_with_capture method that records a step into a HIP graph     (src/Device.jl:108-121)
 #   * DecodeAttentionOp + decode_attention, the fused form of the cached single-token attention
 #     subgraph (src/Whisper.jl:584-620) with the GQA head sharing of src/NN.jl:305-317
+#   * RotaryEmbeddingOp / KVAppendOp graph nodes (apply_rotary_embeddings, src/NN.jl:253-303; _kv_scatter,
+#     src/Whisper.jl:552-570) whose positions are device tensors, so one graph serves every decode position
+#   * the array methods Luminal's interpreter and compiled graphs apply to whatever to_device returned
+#     (length, reshape, similar, copyto!: src/Execution.jl:92-97, :253; src/Compiler.jl:82-90)
+#   * compile_hip(graph): Luminal.compile (src/Compiler.jl:181-255) with the node buffers on the device,
+#     returning Luminal's own CompiledGraph
 # and calls the C ABI of include/luminal_hip.h through `ccall`. There are no AMDGPU.jl kernels here.
 #
 # Layout: Luminal tensors are column-major (B,H,S,D) arrays (B fastest). The library takes
@@ -17,8 +23,9 @@
 module LuminalHIP
 
 using Luminal
-import Luminal: AbstractDevice, Op, FlashAttentionOp, GraphTensor, add_op!, realized_dims,
+import Luminal: AbstractDevice, Op, FlashAttentionOp, GraphTensor, add_op!, realized_dims, eval_dim, realize_view,
                 to_device, from_device, execute_op, execute_op!, execute_with_capture
+# Luminal exports an Op called `Function`; the Julia type is always written Base.Function here.
 
 const libluminal_hip = get(ENV, "LUMINAL_HIP_LIB", joinpath(@__DIR__, "..", "lib", "libluminal_hip.so"))
 
@@ -27,6 +34,12 @@ const LMH_F32, LMH_F16, LMH_BF16 = Int32(0), Int32(1), Int32(2)
 const HEADMAP_INTERLEAVED, HEADMAP_BLOCKED = Int32(0), Int32(1)
 # bf16 tensors are carried as UInt16 bit patterns (Julia has no native BFloat16 array type)
 struct BF16Bits; bits::UInt16; end
+function BF16Bits(x::Float32)           # round to nearest even, NaN stays NaN
+    u = reinterpret(UInt32, x)
+    isnan(x) && return BF16Bits(((u >> 16) | 0x00000040) % UInt16)
+    return BF16Bits(((u + 0x00007fff + ((u >> 16) & 0x00000001)) >> 16) % UInt16)
+end
+Base.Float32(b::BF16Bits) = reinterpret(Float32, UInt32(b.bits) << 16)
 dtype_code(::Type{Float32}) = LMH_F32
 dtype_code(::Type{Float16}) = LMH_F16
 dtype_code(::Type{BF16Bits}) = LMH_BF16
@@ -69,15 +82,38 @@ mutable struct HipArray{T,N}
     # same memory under other dims (Base.reshape); frees nothing and keeps the owner reachable
     HipArray{T,N}(ptr::Ptr{Cvoid}, dims::NTuple{N,Int}, owner) where {T,N} = new{T,N}(ptr, dims, owner)
 end
+# ---- what Luminal applies to its arrays on the interpreter and compiled paths ----
+# length: src/Execution.jl:95, src/Compiler.jl:86; similar: src/Execution.jl:253; size / ndims / eltype: executors
 Base.size(a::HipArray) = a.dims
 Base.size(a::HipArray, i::Integer) = a.dims[i]
 Base.length(a::HipArray) = prod(a.dims)
+Base.ndims(::HipArray{T,N}) where {T,N} = N
 Base.eltype(::HipArray{T}) where {T} = T
 Base.similar(a::HipArray{T,N}) where {T,N} = HipArray{T,N}(a.dims)
+Base.similar(a::HipArray{T}, dims::NTuple{N,Int}) where {T,N} = HipArray{T,N}(dims)
+owner(a::HipArray) = a.parent === nothing ? a : a.parent
+
+"Freshly allocated, zero-filled device array (zeros(T, dims...) of src/Compiler.jl:227)."
+function zeros_hip(::Type{T}, dims::NTuple{N,Int}) where {T,N}
+    a = HipArray{T,N}(dims)
+    check(ccall((:lmh_memset, libluminal_hip), Cint, (Ptr{Cvoid}, Cint, Csize_t, Ptr{Cvoid}),
+                a.ptr, 0, max(prod(dims), 1) * sizeof(T), C_NULL))
+    return a
+end
+
+# Host values in the element type of the device array.
+to_storage(::Type{T}, x::AbstractArray) where {T} = eltype(x) === T ? x : convert_elements(T, x)
+convert_elements(::Type{T}, x::AbstractArray) where {T<:Number} = T.(x)
+convert_elements(::Type{BF16Bits}, x::AbstractArray{UInt16}) = BF16Bits.(x)       # already bit patterns
+convert_elements(::Type{BF16Bits}, x::AbstractArray) = BF16Bits.(Float32.(x))      # values: round to bf16
+
+# Column-major (d1 fastest) host array -> the same values with the dimension order reversed, i.e. the
+# memory order of row-major [d1, ..., dN] (dN contiguous), and back.
+reverse_dims(x::AbstractArray{T,N}) where {T,N} = N <= 1 ? Array(x) : Array(permutedims(x, ntuple(i -> N + 1 - i, N)))
 
 "Host array -> device, reversing the dimension order so that D becomes the contiguous axis."
 function to_device(data::AbstractArray{T,N}, ::HIPDevice) where {T,N}
-    host = Array(permutedims(data, ntuple(i -> N + 1 - i, N)))
+    host = reverse_dims(data)
     dev = HipArray{T,N}(size(data))
     check(ccall((:lmh_memcpy_h2d, libluminal_hip), Cint, (Ptr{Cvoid}, Ptr{Cvoid}, Csize_t, Ptr{Cvoid}),
                 dev.ptr, host, sizeof(host), C_NULL))
@@ -90,8 +126,49 @@ function from_device(a::HipArray{T,N}) where {T,N}
     host = Array{T,N}(undef, reverse(a.dims))
     check(ccall((:lmh_memcpy_d2h, libluminal_hip), Cint, (Ptr{Cvoid}, Ptr{Cvoid}, Csize_t, Ptr{Cvoid}),
                 host, a.ptr, sizeof(host), C_NULL))
-    return permutedims(host, ntuple(i -> N + 1 - i, N))
+    return reverse_dims(host)
 end
+
+# Base.reshape(data, dims...) is the first thing realize_view does to every node input (src/Execution.jl:94-97,
+# :101-104; called at :639 and src/Compiler.jl:252). Equal dims (the buffer "already matches logical size") and
+# dims that differ only in singleton axes are the same memory: a view that keeps the owner alive. A reshape
+# that regroups axes is a different permutation of a row-major buffer than of Julia's column-major arrays, so
+# it goes through the host (correct, slow, and no longer a view).
+Base.reshape(a::HipArray, dims::Int...) = Base.reshape(a, dims)
+function Base.reshape(a::HipArray{T}, dims::NTuple{N,Int}) where {T,N}
+    prod(dims) == length(a) ||
+        throw(DimensionMismatch("reshape: HipArray of size $(a.dims) has $(length(a)) elements, $(dims) needs $(prod(dims))"))
+    dims == a.dims && return a
+    if [d for d in dims if d != 1] == [d for d in a.dims if d != 1]
+        return HipArray{T,N}(a.ptr, dims, owner(a))
+    end
+    return to_device(Base.reshape(from_device(a), dims), HIPDevice())
+end
+"true when `v` is `a` itself or a view of `a`'s memory (what compile_hip requires of captured step arguments)"
+same_memory(v::HipArray, a::HipArray) = v.ptr == a.ptr && length(v) == length(a)
+same_memory(v, a) = v === a
+
+# copyto!(cg.results[k], v) is how a compiled graph takes its inputs (src/Compiler.jl:82-90), and how compile
+# fills constants (:229-234). Like copyto! between Arrays it copies in linear (column-major) order.
+function Base.copyto!(dst::HipArray{T,N}, src::AbstractArray) where {T,N}
+    length(src) == length(dst) ||
+        throw(DimensionMismatch("copyto!: HipArray has $(length(dst)) elements, the source $(length(src))"))
+    shaped = size(src) == dst.dims ? src : Base.reshape(src, dst.dims)
+    host = reverse_dims(to_storage(T, shaped))
+    check(ccall((:lmh_memcpy_h2d, libluminal_hip), Cint, (Ptr{Cvoid}, Ptr{Cvoid}, Csize_t, Ptr{Cvoid}),
+                dst.ptr, host, sizeof(host), C_NULL))
+    return dst
+end
+function Base.copyto!(dst::HipArray{T}, src::HipArray{T}) where {T}
+    length(src) == length(dst) ||
+        throw(DimensionMismatch("copyto!: HipArray has $(length(dst)) elements, the source $(length(src))"))
+    [d for d in dst.dims if d != 1] == [d for d in src.dims if d != 1] ||
+        error("copyto! between HipArrays of sizes $(src.dims) and $(dst.dims) would regroup axes; reshape on the host")
+    check(ccall((:lmh_memcpy_d2d, libluminal_hip), Cint, (Ptr{Cvoid}, Ptr{Cvoid}, Csize_t, Ptr{Cvoid}),
+                dst.ptr, src.ptr, length(dst) * sizeof(T), current_stream()))
+    return dst
+end
+Base.copyto!(dst::Array, src::HipArray) = copyto!(dst, from_device(src))
 
 # ------------------------------------------------------------------------------------------
 # parameter blocks (field order and types mirror include/luminal_hip.h)
@@ -149,6 +226,10 @@ struct DecodeAttentionOp <: Op
     head_map::Int32
 end
 
+"""
+q: (B,H,D), or (B,H,1,D) as the projections of one decode step produce it; caches (B,Hkv,max_seq,D); kv_len (B,)
+Int32. The output has q's shape.
+"""
 function decode_attention(q::GraphTensor, k_cache::GraphTensor, v_cache::GraphTensor, kv_len::GraphTensor;
                           scale=nothing, head_map::Int32=HEADMAP_INTERLEAVED)
     q_dims = realized_dims(q.shape)
@@ -188,6 +269,16 @@ function execute_op!(out::HipArray{TO,3}, op::DecodeAttentionOp, q::HipArray{T,3
                          dtype_code(T), op.scale, op.head_map, out_f32, splits,
                          ws === nothing ? C_NULL : ws.ptr, need, current_stream()))
     check(ccall((:lmh_decode_attn, libluminal_hip), Cint, (Ref{DecodeParams},), p))
+    return out
+end
+
+# q and out as (B,H,1,D): the same memory as (B,H,D)
+function execute_op!(out::HipArray{TO,4}, op::DecodeAttentionOp, q::HipArray{T,4}, kc::HipArray{T,4}, vc::HipArray{T,4},
+                     kv_len::HipArray{Int32,1}; static_scratch::Bool=false) where {TO,T}
+    size(q, 3) == 1 || error("DecodeAttentionOp takes one query token per sequence; got q of size $(size(q))")
+    size(out) == size(q) || error("DecodeAttentionOp: output shape $(size(out)) differs from q shape $(size(q))")
+    dims3 = (size(q, 1), size(q, 2), size(q, 4))
+    execute_op!(Base.reshape(out, dims3), op, Base.reshape(q, dims3), kc, vc, kv_len; static_scratch=static_scratch)
     return out
 end
 
@@ -241,6 +332,69 @@ function kv_append!(kc::HipArray{T,4}, vc::HipArray{T,4}, k_new::HipArray{T,4}, 
 end
 
 # ------------------------------------------------------------------------------------------
+# The same two operators as graph nodes, so that a decode step is a Luminal graph whose positions are
+# tensors: one graph (interpreted or compiled) then serves every position, where the reference bakes
+# step_pos into the slices of one graph per position (src/Whisper.jl:673-675, src/Decoding.jl:98-106).
+# ------------------------------------------------------------------------------------------
+"apply_rotary_embeddings(input, prev_seq; base) (src/NN.jl:253-303) as one node; inputs (x,) or (x, pos0)."
+struct RotaryEmbeddingOp <: Op
+    prev_seq::Int32
+    base::Float32
+end
+
+"""
+x: (B,H,S,D). Row s of sequence b is rotated by position prev_seq + s, or pos0[b] + s when the Int32 (B,)
+tensor pos0 is given. Output shape = x's.
+"""
+function rotary_embedding(x::GraphTensor; prev_seq::Integer=0, base::Real=10000.0f0,
+                          pos0::Union{Nothing,GraphTensor}=nothing)
+    inputs = [(x.id, 0, x.shape)]
+    pos0 === nothing || push!(inputs, (pos0.id, 0, pos0.shape))
+    return add_op!(x.graph_ref, RotaryEmbeddingOp(Int32(prev_seq), Float32(base)), inputs, x.shape)
+end
+
+function execute_op!(out::HipArray{T,4}, op::RotaryEmbeddingOp, x::HipArray{T,4},
+                     pos0::Union{Nothing,HipArray{Int32,1}}=nothing) where {T}
+    size(out) == size(x) || error("RotaryEmbeddingOp: output shape $(size(out)) differs from input shape $(size(x))")
+    B, H, S, D = size(x)
+    p = Ref(RopeParams(out.ptr, x.ptr, pos0 === nothing ? Ptr{Int32}(C_NULL) : Ptr{Int32}(pos0.ptr), op.prev_seq,
+                       B, H, S, D, Z3, Z3, dtype_code(T), op.base, Int32(0), current_stream()))
+    check(ccall((:lmh_rope, libluminal_hip), Cint, (Ref{RopeParams},), p))
+    return out
+end
+execute_op(op::RotaryEmbeddingOp, x::HipArray, pos0::HipArray...) = execute_op!(similar(x), op, x, pos0...)
+
+"""
+In-place cache update as a node; inputs (k_cache, v_cache, k_new, v_new, pos) plus, with rope_q, this step's
+queries. The node's value IS its k_cache input (the same buffer, rows pos[b] .. pos[b]+T-1 overwritten, K rotated
+on the way in when rope_k); v_cache and the queries are updated in place as well, so later nodes that read them
+through their own ids see the new contents — nodes run in graph order (src/Execution.jl:630, src/Compiler.jl:92-96).
+"""
+struct KVAppendOp <: Op
+    rope_k::Bool
+    rope_q::Bool
+    base::Float32
+end
+
+function kv_cache_append(k_cache::GraphTensor, v_cache::GraphTensor, k_new::GraphTensor, v_new::GraphTensor,
+                         pos::GraphTensor; rope_k::Bool=false, base::Real=10000.0f0,
+                         q::Union{Nothing,GraphTensor}=nothing)
+    inputs = [(k_cache.id, 0, k_cache.shape), (v_cache.id, 0, v_cache.shape), (k_new.id, 0, k_new.shape),
+              (v_new.id, 0, v_new.shape), (pos.id, 0, pos.shape)]
+    q === nothing || push!(inputs, (q.id, 0, q.shape))
+    return add_op!(k_cache.graph_ref, KVAppendOp(rope_k, q !== nothing, Float32(base)), inputs, k_cache.shape)
+end
+
+function execute_op!(out::HipArray{T,4}, op::KVAppendOp, kc::HipArray{T,4}, vc::HipArray{T,4}, k_new::HipArray{T,4},
+                     v_new::HipArray{T,4}, pos::HipArray{Int32,1}, q::Union{Nothing,HipArray{T,4}}=nothing) where {T}
+    same_memory(out, kc) || error("KVAppendOp works in place: its output buffer must be its k_cache input")
+    (q !== nothing) == op.rope_q || error("KVAppendOp: rope_q is $(op.rope_q) but the node has $(q === nothing ? 5 : 6) inputs")
+    kv_append!(kc, vc, k_new, v_new, pos; rope_k=op.rope_k, base=op.base, q=q)
+    return out
+end
+execute_op(op::KVAppendOp, kc::HipArray, rest::HipArray...) = execute_op!(kc, op, kc, rest...)
+
+# ------------------------------------------------------------------------------------------
 # What the attention layers do between their projections, as fused calls on device arrays.
 # SelfAttention (src/NN.jl:352-382) = rotary embedding of Q and K, repeat_kv, scaled causal softmax
 # attention; the fused op reads the Hkv key/value heads directly in the head order repeat_kv produces
@@ -277,16 +431,105 @@ function cached_self_attention_core!(out::HipArray{TO,3}, q::HipArray{T,4}, k_ne
     return execute_op!(out, DecodeAttentionOp(s, head_map), q3, kc, vc, kv_len)
 end
 
+# The same two cores as graph builders (GraphTensor in, GraphTensor out), for model code that builds a Luminal graph.
+function self_attention_core(q::GraphTensor, k::GraphTensor, v::GraphTensor; causal::Bool=true, prev_seq::Integer=0,
+                             rope_base=nothing, scale=nothing)
+    if rope_base !== nothing
+        q = rotary_embedding(q; prev_seq=prev_seq, base=rope_base)
+        k = rotary_embedding(k; prev_seq=prev_seq, base=rope_base)
+    end
+    # FlashAttentionOp reads the Hkv key/value heads in the order repeat_kv produces (src/NN.jl:305-317)
+    return Luminal.flash_attention(q, k, v; scale=scale, causal=causal)
+end
+
+"Returns (out, k_cache): `out` has q's shape (B,Hq,1,D); `k_cache` is the append node (the updated cache)."
+function cached_self_attention_core(q::GraphTensor, k_new::GraphTensor, v_new::GraphTensor, k_cache::GraphTensor,
+                                    v_cache::GraphTensor, pos::GraphTensor, kv_len::GraphTensor;
+                                    rope_base=nothing, scale=nothing, head_map::Int32=HEADMAP_INTERLEAVED)
+    kc = kv_cache_append(k_cache, v_cache, k_new, v_new, pos; rope_k=(rope_base !== nothing),
+                         base=something(rope_base, 10000.0f0), q=(rope_base !== nothing ? q : nothing))
+    # q and v_cache were updated in place by the append node, which precedes this one in graph order
+    out = decode_attention(q, kc, v_cache, kv_len; scale=scale, head_map=head_map)
+    return out, kc
+end
+
+# ------------------------------------------------------------------------------------------
+# compile_hip(graph): Luminal.compile (src/Compiler.jl:181-255) for graphs of the operators above, with the
+# node buffers on the device. Luminal.compile itself cannot serve: it allocates host `zeros` for every
+# non-CUDA device (:224-228) and its step closures capture those host arrays at compile time (:250-255), so
+# nothing done to cg.results afterwards reaches them. The result is Luminal's own CompiledGraph, so calling
+# it is the reference's code (src/Compiler.jl:81-100): length and copyto! on the node buffers, then
+# execute_with_capture(device, run_graph, cache) — all of which have HipArray / HIPDevice methods above.
+#   eltypes: node id => element type for input nodes (default Float32; inputs consumed as positions or
+#            lengths default to Int32) and, optionally, for op nodes (default: the type of their first
+#            input; Float32 on a half-precision attention node asks for the fp32 result).
+# ------------------------------------------------------------------------------------------
+const DeviceOp = Union{FlashAttentionOp,DecodeAttentionOp,RotaryEmbeddingOp,KVAppendOp}
+is_input_node(op) = op isa Luminal.Function && op.name == "InputTensor"
+
+function compile_hip(graph::Luminal.Graph; eltypes::AbstractDict=Dict{Int,DataType}())
+    functional() || error("compile_hip: no gfx950 device answers libluminal_hip.so")
+    n = length(graph.nodes)
+    int_inputs = Set{Int}()                      # nodes read as Int32 positions / lengths
+    for node in graph.nodes
+        op = node.op
+        op isa DecodeAttentionOp && push!(int_inputs, node.inputs[4][1])
+        op isa KVAppendOp && push!(int_inputs, node.inputs[5][1])
+        op isa RotaryEmbeddingOp && length(node.inputs) >= 2 && push!(int_inputs, node.inputs[2][1])
+    end
+    # 1. allocate results (src/Compiler.jl:218-235)
+    eltype_of = Vector{DataType}(undef, n)
+    results = Vector{Any}(undef, n)
+    for (node_id, node) in enumerate(graph.nodes)
+        op = node.op
+        dims = Tuple(Int.(eval_dim.(realized_dims(graph.shapes[node_id]))))
+        if is_input_node(op)
+            eltype_of[node_id] = get(eltypes, node_id, node_id in int_inputs ? Int32 : Float32)
+            results[node_id] = zeros_hip(eltype_of[node_id], dims)
+        elseif op isa KVAppendOp                 # in place: the node's value is its k_cache input
+            eltype_of[node_id] = eltype_of[node.inputs[1][1]]
+            results[node_id] = results[node.inputs[1][1]]
+        elseif op isa DeviceOp
+            eltype_of[node_id] = get(eltypes, node_id, eltype_of[node.inputs[1][1]])
+            results[node_id] = zeros_hip(eltype_of[node_id], dims)
+        else
+            error("compile_hip: node $node_id is a $(typeof(op)), which has no executor in libluminal_hip.so; this " *
+                  "backend covers the attention path (FlashAttentionOp, DecodeAttentionOp, RotaryEmbeddingOp, KVAppendOp)")
+        end
+    end
+    # 2. one in-place step per op; arguments are views of the persistent buffers, captured once (:250-255)
+    steps = Base.Function[]
+    for (node_id, node) in enumerate(graph.nodes)
+        op = node.op
+        is_input_node(op) && continue
+        step_args = [realize_view(results[id], st) for (id, _, st) in node.inputs]
+        for (k, (id, _, _)) in enumerate(node.inputs)
+            same_memory(step_args[k], results[id]) ||
+                error("compile_hip: input $k of node $node_id is a reshape that regroups axes; not supported on device buffers")
+        end
+        target_buf = results[node_id]
+        push!(steps, (results, device) -> execute_op!(target_buf, op, step_args...))
+    end
+    return Luminal.CompiledGraph(steps, results, Dict{Symbol,Any}())
+end
+
+"From the next call on, run the compiled steps as one recorded HIP graph (see execute_with_capture below)."
+enable_capture!(cg::Luminal.CompiledGraph) = (cg.cache[:hip_capture] = true; cg)
+
 # ------------------------------------------------------------------------------------------
 # execute_with_capture(device, f, cache) (src/Device.jl:108-121; called by the compiled step closure,
 # src/Compiler.jl:98). The reference stubs its CUDA method out because transient workspaces freed after
 # the recording invalidated it. Here every buffer a step touches outlives the recording (the caches and
 # results belong to the compiled graph, the split-KV workspace to this module and it only grows before
 # the recording: the first call runs eagerly), and positions / lengths are device tensors, so one
-# recording serves every decode position. Every call runs f's work exactly once.
+# recording serves every decode position. Every call runs f's work exactly once. Off unless the cache holds
+# :hip_capture => true (enable_capture!(cg) for a compiled graph).
 # `f` must enqueue only through the executors of this module and must not upload or download.
 # ------------------------------------------------------------------------------------------
 function execute_with_capture(::HIPDevice, f, cache::Dict)
+    # Opt-in (enable_capture!): on this runtime a recording of three kernel launches replays no faster than the
+    # launches themselves, so the default is the plain loop, like the reference's stub.
+    get(cache, :hip_capture, false) || return f()
     if !haskey(cache, :hip_exec)
         if !get(cache, :hip_warm, false)
             cache[:hip_warm] = true
@@ -331,10 +574,12 @@ function release_capture!(cache::Dict)
     end
     delete!(cache, :hip_warm)
     delete!(cache, :hip_workspace)
+    delete!(cache, :hip_capture)
     return nothing
 end
 
-export HIPDevice, HipArray, release_capture!, DecodeAttentionOp, decode_attention, get_device, functional, rope!, kv_append!,
-       self_attention_core!, cached_self_attention_core!
+export HIPDevice, HipArray, BF16Bits, release_capture!, enable_capture!, compile_hip, DecodeAttentionOp, decode_attention,
+       RotaryEmbeddingOp, rotary_embedding, KVAppendOp, kv_cache_append, get_device, functional, rope!, kv_append!,
+       self_attention_core!, cached_self_attention_core!, self_attention_core, cached_self_attention_core
 
 end # module

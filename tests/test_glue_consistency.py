@@ -94,3 +94,185 @@ def test_julia_glue_matches_the_header():
     codes = re.search(r"const LMH_F32, LMH_F16, LMH_BF16 = Int32\((\d)\), Int32\((\d)\), Int32\((\d)\)", text)
     want = dict(re.findall(r"#define (LMH_(?:F32|F16|BF16)) (\d+)", header_text()))
     assert codes and list(codes.groups()) == [want["LMH_F32"], want["LMH_F16"], want["LMH_BF16"]]
+
+
+# ---------------------------------------------------------------------------------------------
+# Static walk of the Julia glue (no Julia here to run it): every function Luminal applies to the arrays
+# that to_device returned, on the interpreter and compiled-graph call paths, must have a HipArray method.
+# ---------------------------------------------------------------------------------------------
+# (what Luminal calls, reference file, line, text expected on that line, regex of the glue's method)
+ARRAY_PROTOCOL = [
+    ("to_device(inputs, device)", "src/Execution.jl", 621, "to_device(initial_inputs, device)",
+     r"^function to_device\(data::AbstractArray\{T,N\}, ::HIPDevice\)"),
+    ("length(data) in realize_view", "src/Execution.jl", 95, "length(data)", r"^Base\.length\(a::HipArray\)"),
+    ("Base.reshape(data, dims...) in realize_view", "src/Execution.jl", 96, "Base.reshape(data,",
+     r"^Base\.reshape\(a::HipArray, dims::Int\.\.\.\)"),
+    ("Base.reshape(data, fill(1, n)...) for one-element data", "src/Execution.jl", 103, "Base.reshape(data, fill(1",
+     r"^function Base\.reshape\(a::HipArray\{T\}, dims::NTuple\{N,Int\}\)"),
+    ("realize_view on every interpreter input", "src/Execution.jl", 639, "realize_view(raw_data, st)", None),
+    ("execute_op(op, input_values...)", "src/Execution.jl", 652, "execute_op(op, input_values...)",
+     r"^function execute_op\(op::FlashAttentionOp, q::HipArray, k::HipArray, v::HipArray\)"),
+    ("similar(q) in execute_op", "src/Execution.jl", 253, "similar(q)", r"^Base\.similar\(a::HipArray\{T,N\}\)"),
+    ("execute_op!(out, op, q, k, v)", "src/Execution.jl", 565, "function execute_op!(out, op::FlashAttentionOp",
+     r"^function execute_op!\(out::HipArray\{TO,4\}, op::FlashAttentionOp, q::HipArray\{T,4\}"),
+    ("from_device(results[id])", "src/Execution.jl", 662, "from_device(results[id])",
+     r"^function from_device\(a::HipArray\{T,N\}\)"),
+    ("length(cg.results[k]) in a compiled call", "src/Compiler.jl", 86, "length(cg.results[k])",
+     r"^Base\.length\(a::HipArray\)"),
+    ("copyto!(cg.results[k], v)", "src/Compiler.jl", 89, "copyto!(cg.results[k], v)",
+     r"^function Base\.copyto!\(dst::HipArray\{T,N\}, src::AbstractArray\)"),
+    ("copyto!(results[id], to_device(...)) for constants", "src/Compiler.jl", 230, "copyto!(results[node_id], to_device(",
+     r"^function Base\.copyto!\(dst::HipArray\{T\}, src::HipArray\{T\}\)"),
+    ("execute_with_capture(device, run_graph, cg.cache)", "src/Compiler.jl", 98, "execute_with_capture(device, run_graph, cg.cache)",
+     r"^function execute_with_capture\(::HIPDevice, f, cache::Dict\)"),
+    ("realize_view(results[id], st) captured by the step closure", "src/Compiler.jl", 252, "realize_view(results[id], st)",
+     r"step_args = \[realize_view\(results\[id\], st\) for \(id, _, st\) in node\.inputs\]"),
+    ("execute_op!(target_buf, op, step_args...)", "src/Compiler.jl", 254, "execute_op!(target_buf, op, step_args...)",
+     r"push!\(steps, \(results, device\) -> execute_op!\(target_buf, op, step_args\.\.\.\)\)"),
+    ("CompiledGraph(steps, results, cache)", "src/Compiler.jl", 75, "struct CompiledGraph",
+     r"return Luminal\.CompiledGraph\(steps, results, Dict\{Symbol,Any\}\(\)\)"),
+]
+EXTRA_METHODS = [  # used by the glue's own executors on HipArray arguments
+    r"^Base\.size\(a::HipArray\)", r"^Base\.size\(a::HipArray, i::Integer\)", r"^Base\.ndims\(::HipArray\{T,N\}\)",
+    r"^Base\.eltype\(::HipArray\{T\}\)", r"^to_device\(data::HipArray, ::HIPDevice\)",
+    r"^function compile_hip\(graph::Luminal\.Graph",
+]
+REFERENCE = "/root/reference"
+
+
+def glue_text():
+    return open(os.path.join(ROOT, "luminal.jl_amd", "julia", "LuminalHIP.jl")).read()
+
+
+def test_glue_defines_every_array_method_the_reference_call_paths_use():
+    text = glue_text()
+    for what, ref_file, ref_line, ref_text, pattern in ARRAY_PROTOCOL:
+        if pattern is not None:
+            assert re.search(pattern, text, flags=re.M), "no HipArray method for: %s (%s:%d)" % (what, ref_file, ref_line)
+    for pattern in EXTRA_METHODS:
+        assert re.search(pattern, text, flags=re.M), pattern
+    # where a checkout of the reference is at hand, the cited lines must say what this table says they do
+    if os.path.isdir(REFERENCE):
+        for what, ref_file, ref_line, ref_text, _ in ARRAY_PROTOCOL:
+            lines = open(os.path.join(REFERENCE, ref_file)).read().split("\n")
+            window = "\n".join(lines[max(ref_line - 3, 0):ref_line + 2])
+            assert ref_text in window, "%s:%d does not contain %r" % (ref_file, ref_line, ref_text)
+
+
+def test_glue_graph_nodes_have_builders_and_executors():
+    # N1 / N2 / N4 on the Julia side: the rotary embedding and the cache append are graph nodes with an Op struct,
+    # a builder that calls add_op!, an in-place executor and an allocating one; compile_hip knows all four ops
+    text = glue_text()
+    for op, builder in (("DecodeAttentionOp", "decode_attention"), ("RotaryEmbeddingOp", "rotary_embedding"),
+                        ("KVAppendOp", "kv_cache_append")):
+        assert re.search(r"^struct %s <: Op$" % op, text, flags=re.M), op
+        body = re.search(r"^function %s\(.*?^end$" % builder, text, flags=re.M | re.S)
+        assert body and "add_op!(" in body.group(0) and op + "(" in body.group(0), builder
+        assert re.search(r"^function execute_op!\(out::HipArray\{\w+,\d\}, op::%s," % op, text, flags=re.M), op
+        assert re.search(r"^execute_op\(op::%s, " % op, text, flags=re.M), op
+    assert re.search(r"^const DeviceOp = Union\{FlashAttentionOp,DecodeAttentionOp,RotaryEmbeddingOp,KVAppendOp\}$", text,
+                     flags=re.M)
+    exported = re.search(r"^export (.*?)\n\n", text, flags=re.M | re.S).group(1)
+    for name in ("compile_hip", "HipArray", "HIPDevice", "rotary_embedding", "kv_cache_append", "decode_attention",
+                 "cached_self_attention_core", "self_attention_core", "enable_capture!"):
+        assert name in re.split(r"[,\s]+", exported), name
+
+
+def _strip_julia(text):
+    """Julia source with comments and string contents blanked (interpolations included), newlines kept."""
+    out, i, n = [], 0, len(text)
+    while i < n:
+        c = text[i]
+        if text.startswith('"""', i):
+            j = text.index('"""', i + 3)
+            out.append("".join(ch if ch == "\n" else " " for ch in text[i:j + 3]))
+            i = j + 3
+        elif c == '"':
+            j = i + 1
+            depth = 0
+            while j < n and not (text[j] == '"' and depth == 0):
+                if text[j] == "\\":
+                    j += 1
+                elif text.startswith("$(", j):
+                    depth += 1
+                    j += 1
+                elif text[j] == "(" and depth > 0:
+                    depth += 1
+                elif text[j] == ")" and depth > 0:
+                    depth -= 1
+                j += 1
+            out.append(" " * (j + 1 - i))
+            i = j + 1
+        elif c == "#":
+            j = text.find("\n", i)
+            j = n if j < 0 else j
+            out.append(" " * (j - i))
+            i = j
+        else:
+            out.append(c)
+            i += 1
+    return "".join(out)
+
+
+def test_glue_blocks_and_brackets_balance():
+    # a syntax slip (a missing `end`, an unclosed bracket) would otherwise go unnoticed until someone runs Julia
+    code = _strip_julia(glue_text())
+    depth_brackets, blocks = [], []
+    openers = {"function", "struct", "if", "for", "while", "try", "let", "begin", "module", "macro", "quote", "do"}
+    for m in re.finditer(r"[A-Za-z_!][A-Za-z_0-9!]*|[\[\](){}]", code):
+        tok = m.group(0)
+        if tok in "([{":
+            depth_brackets.append(tok)
+        elif tok in ")]}":
+            assert depth_brackets, "unmatched %s at offset %d" % (tok, m.start())
+            assert {"(": ")", "[": "]", "{": "}"}[depth_brackets.pop()] == tok, "bracket mismatch at offset %d" % m.start()
+        elif depth_brackets:
+            continue  # comprehensions (`for`, `if`) and `end` as an index live inside brackets
+        elif tok in openers:
+            if tok == "struct" and blocks and blocks[-1] == "mutable":
+                blocks[-1] = "struct"
+            else:
+                blocks.append(tok)
+        elif tok == "mutable":
+            blocks.append("mutable")
+        elif tok == "end":
+            assert blocks, "`end` without an open block at offset %d" % m.start()
+            blocks.pop()
+    assert not depth_brackets and not blocks, (depth_brackets, blocks)
+
+
+def _split_top_level(s):
+    parts, depth, cur = [], 0, []
+    for ch in s:
+        if ch in "([{":
+            depth += 1
+        elif ch in ")]}":
+            depth -= 1
+        if ch == "," and depth == 0:
+            parts.append("".join(cur).strip())
+            cur = []
+        else:
+            cur.append(ch)
+    if "".join(cur).strip():
+        parts.append("".join(cur).strip())
+    return parts
+
+
+def test_glue_ccalls_pass_as_many_arguments_as_the_header_declares():
+    code = _strip_julia(glue_text())
+    protos = {name: args for name, args in re.findall(r"\b(lmh_\w+)\s*\(([^)]*)\)\s*;", header_text())}
+    seen = 0
+    for m in re.finditer(r"ccall\(", code):
+        i, depth = m.end(), 1
+        while depth:
+            depth += {"(": 1, ")": -1}.get(code[i], 0)
+            i += 1
+        parts = _split_top_level(code[m.end():i - 1])
+        name = re.match(r"\(:(lmh_\w+)", parts[0]).group(1)
+        types = _split_top_level(parts[2].strip()[1:-1])
+        values = parts[3:]
+        assert len(types) == len(values), "ccall of %s: %d types, %d values" % (name, len(types), len(values))
+        declared = [a for a in protos[name].split(",") if a.strip() and a.strip() != "void"]
+        assert len(declared) == len(types), "ccall of %s: header declares %d parameters" % (name, len(declared))
+        seen += 1
+    assert seen >= 20
