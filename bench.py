@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the attention hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--only all|prefill|decode|copy]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--only all|prefill|decode|other|c1|c3|c4|ops|step|copy]
 
 A step is one pass of the hot path over one batch of synthetic input, inputs resident in HBM:
   prefill leg (the headline `value`): causal flash attention, Phi-3-mini shape
@@ -17,9 +17,12 @@ only); decode bytes = 2 * sum_b kv_len[b] * Hkv * D * 2 (K and V once per KV hea
 Kernel time is measured with HIP events on the launch stream around the timed steps; the CPU
 baseline is the oracle (a C restatement of the reference's flash_attn_cpu) on a bounded sample of
 the same workload, whose output also serves as a parity check of the GPU result.
+Inputs come from the package's seeded generator (SplitMix64 -> Box-Muller, luminal.jl_amd/synth.py) with the
+seeds the parity tests use for the same configurations; they are generated before any timed region.
 One JSON line on stdout; progress on stderr.
 """
 import argparse
+import hashlib
 import json
 import os
 import sys
@@ -33,12 +36,33 @@ sys.path.insert(0, ROOT)
 PEAK_FP32_TFLOPS = 157.3  # dense fp32 MFMA
 PEAK_FP16_TFLOPS = 2500.0  # MI355X dense fp16/bf16 MFMA
 PEAK_HBM_GBS = 8000.0      # MI355X HBM3E
-# HBM-side bytes per launch of the two headline workloads, from rocprofv3 --pmc FETCH_SIZE and
-# WRITE_SIZE runs of this script (--only prefill / --only decode), each scaled by what the same
-# counter reads for the calibration copy kernel (--only copy: factor 2.0 for FETCH_SIZE, 1.0 for
-# WRITE_SIZE). Counters cannot be read from inside a timed run, so the figures are recorded here.
-PREFILL_TRAFFIC_BYTES = 105.2e6 + 25.2e6           # vs 75.5 MB + 25.2 MB compulsory
-DECODE_TRAFFIC_BYTES = 5.2718e9 + 2.8e6 + 4.7e6    # split kernel read + partials + merge kernel
+# HBM-side bytes per launch (`roofline.traffic`) come from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this
+# script, each scaled by what the same counter reads for the calibration copy kernel (--only copy). Counters
+# cannot be read from inside a timed run, so the figures live in profiles/traffic.json next to the summaries they
+# were taken from, each with the hash of the kernel source it was measured on; a figure whose kernel source has
+# changed since is reported as null rather than as a stale number.
+TRAFFIC_FILE = os.path.join(ROOT, "profiles", "traffic.json")
+
+
+def source_hash(*names):
+    h = hashlib.sha256()
+    for n in names:
+        with open(os.path.join(ROOT, "luminal.jl_amd", "csrc", n), "rb") as f:
+            h.update(f.read())
+    return h.hexdigest()[:16]
+
+
+def measured_traffic(key):
+    """HBM bytes per launch recorded for `key`, or None when there is no record for the current kernel source."""
+    try:
+        with open(TRAFFIC_FILE) as f:
+            rec = json.load(f)[key]
+        if rec["source_sha16"] != source_hash(*rec["sources"]):
+            log("[bench] %s: %s changed since the counters were read; traffic reported as null" % (key, rec["sources"]))
+            return None
+        return float(rec["fetch_bytes"]) + float(rec["write_bytes"])
+    except (OSError, KeyError, ValueError):
+        return None
 
 
 def log(*a):
@@ -124,8 +148,7 @@ def rel_err(got, want):
 # -------------------------------------------------------------------------------------------------
 def prefill_leg(lm, dev, steps, warmup, cpu_seconds):
     B, H, S, D = 1, 32, 4096, 96
-    rng = np.random.default_rng(2)
-    host = [(rng.standard_normal((B, H, S, D), dtype=np.float32) * 0.5).astype(np.float16) for _ in range(3)]
+    host = [lm.synth.normal((B, H, S, D), 2000 + i, 0.5).astype(np.float16) for i in range(3)]  # seeds of the C2 parity test
     dq, dk, dv = (lm.HipArray((B, H, S, D), "f16", dev).copy_from_host(x) for x in host)
     out = lm.HipArray((B, H, S, D), "f16", dev)
     scale = lm.default_scale(D)
@@ -142,7 +165,7 @@ def prefill_leg(lm, dev, steps, warmup, cpu_seconds):
     res = {
         "ms_per_step": wall_ms, "value": tflops,
         "roofline": {"bound": "mfma", "achieved": kern_tflops, "peak": PEAK_FP16_TFLOPS, "unit": "TFLOP/s",
-                     "frac": kern_tflops / PEAK_FP16_TFLOPS, "traffic": PREFILL_TRAFFIC_BYTES,
+                     "frac": kern_tflops / PEAK_FP16_TFLOPS, "traffic": measured_traffic("prefill_C2"),
                      "kernel": "prefill_mfma_kernel<MfmaF16, 96, causal>", "launch_us": ev_ms * 1e3,
                      "algorithmic_flops_per_launch": flops, "launch_us_one_by_one": each,
                      # what a bare MFMA loop sustains on this GPU right now (clock management under load):
@@ -215,16 +238,16 @@ def fill_cache_from_pool(lm, cache, pool, lens, Hkv, Lmax, D, rng):
 
 def decode_leg(lm, dev, steps, warmup, cpu_seconds, num_splits=0):
     B, Hq, Hkv, Lmax, D = 64, 32, 8, 32768, 128
-    rng = np.random.default_rng(5)
-    lens = rng.integers(8192, 32768, size=B, endpoint=True).astype(np.int32)
+    rng = np.random.default_rng(5)  # only picks where in the pools each (sequence, head) slice is taken from
+    lens = lm.synth.uniform_int(B, 5000, 8192, 32768)  # the lengths of the C5 parity test
     pool_rows = 1 << 18  # 256 Ki rows of 128 bf16 = 64 MiB per pool
-    pools_host = [lm.f32_to_bf16_bits(rng.standard_normal((pool_rows, D), dtype=np.float32)) for _ in range(2)]
+    pools_host = [lm.f32_to_bf16_bits(lm.synth.normal((pool_rows, D), 6000 + i)) for i in range(2)]
     kpool, vpool = (lm.HipArray((pool_rows, D), "bf16", dev).copy_from_host(x) for x in pools_host)
     kc = lm.HipArray((B, Hkv, Lmax, D), "bf16", dev).fill_bytes(0xFF)  # tail past kv_len is NaN
     vc = lm.HipArray((B, Hkv, Lmax, D), "bf16", dev).fill_bytes(0xFF)
     kstart = fill_cache_from_pool(lm, kc, kpool, lens, Hkv, Lmax, D, rng)
     vstart = fill_cache_from_pool(lm, vc, vpool, lens, Hkv, Lmax, D, rng)
-    q_host = lm.f32_to_bf16_bits(rng.standard_normal((B, Hq, D), dtype=np.float32))
+    q_host = lm.f32_to_bf16_bits(lm.synth.normal((B, Hq, D), 5001))
     dq = lm.HipArray((B, Hq, D), "bf16", dev).copy_from_host(q_host)
     dl = lm.HipArray((B,), "i32", dev).copy_from_host(lens)
     out = lm.HipArray((B, Hq, D), "f32", dev)
@@ -242,7 +265,7 @@ def decode_leg(lm, dev, steps, warmup, cpu_seconds, num_splits=0):
         "workload": "C5 long ragged GQA decode: B=64 Hq=32 Hkv=8 D=128 bf16, kv_len~U[8192,32768], sum=%d" % int(lens.sum()),
         "value": gbs, "unit": "GB/s", "ms_per_step": wall_ms, "num_splits": int(p.num_splits),
         "roofline": {"bound": "hbm", "achieved": kern_gbs, "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": kern_gbs / PEAK_HBM_GBS,
-                     "traffic": DECODE_TRAFFIC_BYTES if num_splits == 0 else None,
+                     "traffic": measured_traffic("decode_C5") if num_splits == 0 else None,
                      "kernel": "decode_mfma_kernel<Mfma16BF16,128> + decode_merge_kernel",
                      "launch_us": ev_ms * 1e3, "algorithmic_bytes_per_launch": algo_bytes,
                      "launch_us_one_by_one": per_launch_us(fn, 20, lm.binding)},
@@ -277,48 +300,60 @@ def decode_leg(lm, dev, steps, warmup, cpu_seconds, num_splits=0):
     return res
 
 
-def other_configs(lm, dev, check=False):
-    """Short timings of the remaining contract configurations (20 launches each). With `check`, C1, C3 and C4 are
-    also compared with the CPU oracle on the whole output (the parity gate of the five configurations: C2 and C5
-    are checked in their own legs)."""
-    res = {}
-    rng = np.random.default_rng(9)
-    if check:
+def flash_config(lm, dev, res, name, B, Hq, Hkv, Sq, Sk, D, dtype, causal, flops, seed, mul=1.0, tol=None, steps=20,
+                 peak=None):
+    """One flash-attention configuration: 20 timed launches; with `tol`, the whole output against the CPU oracle."""
+    hq, hk, hv = (lm.synth.normal(shp, seed + i, mul) for i, shp in enumerate(((B, Hq, Sq, D), (B, Hkv, Sk, D), (B, Hkv, Sk, D))))
+    q, k, v = (lm.HipArray(x.shape, dtype, dev).copy_from_host(x) for x in (hq, hk, hv))
+    o = lm.HipArray((B, Hq, Sq, D), dtype, dev)
+    p = attn_params(lm, o, q, k, v, dtype, causal, lm.default_scale(D))
+    fn = lambda: lm.binding.flash_attn_fwd(p)
+    _, ev = time_steps(fn, steps, 5, lm.binding)
+    res[name] = {"launch_us": ev * 1e3, "TFLOP/s": flops / (ev * 1e-3) / 1e12,
+                 "launch_us_one_by_one": per_launch_us(fn, 20, lm.binding)}
+    if peak:
+        res[name]["frac_of_mfma_peak"] = res[name]["TFLOP/s"] / peak
+    log("[other] %s: %.1f us, %.2f TFLOP/s" % (name, ev * 1e3, res[name]["TFLOP/s"]))
+    if tol is not None:
         import oracle
-        nthreads = oracle.max_threads()
+        qh, kh, vh = (np.asarray(x.to_host(), np.float32) for x in (q, k, v))  # the element-type-rounded inputs
+        want = oracle.flash_attn(qh, kh, vh, scale=lm.default_scale(D), causal=causal, nthreads=oracle.max_threads())
+        err = float(np.max(np.abs(np.asarray(o.to_host(), np.float32) - want)) / np.max(np.abs(want)))
+        res[name]["parity"] = {"max_rel_err": err, "tolerance": tol, "checked": "whole output vs CPU oracle"}
+        log("[other] %s: GPU vs oracle rel err %.2e (tolerance %g)" % (name, err, tol))
 
-    def flash(name, B, Hq, Hkv, Sq, Sk, D, dtype, causal, flops, tol=None):
-        q = lm.HipArray((B, Hq, Sq, D), dtype, dev).copy_from_host(rng.standard_normal((B, Hq, Sq, D), dtype=np.float32))
-        k = lm.HipArray((B, Hkv, Sk, D), dtype, dev).copy_from_host(rng.standard_normal((B, Hkv, Sk, D), dtype=np.float32))
-        v = lm.HipArray((B, Hkv, Sk, D), dtype, dev).copy_from_host(rng.standard_normal((B, Hkv, Sk, D), dtype=np.float32))
-        o = lm.HipArray((B, Hq, Sq, D), dtype, dev)
-        p = attn_params(lm, o, q, k, v, dtype, causal, lm.default_scale(D))
-        _, ev = time_steps(lambda: lm.binding.flash_attn_fwd(p), 20, 5, lm.binding)
-        res[name] = {"launch_us": ev * 1e3, "TFLOP/s": flops / (ev * 1e-3) / 1e12}
-        log("[other] %s: %.1f us, %.2f TFLOP/s" % (name, ev * 1e3, res[name]["TFLOP/s"]))
-        if check and tol is not None:
-            qh, kh, vh = (np.asarray(x.to_host(), np.float32) for x in (q, k, v))  # the element-type-rounded inputs
-            want = oracle.flash_attn(qh, kh, vh, scale=lm.default_scale(D), causal=causal, nthreads=nthreads)
-            err = float(np.max(np.abs(np.asarray(o.to_host(), np.float32) - want)) / np.max(np.abs(want)))
-            res[name]["parity"] = {"max_rel_err": err, "tolerance": tol, "checked": "whole output vs CPU oracle"}
-            log("[other] %s: GPU vs oracle rel err %.2e (tolerance %g)" % (name, err, tol))
 
-    flash("C1 causal fp32 B=1 H=8 S=128 D=64", 1, 8, 8, 128, 128, 64, "f32", True, 4.0 * 8 * 64 * 128 * 129 / 2, tol=1e-5)
-    # the reference's element type on the C2 shape (an extra line, not one of the five configurations): fp32 matrix-core kernel
-    flash("C2 shape in fp32 (causal B=1 H=32 S=4096 D=96)", 1, 32, 32, 4096, 4096, 96, "f32", True, 4.0 * 32 * 96 * 4096 * 4097 / 2)
-    res["C2 shape in fp32 (causal B=1 H=32 S=4096 D=96)"]["frac_of_fp32_mfma_peak"] = \
-        res["C2 shape in fp32 (causal B=1 H=32 S=4096 D=96)"]["TFLOP/s"] / PEAK_FP32_TFLOPS
-    flash("C3 cross fp16 B=4 H=20 Sq=448 Sk=1500 D=64", 4, 20, 20, 448, 1500, 64, "f16", False, 4.0 * 4 * 20 * 448 * 1500 * 64, tol=2e-3)
+def c1_leg(lm, dev, res, check):
+    flash_config(lm, dev, res, "C1 causal fp32 B=1 H=8 S=128 D=64", 1, 8, 8, 128, 128, 64, "f32", True,
+                 4.0 * 8 * 64 * 128 * 129 / 2, 1000, tol=1e-5 if check else None)
+    # the reference's element type on the C2 shape (an extra line, not one of the five configurations)
+    name = "C2 shape in fp32 (causal B=1 H=32 S=4096 D=96)"
+    flash_config(lm, dev, res, name, 1, 32, 32, 4096, 4096, 96, "f32", True, 4.0 * 32 * 96 * 4096 * 4097 / 2, 2000, mul=0.5)
+    res[name]["frac_of_fp32_mfma_peak"] = res[name]["TFLOP/s"] / PEAK_FP32_TFLOPS
 
-    # C4: B=16 L=4096 decode; 268 MB would sit in the 256 MB last-level cache, so rotate over 4 caches
-    B, Hq, Hkv, L, D = 16, 32, 8, 4096, 128
-    pool = lm.f32_to_bf16_bits(rng.standard_normal((B * Hkv * L, D), dtype=np.float32))
+
+def c3_leg(lm, dev, res, check):
+    flash_config(lm, dev, res, "C3 cross fp16 B=4 H=20 Sq=448 Sk=1500 D=64", 4, 20, 20, 448, 1500, 64, "f16", False,
+                 4.0 * 4 * 20 * 448 * 1500 * 64, 3000, tol=2e-3 if check else None, steps=40, peak=PEAK_FP16_TFLOPS)
+
+
+def c4_caches(lm, dev):
+    """C4's caches, four times over: 268 MB would sit in the 256 MB last-level cache, so launches rotate over 4 copies
+    (each a different roll of the same seeded pool)."""
+    B, Hkv, L, D = 16, 8, 4096, 128
+    pool = lm.f32_to_bf16_bits(lm.synth.normal((B * Hkv * L, D), 4001))
     caches = []
     for i in range(4):
         kc = lm.HipArray((B, Hkv, L, D), "bf16", dev).copy_from_host(np.roll(pool, 977 * i, axis=0))
         vc = lm.HipArray((B, Hkv, L, D), "bf16", dev).copy_from_host(np.roll(pool, 977 * i + 401, axis=0))
         caches.append((kc, vc))
-    q = lm.HipArray((B, Hq, D), "bf16", dev).copy_from_host(rng.standard_normal((B, Hq, D), dtype=np.float32))
+    return caches
+
+
+def c4_leg(lm, dev, res, check, caches=None):
+    B, Hq, Hkv, L, D = 16, 32, 8, 4096, 128
+    caches = caches or c4_caches(lm, dev)
+    q = lm.HipArray((B, Hq, D), "bf16", dev).copy_from_host(lm.synth.normal((B, Hq, D), 4000))
     o = lm.HipArray((B, Hq, D), "f32", dev)
     ws = lm.HipArray((max(lm.binding.decode_workspace_bytes(B, Hq, Hkv, L, D, 0) // 4, 4),), "f32", dev)
     ps = [decode_params(lm, o, q, kc, vc, None, "bf16", lm.default_scale(D), ws) for kc, vc in caches]
@@ -330,21 +365,25 @@ def other_configs(lm, dev, check=False):
 
     _, ev = time_steps(step, 40, 8, lm.binding)
     nbytes = 2.0 * B * L * Hkv * D * 2 + B * Hq * D * 6
-    res["C4 decode bf16 B=16 Hq=32 Hkv=8 L=4096 D=128 (4 caches rotated)"] = {
-        "launch_us": ev * 1e3, "GB/s": nbytes / (ev * 1e-3) / 1e9, "frac_of_hbm_peak": nbytes / (ev * 1e-3) / 1e9 / PEAK_HBM_GBS}
-    log("[other] C4 decode: %.1f us, %.0f GB/s" % (ev * 1e3, nbytes / (ev * 1e-3) / 1e9))
+    name = "C4 decode bf16 B=16 Hq=32 Hkv=8 L=4096 D=128 (4 caches rotated)"
+    res[name] = {"launch_us": ev * 1e3, "GB/s": nbytes / (ev * 1e-3) / 1e9, "frac_of_hbm_peak": nbytes / (ev * 1e-3) / 1e9 / PEAK_HBM_GBS,
+                 "num_splits": int(ps[0].num_splits), "launch_us_one_by_one": per_launch_us(step, 20, lm.binding)}
+    log("[other] C4 decode: %.1f us, %.0f GB/s, %d splits" % (ev * 1e3, nbytes / (ev * 1e-3) / 1e9, ps[0].num_splits))
     if check:
+        import oracle
         lm.binding.decode_attn(ps[0])
         qh = np.asarray(q.to_host(), np.float32)
         kh, vh = (np.asarray(x.to_host(), np.float32) for x in caches[0])
-        want = oracle.decode_attn(qh, kh, vh, scale=lm.default_scale(D), nthreads=nthreads)
+        want = oracle.decode_attn(qh, kh, vh, scale=lm.default_scale(D), nthreads=oracle.max_threads())
         err = float(np.max(np.abs(np.asarray(o.to_host(), np.float32) - want)) / np.max(np.abs(want)))
-        res["C4 decode bf16 B=16 Hq=32 Hkv=8 L=4096 D=128 (4 caches rotated)"]["parity"] = {
-            "max_rel_err": err, "tolerance": 2e-3, "checked": "whole output vs CPU oracle"}
+        res[name]["parity"] = {"max_rel_err": err, "tolerance": 2e-3, "checked": "whole output vs CPU oracle"}
         log("[other] C4 decode: GPU vs oracle rel err %.2e (tolerance 2e-3)" % err)
+    return caches
 
-    # the two operators in front of attention: rotary embedding of a prompt's Q, and the cache append (K rotated on
-    # the way in) for a whole prompt and for one decode step. Algorithmic bytes = every element read once, written once.
+
+def ops_leg(lm, dev, res, caches=None):
+    """The two operators in front of attention: rotary embedding of a prompt's Q, and the cache append (K rotated on
+    the way in) for a whole prompt and for one decode step. Algorithmic bytes = every element read once, written once."""
     def hbm_line(name, fn, nbytes, n=20):
         _, ev = time_steps(fn, n, 5, lm.binding)
         res[name] = {"launch_us": ev * 1e3, "GB/s": nbytes / (ev * 1e-3) / 1e9, "frac_of_hbm_peak": nbytes / (ev * 1e-3) / 1e9 / PEAK_HBM_GBS}
@@ -352,7 +391,8 @@ def other_configs(lm, dev, check=False):
 
     B, H, S, D = 1, 32, 4096, 96
     # 12 inputs of 25 MB in rotation, more than the 256 MB last-level cache holds: every launch reads from HBM
-    xs = [lm.HipArray((B, H, S, D), "f16", dev).copy_from_host(rng.standard_normal((B, H, S, D), dtype=np.float32)) for _ in range(12)]
+    x0 = lm.synth.normal((B, H, S, D), 2000, 0.5)
+    xs = [lm.HipArray((B, H, S, D), "f16", dev).copy_from_host(np.roll(x0, 131 * i, axis=2)) for i in range(12)]
     y = lm.HipArray((B, H, S, D), "f16", dev)
     rps = []
     for x in xs:
@@ -370,20 +410,23 @@ def other_configs(lm, dev, check=False):
     hbm_line("rotary embedding fp16 B=1 H=32 S=4096 D=96 (C2's Q, 12 inputs rotated)", rope_step, 2.0 * B * H * S * D * 2, n=36)
     del xs
 
+    caches = caches or c4_caches(lm, dev)
     for T, label in ((4096, "whole prompt T=4096"), (1, "one decode step T=1")):
         B, Hkv, L, D = 16, 8, 4096, 128
         kc, vc = caches[0]
-        kn = lm.HipArray((B, Hkv, T, D), "bf16", dev).copy_from_host(rng.standard_normal((B, Hkv, T, D), dtype=np.float32))
-        vn = lm.HipArray((B, Hkv, T, D), "bf16", dev).copy_from_host(rng.standard_normal((B, Hkv, T, D), dtype=np.float32))
+        kn = lm.HipArray((B, Hkv, T, D), "bf16", dev).copy_from_host(lm.synth.normal((B, Hkv, T, D), 4100))
+        vn = lm.HipArray((B, Hkv, T, D), "bf16", dev).copy_from_host(lm.synth.normal((B, Hkv, T, D), 4101))
         ap = lm.binding.KvAppendParams()
         ap.k_cache, ap.v_cache, ap.k_new, ap.v_new, ap.pos, ap.pos_all = kc.ptr, vc.ptr, kn.ptr, vn.ptr, None, (0 if T > 1 else L - 1)
         ap.B, ap.Hkv, ap.T, ap.D, ap.Lmax = B, Hkv, T, D, L
         ap.dtype, ap.rope_k, ap.pairing, ap.base, ap.stream = lm.binding.DTYPE_CODES["bf16"], 1, lm.binding.ROPE_HALF_SPLIT, 10000.0, None
         hbm_line("cache append + rotary K bf16 B=16 Hkv=8 D=128, %s" % label, lambda: lm.binding.kv_append(ap), 4.0 * B * Hkv * T * D * 2)
 
-    # one whole decode step of an attention layer (append with rotary q and K, split-KV attention, merge: 3
-    # kernels), driven from the host step by step and as one recorded HIP graph; wall clock per step. On the C4
-    # shape the GPU is the bottleneck either way; a single short sequence is bound by the host's launches.
+
+def step_leg(lm, dev, res):
+    """One whole decode step of an attention layer (append with rotary q and K, split-KV attention, merge: 3
+    kernels), driven from the host step by step and as one recorded HIP graph; wall clock per step. On the C4
+    shape the GPU is the bottleneck either way; a single short sequence is bound by the host's launches."""
     for B, L in ((16, 4096), (1, 512)):
         Hq, Hkv, D = 32, 8, 128
         g = lm.Graph()
@@ -412,6 +455,24 @@ def other_configs(lm, dev, check=False):
         res["decode step of a layer bf16 B=%d Hq=32 Hkv=8 L=%d D=128 (append with rotary q and K + attention), wall clock" % (B, L)] = {
             "us_per_step_3_launches_from_the_host": eager, "us_per_step_one_hip_graph": replay}
         log("[other] decode step B=%d L=%d, wall clock: %.1f us as 3 host launches, %.1f us as one HIP graph" % (B, L, eager, replay))
+
+
+def other_configs(lm, dev, check=False, only="other"):
+    """Short timings of the remaining contract configurations. With `check`, C1, C3 and C4 are also compared with the
+    CPU oracle on the whole output (the parity gate of the five configurations: C2 and C5 are checked in their own
+    legs). `only` = "other" runs everything, or one of c1 / c3 / c4 / ops / step (a profile of one kernel)."""
+    res = {}
+    caches = None
+    if only in ("other", "c1"):
+        c1_leg(lm, dev, res, check)
+    if only in ("other", "c3"):
+        c3_leg(lm, dev, res, check)
+    if only in ("other", "c4"):
+        caches = c4_leg(lm, dev, res, check)
+    if only in ("other", "ops"):
+        ops_leg(lm, dev, res, caches)
+    if only in ("other", "step"):
+        step_leg(lm, dev, res)
     return res
 
 
@@ -430,7 +491,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--only", choices=["all", "prefill", "decode", "other", "copy"], default="all")
+    ap.add_argument("--only", choices=["all", "prefill", "decode", "other", "c1", "c3", "c4", "ops", "step", "copy"], default="all")
     ap.add_argument("--decode-splits", type=int, default=0, help="KV splits for the decode leg (0 = library heuristic)")
     ap.add_argument("--cpu-seconds", type=float, default=15.0, help="CPU-baseline budget per leg; 0 disables it")
     args = ap.parse_args()
@@ -466,8 +527,8 @@ def main():
             line["cpu_baseline_single_thread"] = r["cpu_baseline_single_thread"]
     if args.only in ("all", "decode"):
         line["decode"] = decode_leg(lm, dev, args.steps, args.warmup, args.cpu_seconds, args.decode_splits)
-    if args.only in ("all", "other"):
-        line["other_configs"] = other_configs(lm, dev, check=args.cpu_seconds > 0)
+    if args.only in ("all", "other", "c1", "c3", "c4", "ops", "step"):
+        line["other_configs"] = other_configs(lm, dev, check=args.cpu_seconds > 0, only="other" if args.only == "all" else args.only)
     gate = [("C2", line.get("parity"))] + [("C5", line.get("decode", {}).get("parity"))] + \
         [(k.split()[0], v.get("parity")) for k, v in line.get("other_configs", {}).items() if isinstance(v, dict) and "parity" in v]
     gate = [(n, p) for n, p in gate if p]

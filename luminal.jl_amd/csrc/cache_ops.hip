@@ -21,13 +21,31 @@
 namespace lmh {
 namespace {
 
+// sin and cos of an fp32 angle (radians, any magnitude an fp32 position reaches) on the hardware's
+// v_sin_f32 / v_cos_f32, which take revolutions. The library sincosf costs ~100 instructions per angle (its
+// large-argument path alone is a table walk) and made the rotary kernels compute-bound at 46 % of the
+// memory roofline. Here the angle is reduced by whole turns with 2 pi split into its fp32 head and the
+// remainder (two fused multiply-adds: the first is exact up to the rounding of a result no larger than
+// ~pi, whatever the number of turns), so |r| <= pi to ~3e-7 rad, and r / 2 pi goes to the hardware.
+__device__ inline void sincos_angle(float angle, float *sn, float *cs) {
+  constexpr float kInv2Pi = 0.15915493667125702f;
+  constexpr float k2PiHead = 6.2831854820251465f;      // fp32(2 pi)
+  constexpr float k2PiTail = -1.7484555314695172e-07f;  // 2 pi - fp32(2 pi)
+  const float turns = rintf(angle * kInv2Pi);
+  float r = fmaf(-turns, k2PiHead, angle);
+  r = fmaf(-turns, k2PiTail, r);
+  const float x = r * kInv2Pi;
+  *sn = __builtin_amdgcn_sinf(x);
+  *cs = __builtin_amdgcn_cosf(x);
+}
+
 template <typename E>
 __device__ inline void rope_pair(float x0, float x1, float pos, int j, int D, float log2_base, float *o0, float *o1) {
   // inv_freq = 1 / exp2((2j/D) * log2(base)), evaluated as the reference does (src/NN.jl:262-263)
   const float freq = (float)j * 2.0f / (float)D;
   const float inv_freq = 1.0f / exp2f(freq * log2_base);
   float sn, cs;
-  sincosf(pos * inv_freq, &sn, &cs);
+  sincos_angle(pos * inv_freq, &sn, &cs);
   *o0 = x0 * cs - x1 * sn;
   *o1 = x0 * sn + x1 * cs;
 }
@@ -135,7 +153,7 @@ __device__ inline void sincos_pairs(float pos, int j0, int n, int D, float log2_
     if (i >= n) break;
     const float freq = (float)(j0 + i) * 2.0f / (float)D;
     const float inv_freq = 1.0f / exp2f(freq * log2_base);
-    sincosf(pos * inv_freq, &sn[i], &cs[i]);
+    sincos_angle(pos * inv_freq, &sn[i], &cs[i]);
   }
 }
 
@@ -157,22 +175,33 @@ __global__ __launch_bounds__(256) void rope_vec_kernel(RopeArgs a, int heads_per
   const float pos = (float)((a.pos0 ? a.pos0[b] : a.prev_seq) + s);
   float sn[V], cs[V];
   sincos_pairs<E>(pos, IL ? c * (V / 2) : c * V, IL ? V / 2 : V, a.D, a.log2_base, sn, cs);
+  // Heads in batches of kHeadBatch: all of a batch's loads are issued before the first is used, so a thread has up
+  // to 2 * kHeadBatch 16-byte loads in flight (the ~1000 workgroups of a launch alone do not keep HBM busy).
+  constexpr int kHeadBatch = 4;
   const int h0 = blockIdx.y * heads_per_block, h1 = min(a.H, h0 + heads_per_block);
-  for (int h = h0; h < h1; h++) {
-    const raw *xp = reinterpret_cast<const raw *>(a.x) + b * a.xs[0] + h * a.xs[1] + (int64_t)s * a.xs[2];
-    raw *op = reinterpret_cast<raw *>(a.out) + b * a.os[0] + h * a.os[1] + (int64_t)s * a.os[2];
-    if (IL) {
-      Chunk<E> ch;
-      ch.u = *reinterpret_cast<const uint4 *>(xp + c * V);
-      rotate_interleaved<E>(ch, sn, cs);
-      *reinterpret_cast<uint4 *>(op + c * V) = ch.u;
-    } else {
-      Chunk<E> c0, c1;
-      c0.u = *reinterpret_cast<const uint4 *>(xp + c * V);
-      c1.u = *reinterpret_cast<const uint4 *>(xp + half + c * V);
-      rotate_chunks<E>(c0, c1, sn, cs);
-      *reinterpret_cast<uint4 *>(op + c * V) = c0.u;
-      *reinterpret_cast<uint4 *>(op + half + c * V) = c1.u;
+  const raw *xrow = reinterpret_cast<const raw *>(a.x) + b * a.xs[0] + (int64_t)s * a.xs[2];
+  raw *orow = reinterpret_cast<raw *>(a.out) + b * a.os[0] + (int64_t)s * a.os[2];
+  for (int hb = h0; hb < h1; hb += kHeadBatch) {
+    Chunk<E> c0[kHeadBatch], c1[kHeadBatch];
+#pragma unroll
+    for (int i = 0; i < kHeadBatch; i++) {
+      if (hb + i >= h1) break;
+      const raw *xp = xrow + (hb + i) * a.xs[1];
+      c0[i].u = *reinterpret_cast<const uint4 *>(xp + c * V);
+      if (!IL) c1[i].u = *reinterpret_cast<const uint4 *>(xp + half + c * V);
+    }
+#pragma unroll
+    for (int i = 0; i < kHeadBatch; i++) {
+      if (hb + i >= h1) break;
+      raw *op = orow + (hb + i) * a.os[1];
+      if (IL) {
+        rotate_interleaved<E>(c0[i], sn, cs);
+        *reinterpret_cast<uint4 *>(op + c * V) = c0[i].u;
+      } else {
+        rotate_chunks<E>(c0[i], c1[i], sn, cs);
+        *reinterpret_cast<uint4 *>(op + c * V) = c0[i].u;
+        *reinterpret_cast<uint4 *>(op + half + c * V) = c1[i].u;
+      }
     }
   }
 }
@@ -245,7 +274,10 @@ void launch_rope_vec(const RopeArgs &a, hipStream_t stream) {
   const int64_t blocks_x = ((int64_t)a.B * a.S * cpr + 255) / 256;
   // about 1024 workgroups fill the chip; beyond that, more heads per thread amortise the sin / cos
   // (C2's Q, 25 MB: 16.9 us with one head per thread, 11.0 us at 3; large tensors lose ~5 % to the longer threads)
-  int blocks_y = (int)((1024 + blocks_x - 1) / blocks_x);
+#ifndef LMH_ROPE_WGS
+#define LMH_ROPE_WGS 1024
+#endif
+  int blocks_y = (int)((LMH_ROPE_WGS + blocks_x - 1) / blocks_x);
   blocks_y = blocks_y < 1 ? 1 : (blocks_y > a.H ? a.H : blocks_y);
   const int heads_per_block = (a.H + blocks_y - 1) / blocks_y;
   blocks_y = (a.H + heads_per_block - 1) / heads_per_block;

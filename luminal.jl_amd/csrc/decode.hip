@@ -134,10 +134,23 @@ __global__ __launch_bounds__(kWaves * 64) void decode_split_kernel(DecodeArgs a,
   int L = a.kv_len ? a.kv_len[b] : a.Lmax;
   L = min(max(L, 0), a.Lmax);
   const int start = split * a.chunk;
-  if (start >= L) return;  // ragged tail: this split does not exist for sequence b
+  const int tid = threadIdx.x;
+  if (start >= L) {  // ragged tail: this split does not exist for sequence b
+    // ... and with a single split nobody else writes the rows of a sequence without keys: zeros, like every
+    // other kernel of the library
+    if (a.num_splits == 1) {
+      for (int idx = tid; idx < G * a.D; idx += kWaves * 64) {
+        const int gi = g0 + idx / a.D;
+        if (gi >= group) continue;
+        const int64_t off = b * a.os[0] + q_head_of(kvh, gi, a.Hq, a.Hkv, a.head_map) * a.os[1] + idx % a.D;
+        if (a.out_f32) reinterpret_cast<float *>(a.out)[off] = 0.f;
+        else reinterpret_cast<raw *>(a.out)[off] = E::st(0.f);
+      }
+    }
+    return;
+  }
   const int end = min(L, start + a.chunk);
 
-  const int tid = threadIdx.x;
   const int lane = tid & 63, wave = tid >> 6;
   const int slot = lane / LPK;
   const int c = lane % LPK;
@@ -285,6 +298,7 @@ __global__ __launch_bounds__(kWaves * 64) void decode_split_kernel(DecodeArgs a,
 // issues independent loads of the partial outputs instead of a chain of dependent ones.
 constexpr int kMergeThreads = 128;
 constexpr int kMergeMaxSlots = 1024;  // weights kept in LDS; more slots than this take the strided path below
+constexpr int kMergePrefetch = 16;     // partial rows fetched before the slot statistics are known
 template <typename E>
 __global__ __launch_bounds__(kMergeThreads) void decode_merge_kernel(DecodeArgs a) {
   using raw = typename E::raw;
@@ -292,12 +306,23 @@ __global__ __launch_bounds__(kMergeThreads) void decode_merge_kernel(DecodeArgs 
   __shared__ float red_m[kMergeThreads / 64], red_l[kMergeThreads / 64];
   const int hq = blockIdx.x, b = blockIdx.y;
   const int tid = threadIdx.x;
-  int L = a.kv_len ? a.kv_len[b] : a.Lmax;
-  L = min(max(L, 0), a.Lmax);
-  const int n = (L + a.chunk - 1) / a.chunk;
   const int64_t off = b * a.os[0] + hq * a.os[1];
   const int64_t row0 = ((int64_t)b * a.Hq + hq) * a.num_splits;
   const float2 *ml = reinterpret_cast<const float2 *>(a.ws_ml) + row0;
+  const float *po = a.ws_o + row0 * a.D;
+
+  // The kernel is a chain of round trips to memory the split kernel has just written (kv_len, the slot statistics,
+  // the partial rows), each about as long as the arithmetic of the whole kernel. The rows of the first slots do
+  // not depend on the others: they are requested first, and travel while the statistics are reduced. Rows of
+  // slots that turn out not to exist or to be empty are unset memory and are discarded unread below.
+  float pre[kMergePrefetch];
+  const int n_pre = min(a.num_splits, kMergePrefetch);
+#pragma unroll
+  for (int u = 0; u < kMergePrefetch; u++) pre[u] = (u < n_pre && tid < a.D) ? po[(int64_t)u * a.D + tid] : 0.f;
+
+  int L = a.kv_len ? a.kv_len[b] : a.Lmax;
+  L = min(max(L, 0), a.Lmax);
+  const int n = (L + a.chunk - 1) / a.chunk;
 
   // running max over the slots
   float M = -INFINITY;
@@ -328,16 +353,26 @@ __global__ __launch_bounds__(kMergeThreads) void decode_merge_kernel(DecodeArgs 
   for (int w = 0; w < kMergeThreads / 64; w++) lsum += red_l[w];
   const float inv = lsum > 0.f ? 1.f / lsum : 0.f;
 
-  const float *po = a.ws_o + row0 * a.D;
   for (int d = tid; d < a.D; d += kMergeThreads) {
     float acc[4] = {0.f, 0.f, 0.f, 0.f};
     int s = 0;
     const int n_lds = min(n, kMergeMaxSlots);
+    if (d == tid) {  // the prefetched rows (same summation order as below: slot s adds to acc[s % 4])
+      const int n_p = min(n_lds, n_pre) & ~3;
+#pragma unroll
+      for (int u = 0; u < kMergePrefetch; u++) {
+        if (u < n_p) {
+          const float w = w_s[u];
+          // the row of a zero-weight slot is unset memory: select, do not multiply
+          acc[u & 3] += w != 0.f ? pre[u] * w : 0.f;
+        }
+      }
+      s = n_p;
+    }
     for (; s + 4 <= n_lds; s += 4) {
 #pragma unroll
       for (int u = 0; u < 4; u++) {
         const float w = w_s[s + u];
-        // the row of a zero-weight slot is unset memory: select, do not multiply
         const float x = po[(int64_t)(s + u) * a.D + d];
         acc[u] += w != 0.f ? x * w : 0.f;
       }

@@ -91,19 +91,26 @@ __global__ __launch_bounds__(kWaves * 64) void decode_mfma_kernel(DecodeArgs a, 
   const int kv_slots = a.Hkv * g_chunks;  // (kv head, slice of <= 16 group members) pairs
 
   // ---- this workgroup's share of the (b, kv slot, chunk) units ----
-  for (int i = tid; i < a.B; i += kWaves * 64) {
-    int L = a.kv_len ? a.kv_len[i] : a.Lmax;
-    L = min(max(L, 0), a.Lmax);
-    s_pref[i + 1] = (L + a.chunk - 1) / a.chunk;
-  }
-  __syncthreads();
-  if (tid == 0) {
-    int run = 0;
-    s_pref[0] = 0;
-    for (int i = 1; i <= a.B; i++) {
-      run += s_pref[i];
-      s_pref[i] = run;
+  // s_pref = exclusive prefix sum of the chunks per sequence. Without kv_len it is a closed form; with it, the
+  // first wave scans 64 sequences at a time with lane shifts (a serial loop over B = 64 by one thread was 3 us).
+  if (!a.kv_len) {
+    const int per_seq = (a.Lmax + a.chunk - 1) / a.chunk;
+    for (int i = tid; i <= a.B; i += kWaves * 64) s_pref[i] = i * per_seq;
+  } else if (wave == 0) {
+    int carry = 0;
+    for (int base = 0; base < a.B; base += 64) {
+      const int i = base + lane;
+      int v = 0;
+      if (i < a.B) v = (min(max(a.kv_len[i], 0), a.Lmax) + a.chunk - 1) / a.chunk;
+#pragma unroll
+      for (int off = 1; off < 64; off <<= 1) {
+        const int up = __shfl_up(v, off);
+        if (lane >= off) v += up;
+      }
+      if (i < a.B) s_pref[i + 1] = carry + v;
+      carry += __shfl(v, 63);
     }
+    if (lane == 0) s_pref[0] = 0;
   }
   __syncthreads();
   const int64_t total_units = (int64_t)s_pref[a.B] * kv_slots;
@@ -312,6 +319,19 @@ __global__ __launch_bounds__(kWaves * 64) void decode_mfma_kernel(DecodeArgs a, 
   }
   __syncthreads();  // the merge buffers are tile memory again in the next segment
   }  // while (u < u_end)
+
+  // A sequence without keys has no unit. With several splits the merge kernel writes its zeros; with one split
+  // nothing else would write its output rows.
+  if (a.num_splits == 1) {
+    for (int b = blockIdx.x; b < a.B; b += gridDim.x) {
+      if (s_pref[b + 1] != s_pref[b]) continue;
+      for (int idx = tid; idx < a.Hq * D; idx += kWaves * 64) {
+        const int64_t off = b * a.os[0] + (idx / D) * a.os[1] + idx % D;
+        if (a.out_f32) reinterpret_cast<float *>(a.out)[off] = 0.f;
+        else reinterpret_cast<uint16_t *>(a.out)[off] = 0;
+      }
+    }
+  }
 }
 
 template <typename MT, int D>

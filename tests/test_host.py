@@ -121,3 +121,18 @@ def test_execute_with_capture_without_a_hip_device_just_runs(lm):
     assert calls == [None] and cache == {}
     lm.release_capture(cache)  # nothing recorded: a no-op
     assert cache == {}
+
+
+def test_package_input_generator_is_the_oracles_generator(lm, oracle):
+    # bench.py draws its inputs from the package's own generator; the tests draw theirs from the oracle's C one.
+    # Same specification, so the same seeds give the same configurations (libm and numpy may differ in the last
+    # bit of a float64 log / cos / sin, which survives the rounding to float32 only rarely).
+    for shape, seed, mul in [((3, 5, 7), 2000, 0.5), ((1001,), 3000, 1.0), ((2, 64), 4002, 1.0)]:
+        a, b = lm.synth.normal(shape, seed, mul), oracle.gen_normal(shape, seed, mul)
+        assert a.shape == b.shape and a.dtype == b.dtype
+        ulp = np.abs(a.view(np.int32).astype(np.int64) - b.view(np.int32).astype(np.int64))
+        assert ulp.max() <= 1 and (ulp != 0).mean() < 1e-3
+    np.testing.assert_array_equal(lm.synth.uniform_int(64, 5000, 8192, 32768), oracle.gen_uniform_int(64, 5000, 8192, 32768))
+    big = lm.synth.normal((1 << 16,), 7, chunk_pairs=1000)  # chunking does not change the stream
+    np.testing.assert_array_equal(big, lm.synth.normal((1 << 16,), 7))
+    assert abs(float(big.mean())) < 0.02 and abs(float(big.std()) - 1.0) < 0.02

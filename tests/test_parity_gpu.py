@@ -437,6 +437,24 @@ def test_decode_without_kv_len_and_poisoned_tail(lm, hip, oracle):
         assert rel_err(got, oracle.decode_attn(q, k, v, kv_len=lens)) <= 2e-3
 
 
+@pytest.mark.parametrize("dtype,D,out_dtype", [("bf16", 128, "f32"), ("f16", 64, "f16"), ("f32", 64, "f32"), ("bf16", 72, "bf16")])
+@pytest.mark.parametrize("splits", [1, 0, 3])
+def test_decode_sequence_without_keys_is_written_as_zeros(lm, hip, oracle, dtype, D, out_dtype, splits):
+    # kv_len[b] == 0 (a fresh cache) does not occur in the reference; like every prefill kernel, every decode path
+    # (matrix-core and vector kernel, with and without a merge pass) writes zeros for it instead of leaving the rows unset
+    B, Hq, Hkv, L = 4, 8, 2, 600
+    q, k, v = inputs(oracle, (B, Hq, D), (B, Hkv, L, D), dtype, 7950 + D)
+    lens = np.array([600, 0, 37, 0], np.int32)
+    dq, dk, dv = (lm.to_device(x, hip, dtype) for x in (q, k, v))
+    out = lm.HipArray((B, Hq, D), out_dtype, hip).fill_bytes(0xFF)  # NaN bit patterns: unwritten rows would show
+    op = lm.DecodeAttentionOp(lm.default_scale(D), 0, splits)
+    lm.host.execute_op_inplace(out, op, dq, dk, dv, lm.to_device(lens, hip))
+    got = out.to_host()
+    assert np.all(got[[1, 3]] == 0)
+    want = oracle.decode_attn(q, k, v, kv_len=np.maximum(lens, 1))
+    assert rel_err(got[[0, 2]], want[[0, 2]]) <= (8e-3 if out_dtype == "bf16" else TOL[dtype])
+
+
 @pytest.mark.parametrize("dtype", ["f16", "bf16"])
 def test_half_output_is_the_rounded_fp32_output(lm, hip, oracle, dtype):
     """out_f32 = 0 writes the same result rounded once to the input element type. The two code paths
