@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the attention hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--only all|prefill|decode|other|c1|c3|c4|ops|step|copy]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--only all|prefill|decode|other|c1|c3|c4|ops|step|copy|ceiling]
 
 A step is one pass of the hot path over one batch of synthetic input, inputs resident in HBM:
   prefill leg (the headline `value`): causal flash attention, Phi-3-mini shape
@@ -408,6 +408,12 @@ def ops_leg(lm, dev, res, caches=None):
         rstate["i"] += 1
 
     hbm_line("rotary embedding fp16 B=1 H=32 S=4096 D=96 (C2's Q, 12 inputs rotated)", rope_step, 2.0 * B * H * S * D * 2, n=36)
+
+    def copy_step():  # the same bytes through the plain copy kernel: what this size allows (ramp-up is a third of it)
+        lm.binding.calib_copy(y.ptr, xs[rstate["i"] % len(xs)].ptr, B * H * S * D * 2)
+        rstate["i"] += 1
+
+    hbm_line("plain copy of the same 25 MB (reference for the line above)", copy_step, 2.0 * B * H * S * D * 2, n=36)
     del xs
 
     caches = caches or c4_caches(lm, dev)
@@ -457,6 +463,43 @@ def step_leg(lm, dev, res):
         log("[other] decode step B=%d L=%d, wall clock: %.1f us as 3 host launches, %.1f us as one HIP graph" % (B, L, eager, replay))
 
 
+def ceiling_leg(lm, dev):
+    """What the matrix cores sustain, and how it depends on how much of the chip is busy: the bare MFMA loop on the
+    workload's own operand values with 1, 2, 4 and 8 XCDs running it (the others idle), and the attention kernel on
+    a steady-state shape (B=4, non-causal: 4096 equal workgroups). Rates are scaled to the whole chip (x 8 / active)
+    so that they compare; clocks are settled before each timing."""
+    res = {"bare_mfma_loop": {}}
+    B, H, S, D = 4, 32, 4096, 96
+    host = [lm.synth.normal((B, H, S, D), 2100 + i, 0.5).astype(np.float16) for i in range(3)]
+    dq, dk, dv = (lm.HipArray((B, H, S, D), "f16", dev).copy_from_host(x) for x in host)
+    sink = lm.HipArray((512 * 256,), "f32", dev)
+    for active in (1, 2, 4, 8):
+        per_wg = [0.0]
+
+        def fn():
+            per_wg[0] = lm.binding.calib_mfma_xcds(sink.ptr, dq.ptr, 1 << 17, 40000, active)
+        _, ev = time_steps(fn, 3, 1, lm.binding)
+        ran = int((sink.to_host().reshape(512, 256)[:, 0] != -1.0).sum())
+        tf = per_wg[0] * ran / (ev * 1e-3) / 1e12
+        res["bare_mfma_loop"]["%d_xcds" % active] = {
+            "workgroups_that_ran": ran, "TFLOP/s": tf, "TFLOP/s_scaled_to_8_xcds": tf * 8 / active,
+            "frac_of_peak_scaled": tf * 8 / active / PEAK_FP16_TFLOPS}
+        log("[ceiling] bare MFMA loop on %d XCD(s): %d of 512 workgroups ran, %.0f TFLOP/s = %.0f scaled to the chip (%.1f%% of peak)"
+            % (active, ran, tf, tf * 8 / active, 100 * tf * 8 / active / PEAK_FP16_TFLOPS))
+    out = lm.HipArray((B, H, S, D), "f16", dev)
+    p = attn_params(lm, out, dq, dk, dv, "f16", False, lm.default_scale(D))
+    _, ev = time_steps(lambda: lm.binding.flash_attn_fwd(p), 10, 3, lm.binding)
+    active = int(os.environ.get("LMH_BENCH_ACTIVE_XCDS", "8"))  # 8 unless the library was built with -DLMH_ONLY_XCDS=n
+    flops = 4.0 * B * H * D * S * S * active / 8
+    res["attention_steady_state"] = {"shape": "B=4 H=32 S=4096 D=96 fp16 non-causal", "active_xcds": active, "launch_us": ev * 1e3,
+                                     "TFLOP/s_scaled_to_8_xcds": flops / (ev * 1e-3) / 1e12 * 8 / active,
+                                     "frac_of_peak_scaled": flops / (ev * 1e-3) / 1e12 * 8 / active / PEAK_FP16_TFLOPS}
+    log("[ceiling] attention, steady-state shape, %d XCD(s) working: %.1f us, %.0f TFLOP/s scaled to the chip (%.1f%% of peak)"
+        % (active, ev * 1e3, res["attention_steady_state"]["TFLOP/s_scaled_to_8_xcds"],
+           100 * res["attention_steady_state"]["frac_of_peak_scaled"]))
+    return res
+
+
 def other_configs(lm, dev, check=False, only="other"):
     """Short timings of the remaining contract configurations. With `check`, C1, C3 and C4 are also compared with the
     CPU oracle on the whole output (the parity gate of the five configurations: C2 and C5 are checked in their own
@@ -491,7 +534,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--only", choices=["all", "prefill", "decode", "other", "c1", "c3", "c4", "ops", "step", "copy"], default="all")
+    ap.add_argument("--only", choices=["all", "prefill", "decode", "other", "c1", "c3", "c4", "ops", "step", "copy", "ceiling"], default="all")
     ap.add_argument("--decode-splits", type=int, default=0, help="KV splits for the decode leg (0 = library heuristic)")
     ap.add_argument("--cpu-seconds", type=float, default=15.0, help="CPU-baseline budget per leg; 0 disables it")
     args = ap.parse_args()
@@ -516,6 +559,10 @@ def main():
     }
     if args.only == "copy":
         line["calibration_copy"] = copy_leg(lm, dev, args.steps, args.warmup)
+        print(json.dumps(line))
+        return
+    if args.only == "ceiling":
+        line["ceiling"] = ceiling_leg(lm, dev)
         print(json.dumps(line))
         return
     if args.only in ("all", "prefill"):

@@ -107,6 +107,12 @@ int lmh_calib_copy(void *dst_dev, const void *src_dev, size_t bytes, void *strea
  * values (clock management under load), so time it on data like the attention inputs. `sink_dev`
  * receives 512*256 floats; `*flops` (host, optional) the flops of one launch. */
 int lmh_calib_mfma(void *sink_dev, const void *operands_dev, size_t operand_bytes, int iters, double *flops, void *stream);
+/* The same loop on part of the chip: workgroups that land on XCD number `active_xcds` (1..8) or above exit at once
+ * and set their first sink slot (sink[256 * workgroup]) to -1, the others run the loop, so the host can count
+ * them. `*flops_per_workgroup` (host, optional) is what one running workgroup computes. Shows how the rate a CU
+ * sustains depends on how much of the chip is busy (clock and power management). */
+int lmh_calib_mfma_xcds(void *sink_dev, const void *operands_dev, size_t operand_bytes, int iters, int active_xcds,
+                        double *flops_per_workgroup, void *stream);
 
 /* ---- flash attention forward: replaces
  *   execute_op!(out, op::FlashAttentionOp, q, k, v)   reference src/Execution.jl:565-578
@@ -116,7 +122,10 @@ int lmh_calib_mfma(void *sink_dev, const void *operands_dev, size_t operand_byte
  *
  * out[b,hq,i,:] = sum_j softmax_j(scale * q[b,hq,i,:] . k[b,kvh,j,:]) v[b,kvh,j,:]
  * with j restricted to j <= i when causal != 0 (the reference skips j > i,
- * src/Execution.jl:462), and to j < kv_len[b] when kv_len is non-null. ---- */
+ * src/Execution.jl:462), and to j < kv_len[b] when kv_len is non-null.
+ * Head dims up to 256, like decode. The matrix-core kernels take multiples of 8 up to 128 (with 16-byte
+ * aligned pointers and strides, scale > 0); everything else runs on a vector-ALU kernel with the same
+ * results at a fraction of the speed. ---- */
 typedef struct lmh_attn_params {
   void *out;          /* [B,Hq,Sq,D] device */
   const void *q;      /* [B,Hq,Sq,D] device */

@@ -23,7 +23,8 @@ EXPORTS = [
     "lmh_version", "lmh_last_error", "lmh_device_count", "lmh_init", "lmh_device_name", "lmh_malloc", "lmh_free",
     "lmh_memset", "lmh_memcpy_h2d", "lmh_memcpy_d2h", "lmh_memcpy_d2d", "lmh_sync", "lmh_event_create",
     "lmh_event_destroy", "lmh_event_record", "lmh_event_elapsed_ms", "lmh_flash_attn_fwd",
-    "lmh_decode_workspace_bytes", "lmh_decode_auto_splits", "lmh_decode_attn", "lmh_calib_copy", "lmh_calib_mfma", "lmh_rope",
+    "lmh_decode_workspace_bytes", "lmh_decode_auto_splits", "lmh_decode_attn", "lmh_calib_copy", "lmh_calib_mfma",
+    "lmh_calib_mfma_xcds", "lmh_rope",
     "lmh_kv_append", "lmh_stream_create", "lmh_stream_destroy", "lmh_graph_capture_begin", "lmh_graph_capture_end",
     "lmh_graph_launch", "lmh_graph_destroy", "lmh_static_scratch_bytes", "lmh_decode_static_splits",
     "lmh_decode_attn_static",
@@ -130,6 +131,8 @@ def load():
     L.lmh_decode_static_splits.argtypes = [ctypes.c_int32] * 5
     L.lmh_calib_copy.argtypes = [vp, vp, ctypes.c_size_t, vp]
     L.lmh_calib_mfma.argtypes = [vp, vp, ctypes.c_size_t, ctypes.c_int, ctypes.POINTER(ctypes.c_double), vp]
+    L.lmh_calib_mfma_xcds.argtypes = [vp, vp, ctypes.c_size_t, ctypes.c_int, ctypes.c_int, ctypes.POINTER(ctypes.c_double), vp]
+    L.lmh_calib_mfma_xcds.restype = ctypes.c_int
     L.lmh_rope.argtypes = [ctypes.POINTER(RopeParams)]
     L.lmh_kv_append.argtypes = [ctypes.POINTER(KvAppendParams)]
     L.lmh_stream_create.argtypes = [ctypes.POINTER(vp)]
@@ -282,6 +285,13 @@ def calib_mfma(sink, operands, operand_bytes, iters, stream=None):
     """Launch the bare MFMA loop; returns the flops of the launch."""
     flops = ctypes.c_double(0.0)
     check(load().lmh_calib_mfma(sink, operands, operand_bytes, iters, ctypes.byref(flops), stream))
+    return flops.value
+
+
+def calib_mfma_xcds(sink, operands, operand_bytes, iters, active_xcds, stream=None):
+    """The bare MFMA loop on the first `active_xcds` XCDs only; returns the flops of one running workgroup."""
+    flops = ctypes.c_double(0.0)
+    check(load().lmh_calib_mfma_xcds(sink, operands, operand_bytes, iters, active_xcds, ctypes.byref(flops), stream))
     return flops.value
 
 

@@ -276,7 +276,7 @@ int lmh_flash_attn_fwd(const lmh_attn_params *p) {
     return fail(LMH_E_UNSUPPORTED, "lmh_flash_attn_fwd: unknown dtype %d", p->dtype);
   if (p->head_map != LMH_HEADMAP_INTERLEAVED && p->head_map != LMH_HEADMAP_BLOCKED)
     return fail(LMH_E_UNSUPPORTED, "lmh_flash_attn_fwd: unknown head_map %d", p->head_map);
-  if (p->D > 128) return fail(LMH_E_UNSUPPORTED, "lmh_flash_attn_fwd: head dim %d > 128 is not supported", p->D);
+  if (p->D > 256) return fail(LMH_E_UNSUPPORTED, "lmh_flash_attn_fwd: head dim %d > 256 is not supported", p->D);
   if (!(p->scale == p->scale)) return fail(LMH_E_SHAPE, "lmh_flash_attn_fwd: scale is NaN");
 
   PrefillArgs a;

@@ -16,8 +16,17 @@ typedef float calib_floatx16_t __attribute__((ext_vector_type(16)));
 constexpr int kCalibMfmaGrid = 512;    // two workgroups per CU
 constexpr int kCalibMfmaPerIter = 8;   // MFMAs per wave per loop iteration
 
+// active_xcds < 8: workgroups that land on XCD `active_xcds` or above (the hardware's own XCC_ID) leave at once and
+// mark their first sink slot with -1, so the loop runs on part of the chip while the rest idles.
 __global__ __launch_bounds__(256, 2) void calib_mfma_kernel(float *__restrict__ sink, const calib_half8_t *__restrict__ operands,
-                                                            int n_operands, int iters) {
+                                                            int n_operands, int iters, int active_xcds) {
+  if (active_xcds < 8) {
+    const int xcc = __builtin_amdgcn_s_getreg(20 | (3 << 11)) & 15;  // HW_REG_XCC_ID, bits 3:0
+    if (xcc >= active_xcds) {
+      if (threadIdx.x == 0) sink[blockIdx.x * 256] = -1.f;
+      return;
+    }
+  }
   calib_half8_t a[4], b[4];
 #pragma unroll
   for (int i = 0; i < 4; i++) {
@@ -62,14 +71,23 @@ extern "C" int lmh_calib_copy(void *dst, const void *src, size_t bytes, void *st
   return LMH_OK;
 }
 
-extern "C" int lmh_calib_mfma(void *sink, const void *operands, size_t operand_bytes, int iters, double *flops, void *stream) {
+extern "C" int lmh_calib_mfma_xcds(void *sink, const void *operands, size_t operand_bytes, int iters, int active_xcds,
+                                   double *flops_per_workgroup, void *stream) {
   using namespace lmh;
   if (!sink || !operands) return fail(LMH_E_NULL, "lmh_calib_mfma: null pointer");
   if (operand_bytes < 32 || operand_bytes % 16 != 0 || (reinterpret_cast<uintptr_t>(operands) & 15u) || iters < 1)
     return fail(LMH_E_SHAPE, "lmh_calib_mfma: operands must be >= 32 bytes, a multiple of 16, 16-byte aligned; iters >= 1");
+  if (active_xcds < 1 || active_xcds > 8) return fail(LMH_E_SHAPE, "lmh_calib_mfma_xcds: active_xcds must be 1..8");
   hipLaunchKernelGGL(calib_mfma_kernel, dim3(kCalibMfmaGrid), dim3(256), 0, (hipStream_t)stream, reinterpret_cast<float *>(sink),
-                     reinterpret_cast<const calib_half8_t *>(operands), (int)(operand_bytes / 16), iters);
+                     reinterpret_cast<const calib_half8_t *>(operands), (int)(operand_bytes / 16), iters, active_xcds);
   LMH_HIP_TRY(hipGetLastError());
-  if (flops) *flops = (double)kCalibMfmaGrid * 4.0 * iters * kCalibMfmaPerIter * (2.0 * 32 * 32 * 16);
+  if (flops_per_workgroup) *flops_per_workgroup = 4.0 * iters * kCalibMfmaPerIter * (2.0 * 32 * 32 * 16);
   return LMH_OK;
+}
+
+extern "C" int lmh_calib_mfma(void *sink, const void *operands, size_t operand_bytes, int iters, double *flops, void *stream) {
+  double per_wg = 0.0;
+  const int rc = lmh_calib_mfma_xcds(sink, operands, operand_bytes, iters, 8, &per_wg, stream);
+  if (rc == LMH_OK && flops) *flops = per_wg * lmh::kCalibMfmaGrid;
+  return rc;
 }

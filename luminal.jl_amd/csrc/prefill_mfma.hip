@@ -125,6 +125,11 @@ __global__ __launch_bounds__(64 * NW, WPS) void prefill_mfma_kernel(PrefillArgs 
   __shared__ __attribute__((aligned(16))) uint16_t Ks2[2][BT * LDK];  // double-buffered tiles
   __shared__ __attribute__((aligned(16))) uint16_t Vs2[2][BT * LDV];
 
+#ifdef LMH_ONLY_XCDS
+  // Measurement build (results wrong by construction): only workgroups dispatched to the first LMH_ONLY_XCDS XCDs
+  // work, the rest exit at once — the same instruction stream with part of the chip idle.
+  if ((blockIdx.x & 7) >= LMH_ONLY_XCDS) return;
+#endif
   // ---- which (b, hq, query tile) this workgroup owns ----
   const int bid = blockIdx.x;
   const int xcd = bid & 7;
@@ -479,6 +484,9 @@ int launch_for_d(const PrefillArgs &a, hipStream_t stream) {
   // 46.7 us at B=1 H=32 S=2048 D=96) and loses for non-causal ones (79.8 vs 66.6 us); at three per
   // CU it loses for both.
   const int n_cus = device_cu_count();
+#ifdef LMH_NWX
+  if (!a.causal && a.Sq <= 32 * LMH_NWX * 2 && D == 64) return launch_split<MT, D, 1, LMH_NWX, 2>(a, stream);
+#endif
   const int64_t wgs = (int64_t)((a.B * a.Hq + 7) / 8) * 8 * ((a.Sq + 127) / 128);
   const int64_t limit = a.causal ? 2 * n_cus : 2 * n_cus - 1;
   if (wgs <= limit && a.Sk >= 4 * BN) return launch_split<MT, D, 2, 4>(a, stream);

@@ -1,5 +1,6 @@
 // Flash attention forward on the vector ALUs: the fp32 path (parity budget 1e-5, which rules
-// out half-precision matrix cores) and the fallback for head dims the MFMA kernel does not tile.
+// out half-precision matrix cores) and the fallback for head dims the MFMA kernels do not tile
+// (anything that is not a multiple of 8, and 129 .. 256, the range decode attention accepts too).
 //
 // Same recurrence as flash_attn_cpu (reference src/Execution.jl:453-479), evaluated a tile of
 // 32 keys at a time: m' = max(m, tile max), o = o*exp(m-m') + sum_j exp(s_j-m') v_j,
@@ -16,12 +17,14 @@ namespace {
 
 constexpr int kRowsPerWg = 64;
 constexpr int kLanesPerRow = 4;
-constexpr int kKeysPerTile = 32;
+// keys per staged tile: 32; 16 for head dims above 128, whose fp32 tiles would not fit the 64 KB of static LDS
+template <int DP> constexpr int keys_per_tile() { return DP > 128 ? 16 : 32; }
 
 template <typename E, int DP>
 __global__ __launch_bounds__(256) void prefill_valu_kernel(PrefillArgs a) {
   using raw = typename E::raw;
   constexpr int NCH = DP / 16;  // float4 chunks per lane
+  constexpr int kKeysPerTile = keys_per_tile<DP>();
   __shared__ float4 Ks[kKeysPerTile][DP / 4];
   __shared__ float4 Vs[kKeysPerTile][DP / 4];
 
@@ -141,7 +144,9 @@ int launch_for_dtype(const PrefillArgs &a, hipStream_t stream) {
   else if (a.D <= 64) hipLaunchKernelGGL((prefill_valu_kernel<E, 64>), grid, block, 0, stream, a);
   else if (a.D <= 96) hipLaunchKernelGGL((prefill_valu_kernel<E, 96>), grid, block, 0, stream, a);
   else if (a.D <= 128) hipLaunchKernelGGL((prefill_valu_kernel<E, 128>), grid, block, 0, stream, a);
-  else return fail(LMH_E_UNSUPPORTED, "flash attention: head dim %d > 128 is not supported", a.D);
+  else if (a.D <= 192) hipLaunchKernelGGL((prefill_valu_kernel<E, 192>), grid, block, 0, stream, a);
+  else if (a.D <= 256) hipLaunchKernelGGL((prefill_valu_kernel<E, 256>), grid, block, 0, stream, a);
+  else return fail(LMH_E_UNSUPPORTED, "flash attention: head dim %d > 256 is not supported", a.D);
   LMH_HIP_TRY(hipGetLastError());
   return LMH_OK;
 }

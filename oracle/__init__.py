@@ -131,12 +131,23 @@ def flash_attn(q, k, v, scale=None, causal=False, head_map=HEADMAP_INTERLEAVED, 
 
 
 def decode_attn(q, k_cache, v_cache, kv_len=None, scale=None, head_map=HEADMAP_INTERLEAVED, nthreads=1):
-    """q [B,Hq,D], caches [B,Hkv,Lmax,D] -> [B,Hq,D] fp32."""
-    q = np.ascontiguousarray(q, dtype=np.float32)
+    """q [B,Hq,D], caches [B,Hkv,Lmax,D] -> [B,Hq,D] fp32, through the oracle's own decode entry lmo_decode_attn
+    (the cached attention of reference src/Whisper.jl:610-616: one query row over the first kv_len[b] cache rows)."""
+    q, qp = _f32(q)
+    k, kp = _f32(k_cache)
+    v, vp = _f32(v_cache)
     B, Hq, D = q.shape
-    out = flash_attn(q.reshape(B, Hq, 1, D), k_cache, v_cache, scale=scale, causal=False, head_map=head_map,
-                     kv_len=kv_len, nthreads=nthreads)
-    return out.reshape(B, Hq, D)
+    _, Hkv, Lmax, _ = k.shape
+    assert k.shape == v.shape and k.shape[0] == B and k.shape[3] == D
+    if scale is None:
+        scale = np.float32(1.0) / np.sqrt(np.float32(D))
+    kv, kvp = _i32_or_null(kv_len)
+    out = np.empty_like(q)
+    rc = lib().lmo_decode_attn(out.ctypes.data_as(ctypes.POINTER(ctypes.c_float)), qp, kp, vp, kvp, B, Hq, Hkv, Lmax, D,
+                               float(scale), head_map, nthreads)
+    if rc != 0:
+        raise ValueError("oracle rejected the arguments")
+    return out
 
 
 def naive_attention_f64(q, k, v, scale=None, causal=False, head_map=HEADMAP_INTERLEAVED, kv_len=None):

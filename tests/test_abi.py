@@ -44,7 +44,7 @@ def _attn(lm, **kw):
 
 @pytest.mark.parametrize("kw,code", [
     (dict(q=None), -1), (dict(out=None), -1), (dict(B=0), -2), (dict(D=-3), -2), (dict(Hq=5), -2),
-    (dict(dtype=7), -3), (dict(head_map=9), -3), (dict(D=256), -3), (dict(scale=float("nan")), -2),
+    (dict(dtype=7), -3), (dict(head_map=9), -3), (dict(D=264), -3), (dict(scale=float("nan")), -2),
 ])
 def test_flash_attn_argument_errors(lm, kw, code):
     with pytest.raises(lm.LuminalHipError) as e:

@@ -224,3 +224,20 @@ def test_kv_append_equals_slice_and_concat_scatter(oracle):
     want[0, :, 1:4] = new[0]
     want[1, :, 3:5] = new[1, :, :2]
     np.testing.assert_array_equal(got, want)
+
+
+def test_decode_entry_is_the_one_row_prefill(oracle):
+    # lmo_decode_attn (what oracle.decode_attn calls) is the restated recurrence on one query row over the first
+    # kv_len[b] cache rows: bit for bit the Sq = 1 non-causal call, and the float64 softmax over exactly those rows
+    B, Hq, Hkv, L, D = 3, 8, 2, 77, 32
+    q = oracle.gen_normal((B, Hq, D), 40)
+    k = oracle.gen_normal((B, Hkv, L, D), 41)
+    v = oracle.gen_normal((B, Hkv, L, D), 42)
+    lens = np.array([77, 1, 30], np.int32)
+    for head_map in (0, 1):
+        got = oracle.decode_attn(q, k, v, kv_len=lens, head_map=head_map)
+        same = oracle.flash_attn(q[:, :, None], k, v, kv_len=lens, head_map=head_map)[:, :, 0]
+        np.testing.assert_array_equal(got, same)
+        for b, n in enumerate(lens):
+            ref = oracle.naive_attention_np(q[b:b + 1, :, None], k[b:b + 1, :, :n], v[b:b + 1, :, :n], head_map=head_map)[:, :, 0]
+            np.testing.assert_allclose(got[b:b + 1], ref, rtol=1e-5, atol=1e-6)

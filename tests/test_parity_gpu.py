@@ -160,6 +160,17 @@ def test_fp32_head_dims(lm, hip, oracle, D, causal):
     assert rel_err(run_flash(lm, hip, q, k, v, "f32", causal), oracle.flash_attn(q, k, v, causal=causal)) <= 1e-5
 
 
+@pytest.mark.parametrize("dtype", ["f32", "f16", "bf16"])
+@pytest.mark.parametrize("D", [136, 160, 192, 256])
+def test_head_dims_above_128_run_on_the_vector_kernel(lm, hip, oracle, dtype, D):
+    # decode accepts head dims up to 256; prefill does too (a model with D = 256 must be able to do both)
+    q, k, v = inputs(oracle, (2, 4, 70, D), (2, 2, 90, D), dtype, 7150 + D)
+    lens = np.array([90, 41], np.int32)
+    for causal in (False, True):
+        got = run_flash(lm, hip, q, k, v, dtype, causal, kv_len=lens)
+        assert rel_err(got, oracle.flash_attn(q, k, v, causal=causal, kv_len=lens)) <= TOL[dtype]
+
+
 @pytest.mark.parametrize("Sq,Sk", [(1, 1), (1, 77), (7, 7), (64, 64), (65, 130), (130, 65), (257, 300)])
 @pytest.mark.parametrize("causal", [False, True])
 def test_fp32_sequence_shapes(lm, hip, oracle, Sq, Sk, causal):
