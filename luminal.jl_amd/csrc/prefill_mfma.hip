@@ -170,13 +170,6 @@ __global__ __launch_bounds__(64 * NW, WPS) void prefill_mfma_kernel(PrefillArgs 
     uint4 raw = make_uint4(0, 0, 0, 0);
     if (qi < a.Sq && 16 * ks + 8 * g < a.D) raw = *reinterpret_cast<const uint4 *>(qp + (int64_t)qi * a.qs[2] + 16 * ks + 8 * g);
     qreg[ks] = __builtin_bit_cast(vec8, raw);
-#ifdef LMH_FOLD
-    {
-      const float cq = a.scale * kLog2e;
-#pragma unroll
-      for (int e = 0; e < 8; e++) qreg[ks][e] = MT::cvt((float)qreg[ks][e] * cq);
-    }
-#endif
   }
 
   floatx16_t oacc[DB];
@@ -186,14 +179,7 @@ __global__ __launch_bounds__(64 * NW, WPS) void prefill_mfma_kernel(PrefillArgs 
     for (int i = 0; i < 16; i++) oacc[db][i] = 0.f;
   float m_i = -INFINITY;  // running max of the raw (unscaled) scores of query qi
   float l_i = 0.f;        // this lane's half of the running sum
-#ifdef LMH_FOLD
-  const float c = 1.0f;   // the scores leave the matrix cores in log2 units, already minus the running max
-  floatx16_t negm;        // -m_i in every register: the C operand of each block's first MFMA
-#pragma unroll
-  for (int i = 0; i < 16; i++) negm[i] = 0.f;
-#else
   const float c = a.scale * kLog2e;
-#endif
 
   // ---- tile staging: global memory -> LDS directly (buffer_load_dwordx4 ... lds), one tile ahead ----
   // A tile of BT rows x LD elements is BT * LD / 512 blocks of 1 KB. One wave-wide load fills one block:
@@ -289,12 +275,10 @@ __global__ __launch_bounds__(64 * NW, WPS) void prefill_mfma_kernel(PrefillArgs 
     // ---- S^T = K Q^T for the wave's 32-key blocks, two at a time: their fragments are fetched first, then
     // the two accumulator chains alternate so that neither waits on LDS or on its own previous MFMA ----
     floatx16_t sacc[NKB];
-#ifndef LMH_FOLD
 #pragma unroll
     for (int kb = 0; kb < NKB; kb++)
 #pragma unroll
       for (int i = 0; i < 16; i++) sacc[kb][i] = 0.f;
-#endif
     constexpr int KBG = NKB < 2 ? NKB : 2;  // key blocks whose fragments are fetched together
 #pragma unroll
     for (int kb0 = 0; kb0 < NKB; kb0 += KBG) {
@@ -308,11 +292,7 @@ __global__ __launch_bounds__(64 * NW, WPS) void prefill_mfma_kernel(PrefillArgs 
       for (int ks = 0; ks < KS; ks++)
 #pragma unroll
         for (int kb = 0; kb < KBG; kb++) {
-#ifdef LMH_FOLD
-          sacc[kb0 + kb] = MT::mfma(kf[kb][ks], qreg[ks], ks == 0 ? negm : sacc[kb0 + kb]);
-#else
           sacc[kb0 + kb] = MT::mfma(kf[kb][ks], qreg[ks], sacc[kb0 + kb]);
-#endif
         }
     }
 
@@ -335,26 +315,6 @@ __global__ __launch_bounds__(64 * NW, WPS) void prefill_mfma_kernel(PrefillArgs 
 #pragma unroll
       for (int i = 0; i < 16; i++) mx = fmaxf(mx, sacc[kb][i]);
     mx = fmaxf(mx, __shfl_xor(mx, 32));
-#ifdef LMH_FOLD
-    // sacc holds (score - m_i) in log2 units (m_i = 0 before the first tile, whose maximum is always taken)
-    if (__builtin_amdgcn_ballot_w64(m_i == -INFINITY || mx > kLazyRescale) != 0) {  // wave-uniform
-      const float delta = m_i == -INFINITY ? mx : fmaxf(mx, 0.f);  // how far the running max moves
-      const float alpha = m_i == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(-delta);
-      m_i = (m_i == -INFINITY ? 0.f : m_i) + delta;
-      l_i *= alpha;
-#pragma unroll
-      for (int db = 0; db < DB; db++)
-#pragma unroll
-        for (int i = 0; i < 16; i++) oacc[db][i] *= alpha;
-#pragma unroll
-      for (int i = 0; i < 16; i++) negm[i] = -m_i;
-#pragma unroll
-      for (int kb = 0; kb < NKB; kb++)
-#pragma unroll
-        for (int i = 0; i < 16; i++) sacc[kb][i] -= delta;
-    }
-    const float mc = 0.f;
-#else
     // m_i is finite after the first tile (key 0 is visible to every query); -inf before it.
     if (__builtin_amdgcn_ballot_w64((mx - m_i) * c > kLazyRescale) != 0) {  // wave-uniform
       const float m_new = fmaxf(m_i, mx);
@@ -367,7 +327,6 @@ __global__ __launch_bounds__(64 * NW, WPS) void prefill_mfma_kernel(PrefillArgs 
         for (int i = 0; i < 16; i++) oacc[db][i] *= alpha;
     }
     const float mc = m_i * c;
-#endif
     vec8 pf[NKB][2], pf_lo[NKB][2];
 #pragma unroll
     for (int kb = 0; kb < NKB; kb++)
@@ -375,11 +334,7 @@ __global__ __launch_bounds__(64 * NW, WPS) void prefill_mfma_kernel(PrefillArgs 
       for (int t = 0; t < 2; t++) {
 #pragma unroll
         for (int e = 0; e < 8; e++) {
-#ifdef LMH_FOLD
-          const float p = __builtin_amdgcn_exp2f(sacc[kb][8 * t + e]);
-#else
           const float p = __builtin_amdgcn_exp2f(sacc[kb][8 * t + e] * c - mc);
-#endif
           pf[kb][t][e] = MT::cvt(p);
           if (MT::kSplitP) pf_lo[kb][t][e] = MT::cvt(p - (float)pf[kb][t][e]);
         }
@@ -484,9 +439,6 @@ int launch_for_d(const PrefillArgs &a, hipStream_t stream) {
   // 46.7 us at B=1 H=32 S=2048 D=96) and loses for non-causal ones (79.8 vs 66.6 us); at three per
   // CU it loses for both.
   const int n_cus = device_cu_count();
-#ifdef LMH_NWX
-  if (!a.causal && a.Sq <= 32 * LMH_NWX * 2 && D == 64) return launch_split<MT, D, 1, LMH_NWX, 2>(a, stream);
-#endif
   const int64_t wgs = (int64_t)((a.B * a.Hq + 7) / 8) * 8 * ((a.Sq + 127) / 128);
   const int64_t limit = a.causal ? 2 * n_cus : 2 * n_cus - 1;
   if (wgs <= limit && a.Sk >= 4 * BN) return launch_split<MT, D, 2, 4>(a, stream);
