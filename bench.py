@@ -369,6 +369,22 @@ def c4_leg(lm, dev, res, check, caches=None):
     res[name] = {"launch_us": ev * 1e3, "GB/s": nbytes / (ev * 1e-3) / 1e9, "frac_of_hbm_peak": nbytes / (ev * 1e-3) / 1e9 / PEAK_HBM_GBS,
                  "num_splits": int(ps[0].num_splits), "launch_us_one_by_one": per_launch_us(step, 20, lm.binding)}
     log("[other] C4 decode: %.1f us, %.0f GB/s, %d splits" % (ev * 1e3, nbytes / (ev * 1e-3) / 1e9, ps[0].num_splits))
+    # what a kernel that only reads 268 MB takes, launch included (four buffers in rotation, like the caches): the
+    # ceiling of any decode kernel at this size
+    sink = lm.HipArray((4,), "f32", dev)
+    total = 2 * B * Hkv * L * D * 2
+    probes = [lm.HipArray((total // 4,), "f32", dev).fill_bytes(1) for _ in range(4)]
+
+    def read_step():
+        lm.binding.calib_read(probes[state["i"] % 4].ptr, total, sink.ptr)
+        state["i"] += 1
+
+    _, evr = time_steps(read_step, 40, 8, lm.binding)
+    res[name]["plain_read_of_the_same_bytes_us"] = evr * 1e3
+    res[name]["frac_of_plain_read_rate"] = evr / ev
+    for pb in probes:
+        pb.free()
+    log("[other] plain read of 268 MB in one launch: %.1f us, %.0f GB/s" % (evr * 1e3, total / (evr * 1e-3) / 1e9))
     if check:
         import oracle
         lm.binding.decode_attn(ps[0])

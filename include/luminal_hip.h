@@ -100,6 +100,10 @@ int lmh_graph_destroy(void *graph_exec);
  * writes `bytes`; both pointers and the size multiples of 16) used to calibrate HBM traffic
  * counters against a known transfer. */
 int lmh_calib_copy(void *dst_dev, const void *src_dev, size_t bytes, void *stream);
+/* ... and a read-only stream over `bytes` (a multiple of 4096) with non-temporal 16-byte loads, 8 in flight per lane:
+ * the rate the memory system delivers to a kernel that does nothing else, the practical ceiling of the decode
+ * kernels at a given size. `sink4_dev` is 4 bytes of device memory (never written in practice). */
+int lmh_calib_read(const void *src_dev, size_t bytes, void *sink4_dev, void *stream);
 
 /* Measurement aid with no counterpart in the reference: a bare loop of fp16 MFMAs (512 workgroups, 4
  * waves each, 8 v_mfma_f32_32x32x16_f16 per iteration) on operands read from `operands_dev`

@@ -23,7 +23,7 @@ EXPORTS = [
     "lmh_version", "lmh_last_error", "lmh_device_count", "lmh_init", "lmh_device_name", "lmh_malloc", "lmh_free",
     "lmh_memset", "lmh_memcpy_h2d", "lmh_memcpy_d2h", "lmh_memcpy_d2d", "lmh_sync", "lmh_event_create",
     "lmh_event_destroy", "lmh_event_record", "lmh_event_elapsed_ms", "lmh_flash_attn_fwd",
-    "lmh_decode_workspace_bytes", "lmh_decode_auto_splits", "lmh_decode_attn", "lmh_calib_copy", "lmh_calib_mfma",
+    "lmh_decode_workspace_bytes", "lmh_decode_auto_splits", "lmh_decode_attn", "lmh_calib_copy", "lmh_calib_read", "lmh_calib_mfma",
     "lmh_calib_mfma_xcds", "lmh_rope",
     "lmh_kv_append", "lmh_stream_create", "lmh_stream_destroy", "lmh_graph_capture_begin", "lmh_graph_capture_end",
     "lmh_graph_launch", "lmh_graph_destroy", "lmh_static_scratch_bytes", "lmh_decode_static_splits",
@@ -131,6 +131,8 @@ def load():
     L.lmh_decode_static_splits.argtypes = [ctypes.c_int32] * 5
     L.lmh_calib_copy.argtypes = [vp, vp, ctypes.c_size_t, vp]
     L.lmh_calib_mfma.argtypes = [vp, vp, ctypes.c_size_t, ctypes.c_int, ctypes.POINTER(ctypes.c_double), vp]
+    L.lmh_calib_read.argtypes = [vp, ctypes.c_size_t, vp, vp]
+    L.lmh_calib_read.restype = ctypes.c_int
     L.lmh_calib_mfma_xcds.argtypes = [vp, vp, ctypes.c_size_t, ctypes.c_int, ctypes.c_int, ctypes.POINTER(ctypes.c_double), vp]
     L.lmh_calib_mfma_xcds.restype = ctypes.c_int
     L.lmh_rope.argtypes = [ctypes.POINTER(RopeParams)]
@@ -141,7 +143,7 @@ def load():
     L.lmh_graph_capture_end.argtypes = [vp, ctypes.POINTER(vp)]
     L.lmh_graph_launch.argtypes = [vp, vp]
     L.lmh_graph_destroy.argtypes = [vp]
-    for name in ("lmh_rope", "lmh_kv_append", "lmh_calib_copy", "lmh_calib_mfma", "lmh_init", "lmh_device_name", "lmh_malloc", "lmh_free", "lmh_memset", "lmh_memcpy_h2d",
+    for name in ("lmh_rope", "lmh_kv_append", "lmh_calib_copy", "lmh_calib_read", "lmh_calib_mfma", "lmh_init", "lmh_device_name", "lmh_malloc", "lmh_free", "lmh_memset", "lmh_memcpy_h2d",
                  "lmh_memcpy_d2h", "lmh_memcpy_d2d", "lmh_sync", "lmh_event_create", "lmh_event_destroy",
                  "lmh_event_record", "lmh_event_elapsed_ms", "lmh_flash_attn_fwd", "lmh_decode_attn"):
         getattr(L, name).restype = ctypes.c_int
@@ -279,6 +281,10 @@ def graph_destroy(graph_exec):
 
 def calib_copy(dst, src, nbytes, stream=None):
     check(load().lmh_calib_copy(dst, src, nbytes, stream))
+
+
+def calib_read(src, nbytes, sink4, stream=None):
+    check(load().lmh_calib_read(src, nbytes, sink4, stream))
 
 
 def calib_mfma(sink, operands, operand_bytes, iters, stream=None):

@@ -373,7 +373,9 @@ static int decode_launch(const lmh_decode_params *p, const char *fn, int32_t num
   if (a.ks[2] < p->D || a.vs[2] < p->D) return fail(LMH_E_SHAPE, "%s: cache row stride smaller than head dim", fn);
   if (a.qs[0] < 0 || a.qs[1] < 0 || a.os[0] < 0 || a.os[1] < 0) return fail(LMH_E_SHAPE, "%s: negative stride", fn);
 
-  a.mfma_ok = (p->scale > 0.f && aligned16(p->q) && a.qs[0] % 8 == 0 && a.qs[1] % 8 == 0) ? 1 : 0;
+  // the matrix-core kernel addresses a (b, kv head) slice with 32-bit buffer offsets
+  const bool slice_fits = (int64_t)p->Lmax * a.ks[2] * 2 < 0x7ffffff0 && (int64_t)p->Lmax * a.vs[2] * 2 < 0x7ffffff0;
+  a.mfma_ok = (p->scale > 0.f && aligned16(p->q) && a.qs[0] % 8 == 0 && a.qs[1] % 8 == 0 && slice_fits) ? 1 : 0;
   a.num_splits = num_splits;
   a.chunk = decode_chunk_for(p->Lmax, a.num_splits);
   a.ws_o = nullptr;

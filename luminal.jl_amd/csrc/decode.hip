@@ -437,7 +437,9 @@ int decode_chunk_for(int Lmax, int num_splits) {
 }
 
 int launch_decode(const DecodeArgs &a, int dtype, hipStream_t stream) {
-  if (a.mfma_ok && decode_mfma_supported(dtype, a.D, a.B)) {
+  // (the matrix-core kernel deals its (b, kv head slice, chunk) units in 32-bit arithmetic)
+  const int64_t mfma_units = (int64_t)a.B * a.Hkv * ((a.Hq / a.Hkv + 15) / 16) * a.num_splits;
+  if (a.mfma_ok && decode_mfma_supported(dtype, a.D, a.B) && mfma_units < (int64_t(1) << 31)) {
     const int rc = launch_decode_mfma_split(a, dtype, stream);
     if (rc != LMH_OK) return rc;
     return dtype == LMH_F16 ? launch_merge<F16>(a, stream) : launch_merge<BF16>(a, stream);

@@ -113,9 +113,25 @@ __global__ __launch_bounds__(kWaves * 64) void decode_mfma_kernel(DecodeArgs a, 
     if (lane == 0) s_pref[0] = 0;
   }
   __syncthreads();
-  const int64_t total_units = (int64_t)s_pref[a.B] * kv_slots;
-  int64_t u = total_units * blockIdx.x / gridDim.x;
-  const int64_t u_end = total_units * (blockIdx.x + 1) / gridDim.x;
+  // Equal contiguous shares of the units, in 32-bit arithmetic (the launcher routes batches with 2^31 units or more to
+  // the other kernel): the first total % grid workgroups take one unit more. 64-bit divisions are ~100 scalar
+  // instructions each on this hardware, and five of them stood between a workgroup's start and its first load.
+  const uint32_t total_units = (uint32_t)s_pref[a.B] * (uint32_t)kv_slots;
+  const uint32_t share = total_units / gridDim.x, extra = total_units % gridDim.x;
+  uint32_t u = blockIdx.x * share + min((uint32_t)blockIdx.x, extra);
+  const uint32_t u_end = u + share + (blockIdx.x < extra ? 1u : 0u);
+
+  // Per-lane byte offsets of the NL 16-byte loads of a 32-key block, relative to the block's first row: load r of lane l
+  // fetches chunk (r * 64 + l) of the block, i.e. row (r * 64 + l) / CPR, 16-byte column (r * 64 + l) % CPR. They do not
+  // depend on the block, so they are computed once; a block's own position goes into the scalar offset of the load.
+  int k_voff[NL], v_voff[NL];
+#pragma unroll
+  for (int r = 0; r < NL; r++) {
+    const int id = r * 64 + lane;
+    k_voff[r] = (int)(((id / CPR) * a.ks[2] + (id % CPR) * 8) * 2);
+    v_voff[r] = (int)(((id / CPR) * a.vs[2] + (id % CPR) * 8) * 2);
+  }
+  const int k_row_bytes = (int)(a.ks[2] * 2), v_row_bytes = (int)(a.vs[2] * 2);
 
   uint16_t *Ks = reinterpret_cast<uint16_t *>(smem + wave * kTileBytes);
   uint16_t *Vs = Ks + kBlk * LDK;
@@ -128,15 +144,15 @@ __global__ __launch_bounds__(kWaves * 64) void decode_mfma_kernel(DecodeArgs a, 
     int lo = 0, hi = a.B;  // largest b with s_pref[b] * kv_slots <= u
     while (hi - lo > 1) {
       const int mid = (lo + hi) >> 1;
-      if ((int64_t)s_pref[mid] * kv_slots <= u) lo = mid; else hi = mid;
+      if ((uint32_t)s_pref[mid] * (uint32_t)kv_slots <= u) lo = mid; else hi = mid;
     }
     const int b = lo;
     const int n_chunks = s_pref[b + 1] - s_pref[b];
-    const int64_t rem = u - (int64_t)s_pref[b] * kv_slots;
-    const int slot_id = (int)(rem / n_chunks);
-    const int c0 = (int)(rem % n_chunks);
-    const int c1 = (int)min((int64_t)n_chunks, c0 + (u_end - u));
-    u += c1 - c0;
+    const uint32_t rem = u - (uint32_t)s_pref[b] * (uint32_t)kv_slots;
+    const int slot_id = (int)(rem / (uint32_t)n_chunks);
+    const int c0 = (int)(rem % (uint32_t)n_chunks);
+    const int c1 = (int)min((uint32_t)n_chunks, c0 + (u_end - u));
+    u += (uint32_t)(c1 - c0);
     const int kvh = slot_id / g_chunks;
     const int g0 = (slot_id % g_chunks) * 16;  // first group member handled here
     const int n_heads = min(16, group - g0);
@@ -170,19 +186,21 @@ __global__ __launch_bounds__(kWaves * 64) void decode_mfma_kernel(DecodeArgs a, 
   float m_i = -INFINITY;  // running max of the raw scores of head n (same in the 4 lanes of a head)
   float l_i = 0.f;        // this lane's share of the running sum
 
+  // Raw buffer descriptors over the valid rows [0, end) of this (b, kv head) slice: a load past `end` returns zeros
+  // without a branch, so the loads of a block are NL back-to-back instructions (address = lane-invariant offset +
+  // scalar block offset). Non-temporal, like every cache stream of this library.
+  const __amdgpu_buffer_rsrc_t k_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<uint16_t *>(kbase), 0, __builtin_amdgcn_readfirstlane(end * k_row_bytes), 0x00020000);
+  const __amdgpu_buffer_rsrc_t v_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<uint16_t *>(vbase), 0, __builtin_amdgcn_readfirstlane(end * v_row_bytes), 0x00020000);
   uint4 kreg[NL], vreg[NL];
   auto load_tile = [&](int key0) {
+    const int k_soff = __builtin_amdgcn_readfirstlane(key0 * k_row_bytes);
+    const int v_soff = __builtin_amdgcn_readfirstlane(key0 * v_row_bytes);
 #pragma unroll
     for (int r = 0; r < NL; r++) {
-      const int id = r * 64 + lane;
-      const int row = id / CPR, col = id % CPR;
-      const int key = key0 + row;
-      kreg[r] = make_uint4(0, 0, 0, 0);
-      vreg[r] = make_uint4(0, 0, 0, 0);
-      if (key < end) {
-        kreg[r] = load_stream_128(kbase + (int64_t)key * a.ks[2] + col * 8);
-        vreg[r] = load_stream_128(vbase + (int64_t)key * a.vs[2] + col * 8);
-      }
+      kreg[r] = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(k_rsrc, k_voff[r], k_soff, 2));
+      vreg[r] = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(v_rsrc, v_voff[r], v_soff, 2));
     }
   };
   auto store_tile = [&]() {
@@ -351,6 +369,7 @@ int launch_for_d(const DecodeArgs &a, hipStream_t stream) {
   const int group = a.Hq / a.Hkv;
   const int g_chunks = (group + 15) / 16;
   const int64_t max_units = (int64_t)a.B * a.Hkv * g_chunks * a.num_splits;
+  if (max_units >= (int64_t(1) << 31)) return fail(LMH_E_UNSUPPORTED, "MFMA decode: %lld units do not fit 32 bits", (long long)max_units);
   const int n_wgs = (int)(max_units < wgs_per_device ? max_units : wgs_per_device);
   hipLaunchKernelGGL((decode_mfma_kernel<MT, D>), dim3(n_wgs), dim3(kWaves * 64), 0, stream, a, g_chunks);
   LMH_HIP_TRY(hipGetLastError());
