@@ -502,6 +502,20 @@ def ceiling_leg(lm, dev):
             "frac_of_peak_scaled": tf * 8 / active / PEAK_FP16_TFLOPS}
         log("[ceiling] bare MFMA loop on %d XCD(s): %d of 512 workgroups ran, %.0f TFLOP/s = %.0f scaled to the chip (%.1f%% of peak)"
             % (active, ran, tf, tf * 8 / active, 100 * tf * 8 / active / PEAK_FP16_TFLOPS))
+    # the ceiling of a kernel with attention's instruction mix: synthetic interleaved streams on the whole chip
+    mixes = ["MFMA only", "MFMA + 6 vector instr (1 exp)", "MFMA + 6 vector instr (1 exp) + 1 LDS fragment read",
+             "MFMA + 6 vector instr (1 exp) + 1 LDS fragment read per 2 MFMAs", "MFMA + 4 vector instr (1 exp) + 1 LDS fragment read",
+             "MFMA + 4 vector instr (1 exp) + 1 LDS fragment read per 2 MFMAs"]
+    res["instruction_mix_streams"] = {}
+    for mix, label in enumerate(mixes):
+        fl = [0.0]
+
+        def fn():
+            fl[0] = lm.binding.calib_mix(sink.ptr, dq.ptr, 1 << 17, 10000, mix)
+        _, ev = time_steps(fn, 3, 1, lm.binding)
+        tf = fl[0] / (ev * 1e-3) / 1e12
+        res["instruction_mix_streams"][label] = {"TFLOP/s": tf, "frac_of_peak": tf / PEAK_FP16_TFLOPS}
+        log("[ceiling] synthetic stream, %s: %.0f TFLOP/s (%.1f%% of peak)" % (label, tf, 100 * tf / PEAK_FP16_TFLOPS))
     out = lm.HipArray((B, H, S, D), "f16", dev)
     p = attn_params(lm, out, dq, dk, dv, "f16", False, lm.default_scale(D))
     _, ev = time_steps(lambda: lm.binding.flash_attn_fwd(p), 10, 3, lm.binding)

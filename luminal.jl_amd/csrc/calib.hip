@@ -56,6 +56,57 @@ __global__ __launch_bounds__(256) void calib_copy_kernel(uint4 *__restrict__ dst
   const size_t stride = (size_t)gridDim.x * blockDim.x;
   for (; i < n; i += stride) dst[i] = src[i];
 }
+// An interleaved stream with a chosen instruction mix per MFMA: NV vector instructions (NE of them v_exp_f32, the
+// rest fused multiply-adds) and one 16-byte-per-lane LDS read every LDS_EVERY MFMAs (0 = none; the fragment read
+// feeds the A operand of the next LDS_EVERY MFMAs). Two waves per SIMD, operands from caller-supplied values. This
+// is the best case of a kernel with that mix — no barriers, no staging, no dependencies between the MFMA and the
+// vector work — so its rate on the whole chip is the ceiling for an attention kernel of the same mix.
+template <int NV, int NE, int LDS_EVERY>
+__global__ __launch_bounds__(512) void calib_mix_kernel(float *__restrict__ sink, const calib_half8_t *__restrict__ operands,
+                                                        int n_operands, int iters) {
+  __shared__ calib_half8_t lds[4096];
+  for (int i = threadIdx.x; i < 4096; i += 512) lds[i] = operands[i % n_operands];
+  __syncthreads();
+  calib_half8_t a[8], b[4];
+#pragma unroll
+  for (int i = 0; i < 8; i++) a[i] = operands[(threadIdx.x * 4 + i) % n_operands];
+#pragma unroll
+  for (int i = 0; i < 4; i++) b[i] = operands[(threadIdx.x * 4 + i + n_operands / 2) % n_operands];
+  calib_floatx16_t acc[4];
+#pragma unroll
+  for (int c = 0; c < 4; c++)
+#pragma unroll
+    for (int i = 0; i < 16; i++) acc[c][i] = 0.f;
+  float v[8];
+#pragma unroll
+  for (int i = 0; i < 8; i++) v[i] = (float)a[0][i];
+  int idx = threadIdx.x;
+  for (int it = 0; it < iters; it++) {
+#pragma unroll
+    for (int m = 0; m < 8; m++) {
+      const int frag = LDS_EVERY > 1 ? (m / LDS_EVERY) * LDS_EVERY : m;
+      acc[m & 3] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[frag & 7], b[m & 3], acc[m & 3], 0, 0, 0);
+#pragma unroll
+      for (int j = 0; j < NV; j++) {
+        if (j < NE) v[j & 7] = __builtin_amdgcn_exp2f(v[j & 7] * 0.001f);
+        else v[j & 7] = __builtin_fmaf(v[j & 7], 0.999f, 0.25f);
+      }
+      if (LDS_EVERY > 0 && m % LDS_EVERY == 0) {  // the fragment MFMAs m + 4 .. use
+        a[(m + 4) & 7] = lds[idx & 4095];
+        idx += 517;
+      }
+    }
+  }
+  float s = 0.f;
+#pragma unroll
+  for (int c = 0; c < 4; c++)
+#pragma unroll
+    for (int i = 0; i < 16; i++) s += acc[c][i];
+#pragma unroll
+  for (int i = 0; i < 8; i++) s += v[i];
+  sink[blockIdx.x * 512 + threadIdx.x] = s;
+}
+
 // Read-only stream with non-temporal 16-byte loads, 8 in flight per lane: what the memory system delivers to a
 // kernel that does nothing else (256 workgroups of 256 threads, one slab each).
 typedef unsigned calib_u4_t __attribute__((ext_vector_type(4)));
@@ -115,6 +166,30 @@ extern "C" int lmh_calib_mfma_xcds(void *sink, const void *operands, size_t oper
                      reinterpret_cast<const calib_half8_t *>(operands), (int)(operand_bytes / 16), iters, active_xcds);
   LMH_HIP_TRY(hipGetLastError());
   if (flops_per_workgroup) *flops_per_workgroup = 4.0 * iters * kCalibMfmaPerIter * (2.0 * 32 * 32 * 16);
+  return LMH_OK;
+}
+
+extern "C" int lmh_calib_mix(void *sink, const void *operands, size_t operand_bytes, int iters, int mix, double *flops, void *stream) {
+  using namespace lmh;
+  if (!sink || !operands) return fail(LMH_E_NULL, "lmh_calib_mix: null pointer");
+  if (operand_bytes < 32 || operand_bytes % 16 != 0 || (reinterpret_cast<uintptr_t>(operands) & 15u) || iters < 1)
+    return fail(LMH_E_SHAPE, "lmh_calib_mix: operands must be >= 32 bytes, a multiple of 16, 16-byte aligned; iters >= 1");
+  const dim3 grid(256), block(512);  // one workgroup per CU, two waves per SIMD
+  float *snk = reinterpret_cast<float *>(sink);
+  const calib_half8_t *ops = reinterpret_cast<const calib_half8_t *>(operands);
+  const int n_ops = (int)(operand_bytes / 16);
+  const hipStream_t st = (hipStream_t)stream;
+  switch (mix) {
+    case 0: hipLaunchKernelGGL((calib_mix_kernel<0, 0, 0>), grid, block, 0, st, snk, ops, n_ops, iters); break;
+    case 1: hipLaunchKernelGGL((calib_mix_kernel<6, 1, 0>), grid, block, 0, st, snk, ops, n_ops, iters); break;
+    case 2: hipLaunchKernelGGL((calib_mix_kernel<6, 1, 1>), grid, block, 0, st, snk, ops, n_ops, iters); break;
+    case 3: hipLaunchKernelGGL((calib_mix_kernel<6, 1, 2>), grid, block, 0, st, snk, ops, n_ops, iters); break;
+    case 4: hipLaunchKernelGGL((calib_mix_kernel<4, 1, 1>), grid, block, 0, st, snk, ops, n_ops, iters); break;
+    case 5: hipLaunchKernelGGL((calib_mix_kernel<4, 1, 2>), grid, block, 0, st, snk, ops, n_ops, iters); break;
+    default: return fail(LMH_E_UNSUPPORTED, "lmh_calib_mix: mix %d is not one of 0..5", mix);
+  }
+  LMH_HIP_TRY(hipGetLastError());
+  if (flops) *flops = 256.0 * 8.0 * iters * 8.0 * (2.0 * 32 * 32 * 16);
   return LMH_OK;
 }
 

@@ -689,6 +689,19 @@ def test_calibration_kernels(lm, hip):
     assert np.all(got == 64 * 16 * 6)
     with pytest.raises(lm.LuminalHipError):
         lm.binding.calib_mfma(sink.ptr, ones.ptr, 24, 1)
+    # the instruction-mix streams: with operands of ones and no vector work, each of the 4 accumulators takes
+    # 2 MFMAs per iteration, 16 products per element, and the 8 vector registers stay at 1
+    sink.fill_bytes(0xFF)
+    flops = lm.binding.calib_mix(sink.ptr, ones.ptr, 1 << 13, 3, 0)
+    assert flops == 256 * 8 * 3 * 8 * 2 * 32 * 32 * 16
+    assert np.all(sink.to_host() == 64 * 16 * 2 * 3 + 8)
+    for mix in (2, 5):  # LDS fragments are ones too, so the matrix part is unchanged; the vector part is bounded
+        sink.fill_bytes(0xFF)
+        lm.binding.calib_mix(sink.ptr, ones.ptr, 1 << 13, 3, mix)
+        got = sink.to_host()
+        assert np.all(np.isfinite(got)) and np.all(np.abs(got - 64 * 16 * 2 * 3) < 4096)
+    with pytest.raises(lm.LuminalHipError):
+        lm.binding.calib_mix(sink.ptr, ones.ptr, 1 << 13, 3, 6)
 
 
 def test_compiled_decode_step_graph_serves_every_position(lm, hip, oracle):
