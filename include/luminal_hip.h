@@ -23,7 +23,7 @@
 extern "C" {
 #endif
 
-#define LMH_VERSION 102 /* major*10000 + minor*100 + patch */
+#define LMH_VERSION 103 /* major*10000 + minor*100 + patch */
 
 /* status codes */
 #define LMH_OK 0
@@ -159,6 +159,11 @@ typedef struct lmh_attn_params {
 } lmh_attn_params;
 
 int lmh_flash_attn_fwd(const lmh_attn_params *p);
+
+/* Which kernel lmh_flash_attn_fwd would launch for `p` (instantiation, workgroup count), as text in `plan`; nothing
+ * is launched and no tensor is touched. Same validation and return codes as lmh_flash_attn_fwd. No counterpart in the
+ * reference: a test and bench aid (which shapes reach which kernel). */
+int lmh_flash_attn_plan(const lmh_attn_params *p, char *plan, size_t plan_bytes);
 
 /* ---- single-token decode attention over a KV cache: replaces the un-fused subgraph
  *   whisper_self_attn_cached  reference src/Whisper.jl:584-620 (slice 0:step_pos+1, matmul,

@@ -24,7 +24,7 @@ EXPORTS = [
     "lmh_memset", "lmh_memcpy_h2d", "lmh_memcpy_d2h", "lmh_memcpy_d2d", "lmh_sync", "lmh_event_create",
     "lmh_event_destroy", "lmh_event_record", "lmh_event_elapsed_ms", "lmh_flash_attn_fwd",
     "lmh_decode_workspace_bytes", "lmh_decode_auto_splits", "lmh_decode_attn", "lmh_calib_copy", "lmh_calib_read", "lmh_calib_mfma",
-    "lmh_calib_mfma_xcds", "lmh_calib_mix", "lmh_rope",
+    "lmh_calib_mfma_xcds", "lmh_calib_mix", "lmh_flash_attn_plan", "lmh_rope",
     "lmh_kv_append", "lmh_stream_create", "lmh_stream_destroy", "lmh_graph_capture_begin", "lmh_graph_capture_end",
     "lmh_graph_launch", "lmh_graph_destroy", "lmh_static_scratch_bytes", "lmh_decode_static_splits",
     "lmh_decode_attn_static",
@@ -131,6 +131,8 @@ def load():
     L.lmh_decode_static_splits.argtypes = [ctypes.c_int32] * 5
     L.lmh_calib_copy.argtypes = [vp, vp, ctypes.c_size_t, vp]
     L.lmh_calib_mfma.argtypes = [vp, vp, ctypes.c_size_t, ctypes.c_int, ctypes.POINTER(ctypes.c_double), vp]
+    L.lmh_flash_attn_plan.argtypes = [ctypes.POINTER(AttnParams), ctypes.c_char_p, ctypes.c_size_t]
+    L.lmh_flash_attn_plan.restype = ctypes.c_int
     L.lmh_calib_mix.argtypes = [vp, vp, ctypes.c_size_t, ctypes.c_int, ctypes.c_int, ctypes.POINTER(ctypes.c_double), vp]
     L.lmh_calib_mix.restype = ctypes.c_int
     L.lmh_calib_read.argtypes = [vp, ctypes.c_size_t, vp, vp]
@@ -294,6 +296,13 @@ def calib_mfma(sink, operands, operand_bytes, iters, stream=None):
     flops = ctypes.c_double(0.0)
     check(load().lmh_calib_mfma(sink, operands, operand_bytes, iters, ctypes.byref(flops), stream))
     return flops.value
+
+
+def flash_attn_plan(params):
+    """Text naming the kernel lmh_flash_attn_fwd would launch for `params`; launches nothing."""
+    buf = ctypes.create_string_buffer(256)
+    check(load().lmh_flash_attn_plan(ctypes.byref(params), buf, len(buf)))
+    return buf.value.decode()
 
 
 def calib_mix(sink, operands, operand_bytes, iters, mix, stream=None):

@@ -39,6 +39,18 @@ int fail(int code, const char *fmt, ...) {
   return code;
 }
 
+static thread_local char *g_plan_buf = nullptr;
+static thread_local size_t g_plan_bytes = 0;
+
+bool plan_only(const char *fmt, ...) {
+  if (!g_plan_buf) return false;
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_plan_buf, g_plan_bytes, fmt, ap);
+  va_end(ap);
+  return true;
+}
+
 int hip_fail(hipError_t e, const char *what) {
   return fail(LMH_E_HIP, "HIP error %d (%s) in %s", (int)e, hipGetErrorString(e), what);
 }
@@ -314,6 +326,16 @@ int lmh_flash_attn_fwd(const lmh_attn_params *p) {
   if (mfma_ok && p->dtype == LMH_F32) return launch_prefill_f32_mfma(a, (hipStream_t)p->stream);
   if (mfma_ok) return launch_prefill_mfma(a, p->dtype, (hipStream_t)p->stream);
   return launch_prefill_valu(a, p->dtype, (hipStream_t)p->stream);
+}
+
+int lmh_flash_attn_plan(const lmh_attn_params *p, char *plan, size_t plan_bytes) {
+  if (!plan || plan_bytes < 2) return fail(LMH_E_NULL, "lmh_flash_attn_plan: no room for the description");
+  plan[0] = 0;
+  g_plan_buf = plan;
+  g_plan_bytes = plan_bytes;
+  const int rc = lmh_flash_attn_fwd(p);
+  g_plan_buf = nullptr;
+  return rc;
 }
 
 // --------------------------------------------------------------------------------------------

@@ -16,6 +16,9 @@ int fail(int code, const char *fmt, ...) __attribute__((format(printf, 2, 3)));
 // fails). The launchers size their workgroups by it; any value gives correct results.
 int device_cu_count();
 int hip_fail(hipError_t e, const char *what);
+// While a plan query (lmh_flash_attn_plan) runs on this thread, a launcher that calls this with the description of
+// the kernel it has chosen gets `true` back and must return LMH_OK without launching.
+bool plan_only(const char *fmt, ...) __attribute__((format(printf, 1, 2)));
 
 #define LMH_HIP_TRY(expr)                                \
   do {                                                   \

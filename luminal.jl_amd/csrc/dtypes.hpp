@@ -26,18 +26,21 @@ __device__ inline uint16_t f32_to_bf16_bits(float x) {
 }
 
 struct F32 {
+  static constexpr const char *kName = "f32";
   using raw = float;
   static constexpr int kVec = 4;  // elements per 128-bit access
   __device__ static float ld(raw x) { return x; }
   __device__ static raw st(float x) { return x; }
 };
 struct F16 {
+  static constexpr const char *kName = "f16";
   using raw = _Float16;
   static constexpr int kVec = 8;
   __device__ static float ld(raw x) { return (float)x; }
   __device__ static raw st(float x) { return (_Float16)x; }
 };
 struct BF16 {
+  static constexpr const char *kName = "bf16";
   using raw = uint16_t;
   static constexpr int kVec = 8;
   __device__ static float ld(raw x) { return bf16_bits_to_f32(x); }

@@ -291,6 +291,8 @@ int launch_split(const PrefillArgs &a, hipStream_t stream) {
   const int n_q_tiles = (a.Sq + 128 / KSPLIT - 1) / (128 / KSPLIT);
   const int n_bh_groups = (a.B * a.Hq + 7) / 8;
   dim3 grid(8 * n_bh_groups * n_q_tiles), block(256);
+  if (plan_only("prefill_f32_kernel<D=%d, %s, key groups=%d> workgroups=%u", D, a.causal ? "causal" : "full", KSPLIT, grid.x))
+    return LMH_OK;
   if (a.causal)
     hipLaunchKernelGGL((prefill_f32_kernel<D, true, KSPLIT>), grid, block, 0, stream, a, n_q_tiles, n_bh_groups);
   else

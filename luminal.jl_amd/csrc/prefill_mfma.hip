@@ -48,11 +48,15 @@ constexpr float kLazyRescale = 8.0f;
 // Byte offset no K/V slice reaches (the host routes larger ones elsewhere): a buffer load there
 // is out of range and returns zeros.
 constexpr int kOutOfRange = 0x7ffffff0;
+#ifndef LMH_WIDE_MARGIN
+#define LMH_WIDE_MARGIN 0.9
+#endif
 
 typedef short shortx8_t __attribute__((ext_vector_type(8)));
 typedef __attribute__((address_space(3))) shortx4_t lds_shortx4_t;
 
 struct MfmaF16 {
+  static constexpr const char *kName = "f16";
   using vec8 = half8_t;
   static constexpr bool kSplitP = false;  // 11 significant bits in P are within the 2e-3 budget
   __device__ static floatx16_t mfma(vec8 a, vec8 b, floatx16_t c) {
@@ -72,6 +76,7 @@ struct MfmaF16 {
   }
 };
 struct MfmaBF16 {
+  static constexpr const char *kName = "bf16";
   using vec8 = bf16x8_t;
   // A bf16 P has 8 significant bits; on short or peaked rows that alone is ~2.5e-3 of the output
   // range. P is therefore fed to the matrix cores as head + remainder (two MFMAs per V fragment).
@@ -417,16 +422,316 @@ __global__ __launch_bounds__(64 * NW, WPS) void prefill_mfma_kernel(PrefillArgs 
   }
 }
 
+// One workgroup per CU for non-causal launches with too few query rows to go round: the workgroup owns R
+// consecutive 32-row blocks of one (b, hq) and runs R x KG waves — wave (r, kg) takes row block r against the kg-th
+// 32 keys of every staged tile of 32 KG keys, with its own running max / sum / output; the KG partial results of a
+// row block are folded through LDS at the end. With KG chosen so that R x KG is close to a multiple of four, every
+// SIMD of the CU carries the same share of the workgroup's (rows x keys) area, which equal 64-row workgroups dealt
+// two or three to a CU do not achieve, and every K/V tile is staged once for all R row blocks.
+// Measured against those workgroups (B=4 H=20 Sq=448 D=64 fp16, five row blocks x three key groups): 1500 keys 28.7 ->
+// 25.3 us, 3000 keys 51.4 -> 43.7, 750 keys 17.0 -> 16.4, 256 keys 9.2 -> 10.5 (one prologue per CU instead of three
+// that overlap). Taller tiles (two blocks per wave and tile) and a third tile buffer were 1 % and 7 % slower.
+constexpr int kWideMaxKeyGroups = 6;  // tiles of up to 192 keys: two buffers of them fit the LDS at D = 96
+template <typename MT, int D>
+__global__ __launch_bounds__(1024, 4) void prefill_mfma_wide_kernel(PrefillArgs a, int wgs_per_head, int n_bh_groups) {
+  using vec8 = typename MT::vec8;
+  constexpr int KS = D / 16, DB = D / 32;
+  constexpr int LDK = D + kPadK, LDV = D + pad_v<D>();
+  constexpr int KG_MAX = kWideMaxKeyGroups, BT_MAX = 32 * KG_MAX;  // keys per staged tile at most
+  constexpr int NBUF = 2;  // tile kt + 1 is in flight while tile kt is computed
+  constexpr int KC = LDK / 8, VC = LDV / 8;         // 16-byte chunks per LDS row
+  constexpr int NW_MIN = 12;                        // the host launches 12 to 16 waves
+  constexpr int KJ = (KC * BT_MAX / 64 + NW_MIN - 1) / NW_MIN, VJ = (VC * BT_MAX / 64 + NW_MIN - 1) / NW_MIN;
+  constexpr int NF = DB * 16 + 2;                   // floats per lane of a partial result
+  constexpr int K_BUF = BT_MAX * LDK, V_BUF = BT_MAX * LDV;  // elements per tile buffer
+  constexpr int kWideMaxSlots = 12;  // (KG - 1) x R partial results at most; the host picks KG accordingly
+  constexpr int kTileElems = NBUF * (K_BUF + V_BUF), kMergeElems = kWideMaxSlots * NF * 64 * 2;
+  __shared__ __attribute__((aligned(16))) uint16_t lds[kTileElems > kMergeElems ? kTileElems : kMergeElems];  // tiles, then partials
+  static_assert(sizeof(lds) <= 160 * 1024, "LDS of a CU");
+
+  const int cpr = a.D / 8;
+  const int bid = blockIdx.x;
+  const int xcd = bid & 7, idx = bid >> 3;
+  const int j_wg = idx % wgs_per_head;
+  const int bh = (idx / wgs_per_head) * 8 + xcd;
+  if (bh >= a.B * a.Hq) return;
+  const int b = bh / a.Hq, hq = bh % a.Hq;
+  const int kvh = kv_head_of(hq, a.Hq, a.Hkv, a.head_map);
+  // row blocks of this workgroup: the head's ceil(Sq / 32) blocks dealt evenly to its workgroups
+  const int n_blocks = (a.Sq + 31) / 32;
+  const int base = n_blocks / wgs_per_head, extra = n_blocks % wgs_per_head;
+  const int R = base + (j_wg < extra ? 1 : 0);
+  if (R == 0) return;
+  const int block0 = j_wg * base + min(j_wg, extra);
+  const int NW = blockDim.x >> 6;
+  // the host launches R_max x KG waves; a workgroup with fewer row blocks may use more key groups or leave waves idle
+  const int KG = min(min(NW / R, KG_MAX), kWideMaxSlots / R + 1);
+  const int BT = 32 * KG;
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63, wave = tid >> 6;
+  const int n = lane & 31, g = lane >> 5;
+  const int r = wave % R, kg = wave / R;
+  const bool active = kg < KG;  // waves beyond R x KG only help to stage
+  const int qi = (block0 + r) * 32 + n;
+
+  int n_keys = a.kv_len ? a.kv_len[b] : a.Sk;
+  n_keys = min(max(n_keys, 0), a.Sk);
+  const int n_kv_tiles = (n_keys + BT - 1) / BT;
+
+  const uint16_t *qp = reinterpret_cast<const uint16_t *>(a.q) + b * a.qs[0] + hq * a.qs[1];
+  const uint16_t *kp = reinterpret_cast<const uint16_t *>(a.k) + b * a.ks[0] + kvh * a.ks[1];
+  const uint16_t *vp = reinterpret_cast<const uint16_t *>(a.v) + b * a.vs[0] + kvh * a.vs[1];
+
+  vec8 qreg[KS];
+#pragma unroll
+  for (int ks = 0; ks < KS; ks++) {
+    uint4 raw = make_uint4(0, 0, 0, 0);
+    if (active && qi < a.Sq && 16 * ks + 8 * g < a.D) raw = *reinterpret_cast<const uint4 *>(qp + (int64_t)qi * a.qs[2] + 16 * ks + 8 * g);
+    qreg[ks] = __builtin_bit_cast(vec8, raw);
+  }
+  floatx16_t oacc[DB];
+#pragma unroll
+  for (int db = 0; db < DB; db++)
+#pragma unroll
+    for (int i = 0; i < 16; i++) oacc[db][i] = 0.f;
+  float m_i = -INFINITY, l_i = 0.f;
+  const float c = a.scale * kLog2e;
+
+  // ---- staging, as in the kernel above: LDS-writing buffer loads, one tile ahead, wave w issues 1 KB blocks
+  // w, w + NW, ...; the chunk -> (row, column) map does not depend on the tile height, rows past it are not fetched ----
+  typedef int32_t i32x4_t __attribute__((ext_vector_type(4)));
+  typedef __attribute__((address_space(3))) void lds_void_t;
+  const int KI = (KC * BT + 63) / 64, VI = (VC * BT + 63) / 64;
+  const int wave_u = __builtin_amdgcn_readfirstlane(wave);
+  const int nw_u = __builtin_amdgcn_readfirstlane(NW);
+  auto make_desc = [](const uint16_t *base_ptr, int bytes) {
+    const uint64_t pp = (uint64_t)base_ptr;
+    i32x4_t d;
+    d[0] = __builtin_amdgcn_readfirstlane((int)(uint32_t)pp);
+    d[1] = __builtin_amdgcn_readfirstlane((int)((pp >> 32) & 0xffff));
+    d[2] = __builtin_amdgcn_readfirstlane(bytes);
+    d[3] = 0x00020000;
+    return d;
+  };
+  const i32x4_t k_desc = make_desc(kp, (int)((int64_t)n_keys * a.ks[2] * 2));
+  const i32x4_t v_desc = make_desc(vp, (int)((int64_t)n_keys * a.vs[2] * 2));
+  int k_voff[KJ], v_voff[VJ];
+#pragma unroll
+  for (int j = 0; j < KJ; j++) {
+    const int ch = (wave + NW * j) * 64 + lane;
+    const int row = ch / KC, col = ch % KC;
+    k_voff[j] = (col < cpr && row < BT) ? (int)((row * a.ks[2] + col * 8) * 2) : kOutOfRange;
+  }
+#pragma unroll
+  for (int j = 0; j < VJ; j++) {
+    const int ch = (wave + NW * j) * 64 + lane;
+    const int row = ch / VC, col = ch % VC;
+    v_voff[j] = (col < cpr && row < BT) ? (int)((row * a.vs[2] + col * 8) * 2) : kOutOfRange;
+  }
+  const int k_tile_bytes = (int)(BT * a.ks[2] * 2), v_tile_bytes = (int)(BT * a.vs[2] * 2);
+  const uint32_t k_lds0 = (uint32_t)(uintptr_t)(lds_void_t *)&lds[0] + wave_u * 1024;
+  const uint32_t v_lds0 = (uint32_t)(uintptr_t)(lds_void_t *)&lds[NBUF * K_BUF] + wave_u * 1024;
+#pragma clang diagnostic push
+#pragma clang diagnostic ignored "-Winline-asm"  // m0 is a reserved register; it is only written here
+  auto load_block = [](i32x4_t desc, uint32_t lds_addr, int voff, int soff) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
+                 :: "s"(lds_addr), "v"(voff), "s"(desc), "s"(soff) : "memory", "m0");
+  };
+#pragma clang diagnostic pop
+  auto load_tile = [&](int kt, int buf) {
+#pragma unroll
+    for (int j = 0; j < KJ; j++)
+      if (wave_u + nw_u * j < KI)
+        load_block(k_desc, k_lds0 + buf * (K_BUF * 2) + j * (nw_u * 1024), k_voff[j], kt * k_tile_bytes);
+#pragma unroll
+    for (int j = 0; j < VJ; j++)
+      if (wave_u + nw_u * j < VI)
+        load_block(v_desc, v_lds0 + buf * (V_BUF * 2) + j * (nw_u * 1024), v_voff[j], kt * v_tile_bytes);
+  };
+
+  const int k_frag_off = (kg * 32 + n) * LDK + 8 * g;
+  const int i16 = lane & 15;
+  const int v_frag_off = (kg * 32 + 4 * g + (i16 >> 2)) * LDV + 16 * ((lane >> 4) & 1) + 4 * (i16 & 3);
+
+  if (n_kv_tiles > 0) load_tile(0, 0);
+#pragma unroll
+  for (int ks = 0; ks < KS; ks++) asm volatile("" :: "v"(qreg[ks]));
+
+  for (int kt = 0; kt < n_kv_tiles; kt++) {
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wave's blocks of tile kt are in LDS
+    __syncthreads();  // ... and everyone's; tile kt-1 has been consumed, its buffer is free
+    if (kt + 1 < n_kv_tiles) load_tile(kt + 1, (kt + 1) & 1);
+    const int k0 = kt * BT + kg * 32;  // this wave's 32 keys of the tile
+    if (!active || k0 >= n_keys) continue;
+    const uint16_t *Ks = &lds[(kt & 1) * K_BUF];
+    const uint16_t *Vs = &lds[NBUF * K_BUF + (kt & 1) * V_BUF];
+
+    floatx16_t sacc;
+#pragma unroll
+    for (int i = 0; i < 16; i++) sacc[i] = 0.f;
+    vec8 kf[KS];
+#pragma unroll
+    for (int ks = 0; ks < KS; ks++) kf[ks] = *reinterpret_cast<const vec8 *>(&Ks[k_frag_off + 16 * ks]);
+#pragma unroll
+    for (int ks = 0; ks < KS; ks++) sacc = MT::mfma(kf[ks], qreg[ks], sacc);
+    if (k0 + 32 > n_keys) {
+#pragma unroll
+      for (int i = 0; i < 16; i++)
+        if (k0 + 8 * (i >> 2) + 4 * g + (i & 3) >= n_keys) sacc[i] = -INFINITY;
+    }
+    float mx = sacc[0];
+#pragma unroll
+    for (int i = 1; i < 16; i++) mx = fmaxf(mx, sacc[i]);
+    mx = fmaxf(mx, __shfl_xor(mx, 32));
+    if (__builtin_amdgcn_ballot_w64((mx - m_i) * c > kLazyRescale) != 0) {
+      const float m_new = fmaxf(m_i, mx);
+      const float alpha = __builtin_amdgcn_exp2f((m_i - m_new) * c);
+      m_i = m_new;
+      l_i *= alpha;
+#pragma unroll
+      for (int db = 0; db < DB; db++)
+#pragma unroll
+        for (int i = 0; i < 16; i++) oacc[db][i] *= alpha;
+    }
+    const float mc = m_i * c;
+    vec8 pf[2], pf_lo[2];
+#pragma unroll
+    for (int t = 0; t < 2; t++) {
+#pragma unroll
+      for (int e = 0; e < 8; e++) {
+        const float p = __builtin_amdgcn_exp2f(sacc[8 * t + e] * c - mc);
+        pf[t][e] = MT::cvt(p);
+        if (MT::kSplitP) pf_lo[t][e] = MT::cvt(p - (float)pf[t][e]);
+      }
+      l_i = MT::sum8(pf[t], l_i);
+      if (MT::kSplitP) l_i = MT::sum8(pf_lo[t], l_i);
+    }
+#pragma unroll
+    for (int t = 0; t < 2; t++) {
+#pragma unroll
+      for (int db = 0; db < DB; db++) {
+        const uint16_t *vaddr = &Vs[v_frag_off + 16 * t * LDV + db * 32];
+        const shortx4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_shortx4_t *)(vaddr));
+        const shortx4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_shortx4_t *)(vaddr + 8 * LDV));
+        const shortx8_t v8 = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+        oacc[db] = MT::mfma(__builtin_bit_cast(vec8, v8), pf[t], oacc[db]);
+        if (MT::kSplitP) oacc[db] = MT::mfma(__builtin_bit_cast(vec8, v8), pf_lo[t], oacc[db]);
+      }
+    }
+  }
+
+  // ---- fold the key groups of a row block: groups 1 .. KG-1 leave (m, l, O) in LDS, group 0 takes them in order ----
+  float *xch = reinterpret_cast<float *>(&lds[0]) + lane;  // slot s at xch + s * NF * 64, [NF][64 lanes]
+  __syncthreads();  // every wave has read its last tile
+  if (active && kg > 0) {
+    float *slot = xch + ((kg - 1) * R + r) * (NF * 64);
+    slot[0] = m_i;
+    slot[64] = l_i;
+#pragma unroll
+    for (int db = 0; db < DB; db++)
+#pragma unroll
+      for (int i = 0; i < 16; i++) slot[(2 + db * 16 + i) * 64] = oacc[db][i];
+  }
+  __syncthreads();
+  if (!active || kg > 0) return;
+  for (int k2 = 1; k2 < KG; k2++) {
+    const float *slot = xch + ((k2 - 1) * R + r) * (NF * 64);
+    const float m1 = slot[0], l1 = slot[64];
+    const float m_new = fmaxf(m_i, m1);
+    // a group that saw no key has m = -inf, l = 0, O = 0
+    const float a0 = m_i == -INFINITY ? 0.f : __builtin_amdgcn_exp2f((m_i - m_new) * c);
+    const float a1 = m1 == -INFINITY ? 0.f : __builtin_amdgcn_exp2f((m1 - m_new) * c);
+    m_i = m_new;
+    l_i = l_i * a0 + l1 * a1;
+#pragma unroll
+    for (int db = 0; db < DB; db++)
+#pragma unroll
+      for (int i = 0; i < 16; i++) oacc[db][i] = oacc[db][i] * a0 + slot[(2 + db * 16 + i) * 64] * a1;
+  }
+
+  const float l_tot = l_i + __shfl_xor(l_i, 32);
+  const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
+  if (qi < a.Sq) {
+    const int64_t off = b * a.os[0] + hq * a.os[1] + (int64_t)qi * a.os[2];
+    uint16_t *op = reinterpret_cast<uint16_t *>(a.out) + off;
+    float *op32 = reinterpret_cast<float *>(a.out) + off;
+#pragma unroll
+    for (int db = 0; db < DB; db++)
+#pragma unroll
+      for (int i4 = 0; i4 < 4; i4++) {
+        const int d = db * 32 + 8 * i4 + 4 * g;
+        if (d >= a.D) continue;
+        if (a.out_f32) {
+          *reinterpret_cast<float4 *>(op32 + d) =
+              make_float4(oacc[db][4 * i4 + 0] * inv, oacc[db][4 * i4 + 1] * inv, oacc[db][4 * i4 + 2] * inv,
+                          oacc[db][4 * i4 + 3] * inv);
+          continue;
+        }
+        uint2 packed;
+        packed.x = (uint32_t)MT::cvt_bits(oacc[db][4 * i4 + 0] * inv) |
+                   ((uint32_t)MT::cvt_bits(oacc[db][4 * i4 + 1] * inv) << 16);
+        packed.y = (uint32_t)MT::cvt_bits(oacc[db][4 * i4 + 2] * inv) |
+                   ((uint32_t)MT::cvt_bits(oacc[db][4 * i4 + 3] * inv) << 16);
+        *reinterpret_cast<uint2 *>(op + d) = packed;
+      }
+  }
+}
+
 template <typename MT, int D, int KSPLIT, int NW, int WPS = default_wps<D, NW>()>
 int launch_split(const PrefillArgs &a, hipStream_t stream) {
   constexpr int BM = 32 * NW / KSPLIT;
   const int n_q_tiles = (a.Sq + BM - 1) / BM;
   const int n_bh_groups = (a.B * a.Hq + 7) / 8;
   dim3 grid(8 * n_bh_groups * n_q_tiles), block(64 * NW);
+  if (plan_only("prefill_mfma_kernel<%s, D=%d, %s, key groups=%d, waves=%d, waves per SIMD=%d> workgroups=%u", MT::kName, D,
+                a.causal ? "causal" : "full", KSPLIT, NW, WPS, grid.x))
+    return LMH_OK;
   if (a.causal)
     hipLaunchKernelGGL((prefill_mfma_kernel<MT, D, true, KSPLIT, NW, WPS>), grid, block, 0, stream, a, n_q_tiles, n_bh_groups);
   else
     hipLaunchKernelGGL((prefill_mfma_kernel<MT, D, false, KSPLIT, NW, WPS>), grid, block, 0, stream, a, n_q_tiles, n_bh_groups);
+  LMH_HIP_TRY(hipGetLastError());
+  return LMH_OK;
+}
+
+// Plan for the wide kernel: workgroups per head, waves per workgroup. Returns false where it does not apply or the
+// equal 64-row workgroups are expected to do as well. `load` = the share of a 32-row block's keys that the busiest SIMD
+// of the busiest CU walks, the quantity the launch time follows when the chip is not full. Measured (fp16, 1500 keys,
+// wide against 64-row workgroups): load 1.33 vs 1.5 -12 % (D = 64), -14 % (D = 96); 0.75 vs 1.0 -7 ... -12 %; equal loads
+// +-2 %, and +7 % at 1024 keys; under about 500 keys the single prologue per CU costs more than the balance wins.
+inline bool wide_plan(const PrefillArgs &a, int n_cus, int *wgs_per_head, int *n_waves) {
+  const int heads = a.B * a.Hq, heads8 = (heads + 7) / 8 * 8;
+  const int n_blocks = (a.Sq + 31) / 32;
+  if (a.causal || heads8 > n_cus || n_blocks < 2 || a.Sk < 640) return false;
+  const int w = max(1, min(n_cus / heads8, n_blocks / 2));
+  const int r_max = (n_blocks + w - 1) / w;
+  if (r_max > 8) return false;
+  int best_kg = 0;
+  double best = 1e30;
+  for (int kg = 2; kg <= kWideMaxKeyGroups; kg++) {
+    if (r_max * kg < 12 || r_max * kg > 16 || (kg - 1) * r_max > 12) continue;  // 12 to 16 waves, 12 partial results
+    const double load = (double)((r_max * kg + 3) / 4) / kg;
+    if (load <= best) best = load, best_kg = kg;  // on a tie, more waves
+  }
+  if (!best_kg) return false;
+  // the equal 64-row workgroups, wave pairs splitting the keys: up to three resident on a CU, half a block's keys a wave
+  const int64_t n64 = (int64_t)heads8 * ((a.Sq + 63) / 64);
+  const double load_now = 0.5 * (double)((n64 + n_cus - 1) / n_cus);
+  if (best > LMH_WIDE_MARGIN * load_now) return false;
+  *wgs_per_head = w;
+  *n_waves = r_max * best_kg;
+  return true;
+}
+
+template <typename MT, int D>
+int launch_wide(const PrefillArgs &a, int wgs_per_head, int n_waves, hipStream_t stream) {
+  const int n_bh_groups = (a.B * a.Hq + 7) / 8;
+  dim3 grid(8 * n_bh_groups * wgs_per_head), block(64 * n_waves);
+  if (plan_only("prefill_mfma_wide_kernel<%s, D=%d> workgroups per head=%d, waves=%d, workgroups=%u", MT::kName, D, wgs_per_head,
+                n_waves, grid.x))
+    return LMH_OK;
+  hipLaunchKernelGGL((prefill_mfma_wide_kernel<MT, D>), grid, block, 0, stream, a, wgs_per_head, n_bh_groups);
   LMH_HIP_TRY(hipGetLastError());
   return LMH_OK;
 }
@@ -441,7 +746,13 @@ int launch_for_d(const PrefillArgs &a, hipStream_t stream) {
   const int n_cus = device_cu_count();
   const int64_t wgs = (int64_t)((a.B * a.Hq + 7) / 8) * 8 * ((a.Sq + 127) / 128);
   const int64_t limit = a.causal ? 2 * n_cus : 2 * n_cus - 1;
-  if (wgs <= limit && a.Sk >= 4 * BN) return launch_split<MT, D, 2, 4>(a, stream);
+  if (wgs <= limit && a.Sk >= 4 * BN) {
+    if constexpr (D <= 96) {
+      int wgs_per_head, n_waves;
+      if (wide_plan(a, n_cus, &wgs_per_head, &n_waves)) return launch_wide<MT, D>(a, wgs_per_head, n_waves, stream);
+    }
+    return launch_split<MT, D, 2, 4>(a, stream);
+  }
   // Large launches: 256-row workgroups of eight waves. Measured against the 128-row ones at D = 96, fp16:
   // non-causal 512 / 768 / 1024 / 1536 / 2048 workgroups +3 / +2 / +2 / +6 / +5 %, causal 512 -7 %
   // (too few to balance their unequal lengths), 1024 +3 %, 1536 +4..7 %, 2048 +5 %.

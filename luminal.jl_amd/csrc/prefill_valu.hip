@@ -139,6 +139,10 @@ __global__ __launch_bounds__(256) void prefill_valu_kernel(PrefillArgs a) {
 template <typename E>
 int launch_for_dtype(const PrefillArgs &a, hipStream_t stream) {
   dim3 grid((a.Sq + kRowsPerWg - 1) / kRowsPerWg, a.Hq, a.B), block(256);
+  if (a.D <= 256 && plan_only("prefill_valu_kernel<%s, head dim %d padded to %d> workgroups=%u", E::kName, a.D,
+                              a.D <= 16 ? 16 : a.D <= 32 ? 32 : a.D <= 64 ? 64 : a.D <= 96 ? 96 : a.D <= 128 ? 128 : a.D <= 192 ? 192 : 256,
+                              grid.x * grid.y * grid.z))
+    return LMH_OK;
   if (a.D <= 16) hipLaunchKernelGGL((prefill_valu_kernel<E, 16>), grid, block, 0, stream, a);
   else if (a.D <= 32) hipLaunchKernelGGL((prefill_valu_kernel<E, 32>), grid, block, 0, stream, a);
   else if (a.D <= 64) hipLaunchKernelGGL((prefill_valu_kernel<E, 64>), grid, block, 0, stream, a);

@@ -406,6 +406,20 @@ class _Workspaces:
 _workspaces = _Workspaces()
 
 
+def flash_attention_plan(q_shape, kv_shape, dtype, causal=False, scale=None, out_dtype=None):
+    """Name of the kernel (instantiation and workgroup count) a flash-attention launch of these shapes would run,
+    for contiguous 16-byte aligned tensors. Launches nothing and needs no GPU."""
+    p = binding.AttnParams()
+    p.out = p.q = p.k = p.v = 4096  # never dereferenced: the plan query stops in front of the launch
+    p.B, p.Hq, p.Sq, p.D = q_shape
+    p.Hkv, p.Sk = kv_shape[1], kv_shape[2]
+    p.dtype = binding.DTYPE_CODES[dtype]
+    p.scale = default_scale(q_shape[-1]) if scale is None else scale
+    p.causal = int(causal)
+    p.out_f32 = int((out_dtype or dtype) == "f32")
+    return binding.flash_attn_plan(p)
+
+
 def execute_op_inplace(out, op, *inputs, stream=None, workspaces=None):
     """execute_op!(out, op, inputs...) (reference src/Execution.jl:565-578) for the attention ops. `workspaces`
     is where decode attention takes its split-KV scratch from (default: one buffer shared by all eager calls)."""
@@ -736,4 +750,5 @@ __all__ = [
     "RotaryEmbeddingOp", "KVAppendOp", "rotary_embedding", "kv_cache_append", "self_attention_core",
     "cached_self_attention_core", "execute_op", "execute_op_inplace", "execute", "compile", "CompiledGraph", "execute_with_capture", "release_capture", "HEADMAP_INTERLEAVED",
     "HEADMAP_BLOCKED", "LuminalHipError", "apply_rotary_embeddings", "kv_append", "KVCacheState", "encode", "decode", "f32_to_bf16_bits", "bf16_bits_to_f32", "default_scale",
+    "flash_attention_plan",
 ]

@@ -23,7 +23,7 @@ def test_library_exports_every_declared_symbol(lm):
     lib = lm.binding.load()
     for name in header_functions():
         assert hasattr(lib, name), name
-    assert lib.lmh_version() == 102
+    assert lib.lmh_version() == 103
 
 
 def test_struct_layout_matches_header(lm):

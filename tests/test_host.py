@@ -136,3 +136,27 @@ def test_package_input_generator_is_the_oracles_generator(lm, oracle):
     big = lm.synth.normal((1 << 16,), 7, chunk_pairs=1000)  # chunking does not change the stream
     np.testing.assert_array_equal(big, lm.synth.normal((1 << 16,), 7))
     assert abs(float(big.mean())) < 0.02 and abs(float(big.std()) - 1.0) < 0.02
+
+
+def test_kernel_plan_of_the_benchmark_configurations(lm):
+    """Which kernel a launch reaches is decided on the host from shapes alone (the plan query launches nothing and
+    needs no GPU; without one the launchers assume 256 compute units)."""
+    plan = lm.flash_attention_plan
+    # C1: the reference's own fp32 example, far too small to fill the chip -> fp32 matrix cores, keys split four ways
+    assert plan((1, 8, 128, 64), (1, 8, 128, 64), "f32", True).startswith("prefill_f32_kernel<D=64, causal, key groups=4>")
+    # C2: 512 workgroups of 256 rows, one per CU at a time, 128-key tiles
+    assert plan((1, 32, 4096, 96), (1, 32, 4096, 96), "f16", True).startswith(
+        "prefill_mfma_kernel<f16, D=96, causal, key groups=1, waves=8, waves per SIMD=2> workgroups=512")
+    # C3: 80 heads x 14 row blocks on 256 CUs -> three workgroups per head of five row blocks x three key groups
+    assert plan((4, 20, 448, 64), (4, 20, 1500, 64), "f16", False) == \
+        "prefill_mfma_wide_kernel<f16, D=64> workgroups per head=3, waves=15, workgroups=240"
+    # the same heads against few keys, or causal: 64-row workgroups whose wave pairs split the keys
+    assert "key groups=2, waves=4" in plan((4, 20, 448, 64), (4, 20, 512, 64), "f16", False)
+    assert "key groups=2, waves=4" in plan((4, 20, 448, 64), (4, 20, 1500, 64), "f16", True)
+    # 64 heads: two 64-row workgroups per CU already balance
+    assert "prefill_mfma_kernel<f16, D=64, full, key groups=2" in plan((4, 16, 448, 64), (4, 16, 1500, 64), "f16", False)
+    # head dims the matrix-core kernels do not tile, unaligned scale
+    assert plan((2, 4, 100, 136), (2, 4, 100, 136), "bf16", False).startswith("prefill_valu_kernel<bf16, head dim 136 padded to 192>")
+    assert plan((2, 4, 100, 64), (2, 4, 100, 64), "f16", False, scale=-1.0).startswith("prefill_valu_kernel<f16")
+    with pytest.raises(lm.LuminalHipError):
+        plan((2, 4, 100, 264), (2, 4, 100, 264), "f16", False)

@@ -276,6 +276,62 @@ def test_prefill_small_launch_splits_keys_between_wave_pairs(lm, hip, oracle, dt
     assert rel_err(got[keep], want[keep]) <= TOL[dtype]
 
 
+WIDE_CASES = [
+    # dtype, B, Hq, Hkv, Sq, Sk, D, head_map, kv_len (None = all keys), what the case is there for
+    ("bf16", 2, 20, 10, 430, 777, 64, 0, None),             # 6 workgroups per head: 3, 3, 2, 2, 2, 2 row blocks, the last one ragged
+    ("f16", 16, 8, 8, 190, 1000, 96, 0, [1000, 0, 1, 31, 32, 33, 95, 96, 97, 640, 999, 128, 129, 500, 767, 768]),
+    ("bf16", 1, 256, 256, 96, 700, 80, 0, None),             # one workgroup per head, head dim padded to 96
+    ("f16", 4, 20, 20, 448, 1500, 64, 0, [1500, 1499, 97, 0]),  # 5 row blocks x 3 key groups = 15 waves, one SIMD a wave short
+    ("f16", 2, 24, 6, 448, 900, 64, 1, [900, 650]),          # blocked GQA map; 3, 3, 3, 3, 2 row blocks
+    ("bf16", 4, 20, 4, 448, 1500, 96, 0, None),
+    ("f16", 2, 32, 32, 576, 1200, 64, 0, None),              # 5, 5, 4, 4 row blocks on 15 waves: three waves idle where there are 4
+]
+
+
+@pytest.mark.parametrize("dtype,B,Hq,Hkv,Sq,Sk,D,head_map,lens", WIDE_CASES)
+def test_prefill_one_wide_workgroup_per_cu(lm, hip, oracle, dtype, B, Hq, Hkv, Sq, Sk, D, head_map, lens):
+    """Non-causal launches with fewer 64-row workgroups than fill the chip evenly: one workgroup per CU of up to 8 row
+    blocks x up to 6 key groups, partial results folded through LDS. Ragged kv_len with a poisoned tail (lengths on
+    and around block and tile edges, 0 and 1), GQA under both head maps, query counts that end inside a block."""
+    assert "prefill_mfma_wide_kernel" in lm.flash_attention_plan((B, Hq, Sq, D), (B, Hkv, Sk, D), dtype, False)
+    q, k, v = inputs(oracle, (B, Hq, Sq, D), (B, Hkv, Sk, D), dtype, 7480 + D + B, 0.8)
+    kp, vp = k.copy(), v.copy()
+    if lens is not None:
+        lens = np.array(lens, np.int32)
+        for b, n in enumerate(lens):
+            kp[b, :, n:] = np.nan
+            vp[b, :, n:] = np.nan
+    got = run_flash(lm, hip, q, kp, vp, dtype, False, head_map=head_map, kv_len=lens, out_dtype="f32")
+    hq = np.arange(0, Hq, max(1, Hq // 8))  # a spread of heads keeps the CPU oracle at a few seconds
+    if Hq == Hkv:
+        kv_of = hq
+    else:
+        kv_of = hq // (Hq // Hkv) if head_map == 1 else hq % Hkv
+    want_len = None if lens is None else np.maximum(lens, 1)
+    want = oracle.flash_attn(q[:, hq], k[:, kv_of], v[:, kv_of], causal=False, kv_len=want_len, nthreads=NT)
+    keep = np.arange(B) if lens is None else np.nonzero(lens > 0)[0]
+    assert np.isfinite(got).all()
+    assert rel_err(got[keep][:, hq], want[keep]) <= TOL[dtype]
+    if lens is not None:
+        for b in np.nonzero(lens == 0)[0]:
+            assert np.all(got[b] == 0)
+
+
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
+def test_prefill_wide_workgroups_large_logits_and_late_maximum(lm, hip, oracle, dtype):
+    # the key groups of a row block hold different running maxima (scale 1, one key x 6 in the last tile, one x 3 in the
+    # middle) when they are folded
+    B, H, Sq, Sk, D = 1, 40, 448, 700, 64
+    assert "prefill_mfma_wide_kernel" in lm.flash_attention_plan((B, H, Sq, D), (B, H, Sk, D), dtype, False)
+    q, k, v = inputs(oracle, (B, H, Sq, D), (B, H, Sk, D), dtype, 7495)
+    k[:, :, -1] = oracle.round_to(k[:, :, -1] * 6.0, dtype)
+    k[:, :, Sk // 2] = oracle.round_to(k[:, :, Sk // 2] * 3.0, dtype)
+    got = run_flash(lm, hip, q, k, v, dtype, False, scale=1.0)
+    hs = np.arange(0, H, 5)
+    want = oracle.flash_attn(q[:, hs], k[:, hs], v[:, hs], scale=1.0, causal=False, nthreads=NT)
+    assert rel_err(got[:, hs], want) <= TOL[dtype]
+
+
 @pytest.mark.parametrize("causal", [False, True])
 def test_prefill_small_and_large_launches_agree(lm, hip, oracle, causal):
     # the same two heads alone (key-split workgroups) and as part of a launch that fills the chip (128-row workgroups)
