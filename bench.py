@@ -166,7 +166,7 @@ def prefill_leg(lm, dev, steps, warmup, cpu_seconds):
         "ms_per_step": wall_ms, "value": tflops,
         "roofline": {"bound": "mfma", "achieved": kern_tflops, "peak": PEAK_FP16_TFLOPS, "unit": "TFLOP/s",
                      "frac": kern_tflops / PEAK_FP16_TFLOPS, "traffic": measured_traffic("prefill_C2"),
-                     "kernel": "prefill_mfma_kernel<MfmaF16, 96, causal>", "launch_us": ev_ms * 1e3,
+                     "kernel": lm.binding.flash_attn_plan(p), "launch_us": ev_ms * 1e3,
                      "algorithmic_flops_per_launch": flops, "launch_us_one_by_one": each,
                      # what a bare MFMA loop sustains on this GPU right now (clock management under load):
                      # on all-zero operands and on the Q tensor of this workload
@@ -310,7 +310,7 @@ def flash_config(lm, dev, res, name, B, Hq, Hkv, Sq, Sk, D, dtype, causal, flops
     fn = lambda: lm.binding.flash_attn_fwd(p)
     _, ev = time_steps(fn, steps, 5, lm.binding)
     res[name] = {"launch_us": ev * 1e3, "TFLOP/s": flops / (ev * 1e-3) / 1e12,
-                 "launch_us_one_by_one": per_launch_us(fn, 20, lm.binding)}
+                 "launch_us_one_by_one": per_launch_us(fn, 20, lm.binding), "kernel": lm.binding.flash_attn_plan(p)}
     if peak:
         res[name]["frac_of_mfma_peak"] = res[name]["TFLOP/s"] / peak
     log("[other] %s: %.1f us, %.2f TFLOP/s" % (name, ev * 1e3, res[name]["TFLOP/s"]))
