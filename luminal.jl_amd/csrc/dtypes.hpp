@@ -15,6 +15,25 @@ typedef float floatx16_t __attribute__((ext_vector_type(16)));
 typedef float floatx4_t __attribute__((ext_vector_type(4)));
 typedef short shortx4_t __attribute__((ext_vector_type(4)));
 
+// Reductions over lane l and lane l ^ 32 (the two halves of a wave) with v_permlane32_swap_b32: one vector instruction
+// exchanges the upper half of one register with the lower half of another, where __shfl_xor(x, 32) is a round trip
+// through the LDS crossbar (ds_bpermute_b32) plus its index arithmetic. Written as asm: given the same value for both
+// operands the builtin's two results are treated as one. The s_nop covers the instruction's wait after a vector write
+// of its operands.
+__device__ inline void swap_wave_halves(float &a, float &b) {
+  asm volatile("s_nop 1\n\tv_permlane32_swap_b32_e32 %0, %1" : "+v"(a), "+v"(b));
+}
+__device__ inline float max_over_wave_halves(float x) {
+  float a = x, b = x;
+  swap_wave_halves(a, b);  // a = the lower half's x on all lanes, b = the upper half's
+  return fmaxf(a, b);
+}
+__device__ inline float sum_over_wave_halves(float x) {
+  float a = x, b = x;
+  swap_wave_halves(a, b);
+  return a + b;  // lower + upper on every lane: both halves get the same bits
+}
+
 __device__ inline float bf16_bits_to_f32(uint32_t bits16) { return __uint_as_float(bits16 << 16); }
 
 // round-to-nearest-even, NaN kept quiet

@@ -203,7 +203,7 @@ __global__ __launch_bounds__(256, (KSPLIT > 1 ? 1 : D <= 96 ? 3 : 2)) void prefi
     float mx = sacc[0];
 #pragma unroll
     for (int i = 1; i < 16; i++) mx = fmaxf(mx, sacc[i]);
-    mx = fmaxf(mx, __shfl_xor(mx, 32));
+    mx = max_over_wave_halves(mx);
     // m_i is finite after the first tile (key 0 is visible to every query); -inf before it.
     if (__builtin_amdgcn_ballot_w64((mx - m_i) * c > kLazyRescale) != 0) {  // wave-uniform
       const float m_new = fmaxf(m_i, mx);
@@ -270,7 +270,7 @@ __global__ __launch_bounds__(256, (KSPLIT > 1 ? 1 : D <= 96 ? 3 : 2)) void prefi
   }
 
   // ---- epilogue: out[qi][d] = O^T[d][qi] / l ----
-  const float l_tot = l_i + __shfl_xor(l_i, 32);
+  const float l_tot = sum_over_wave_halves(l_i);
   const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
   if (qi < a.Sq) {
     float *op = reinterpret_cast<float *>(a.out) + b * a.os[0] + hq * a.os[1] + (int64_t)qi * a.os[2];

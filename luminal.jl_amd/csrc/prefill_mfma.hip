@@ -319,7 +319,7 @@ __global__ __launch_bounds__(64 * NW, WPS) void prefill_mfma_kernel(PrefillArgs 
     for (int kb = 0; kb < NKB; kb++)
 #pragma unroll
       for (int i = 0; i < 16; i++) mx = fmaxf(mx, sacc[kb][i]);
-    mx = fmaxf(mx, __shfl_xor(mx, 32));
+    mx = max_over_wave_halves(mx);
     // m_i is finite after the first tile (key 0 is visible to every query); -inf before it.
     if (__builtin_amdgcn_ballot_w64((mx - m_i) * c > kLazyRescale) != 0) {  // wave-uniform
       const float m_new = fmaxf(m_i, mx);
@@ -394,7 +394,7 @@ __global__ __launch_bounds__(64 * NW, WPS) void prefill_mfma_kernel(PrefillArgs 
   }
 
   // ---- epilogue: out[qi][d] = O^T[d][qi] / l ----
-  const float l_tot = l_i + __shfl_xor(l_i, 32);
+  const float l_tot = sum_over_wave_halves(l_i);
   const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
   if (qi < a.Sq) {
     const int64_t off = b * a.os[0] + hq * a.os[1] + (int64_t)qi * a.os[2];
@@ -583,7 +583,7 @@ __global__ __launch_bounds__(1024, 4) void prefill_mfma_wide_kernel(PrefillArgs 
     float mx = sacc[0];
 #pragma unroll
     for (int i = 1; i < 16; i++) mx = fmaxf(mx, sacc[i]);
-    mx = fmaxf(mx, __shfl_xor(mx, 32));
+    mx = max_over_wave_halves(mx);
     if (__builtin_amdgcn_ballot_w64((mx - m_i) * c > kLazyRescale) != 0) {
       const float m_new = fmaxf(m_i, mx);
       const float alpha = __builtin_amdgcn_exp2f((m_i - m_new) * c);
@@ -650,7 +650,7 @@ __global__ __launch_bounds__(1024, 4) void prefill_mfma_wide_kernel(PrefillArgs 
       for (int i = 0; i < 16; i++) oacc[db][i] = oacc[db][i] * a0 + slot[(2 + db * 16 + i) * 64] * a1;
   }
 
-  const float l_tot = l_i + __shfl_xor(l_i, 32);
+  const float l_tot = sum_over_wave_halves(l_i);
   const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
   if (qi < a.Sq) {
     const int64_t off = b * a.os[0] + hq * a.os[1] + (int64_t)qi * a.os[2];
