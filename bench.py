@@ -507,15 +507,18 @@ def ceiling_leg(lm, dev):
              "MFMA + 6 vector instr (1 exp) + 1 LDS fragment read per 2 MFMAs", "MFMA + 4 vector instr (1 exp) + 1 LDS fragment read",
              "MFMA + 4 vector instr (1 exp) + 1 LDS fragment read per 2 MFMAs"]
     res["instruction_mix_streams"] = {}
+    mix_sink = lm.HipArray((512 * 512,), "f32", dev)
     for mix, label in enumerate(mixes):
-        fl = [0.0]
+        row = {}
+        for wps in (2, 4):
+            fl = [0.0]
 
-        def fn():
-            fl[0] = lm.binding.calib_mix(sink.ptr, dq.ptr, 1 << 17, 10000, mix)
-        _, ev = time_steps(fn, 3, 1, lm.binding)
-        tf = fl[0] / (ev * 1e-3) / 1e12
-        res["instruction_mix_streams"][label] = {"TFLOP/s": tf, "frac_of_peak": tf / PEAK_FP16_TFLOPS}
-        log("[ceiling] synthetic stream, %s: %.0f TFLOP/s (%.1f%% of peak)" % (label, tf, 100 * tf / PEAK_FP16_TFLOPS))
+            def fn():
+                fl[0] = lm.binding.calib_mix(mix_sink.ptr, dq.ptr, 1 << 17, 10000 // (wps // 2), mix, wps)
+            _, ev = time_steps(fn, 3, 1, lm.binding)
+            row["TFLOP/s at %d waves per SIMD" % wps] = fl[0] / (ev * 1e-3) / 1e12
+        res["instruction_mix_streams"][label] = row
+        log("[ceiling] synthetic stream, %s: %.0f TFLOP/s at 2 waves per SIMD, %.0f at 4" % ((label,) + tuple(row.values())))
     out = lm.HipArray((B, H, S, D), "f16", dev)
     p = attn_params(lm, out, dq, dk, dv, "f16", False, lm.default_scale(D))
     _, ev = time_steps(lambda: lm.binding.flash_attn_fwd(p), 10, 3, lm.binding)

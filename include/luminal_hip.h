@@ -119,13 +119,14 @@ int lmh_calib_mfma_xcds(void *sink_dev, const void *operands_dev, size_t operand
                         double *flops_per_workgroup, void *stream);
 
 /* Measurement aid with no counterpart in the reference: an interleaved instruction stream with the mix of an attention
- * inner loop, two waves per SIMD on the whole chip, no barriers and no dependencies between the matrix and the vector
- * work: the best case for a kernel of that mix. Per v_mfma_f32_32x32x16_f16:
+ * inner loop, `waves_per_simd` (2 or 4) waves per SIMD on the whole chip, no barriers and no dependencies between the
+ * matrix and the vector work: the best case for a kernel of that mix. Per v_mfma_f32_32x32x16_f16:
  *   mix 0: nothing else            mix 1: 6 vector instructions, one of them v_exp_f32
  *   mix 2: mix 1 + one 16-byte-per-lane LDS fragment read      mix 3: mix 1 + one such read per two MFMAs
  *   mix 4: 4 vector instructions (1 exp) + one read            mix 5: 4 vector instructions (1 exp) + one read per two
- * `sink_dev` receives 256*512 floats, operands as for lmh_calib_mfma; `*flops` (host, optional) the flops of the launch. */
-int lmh_calib_mix(void *sink_dev, const void *operands_dev, size_t operand_bytes, int iters, int mix, double *flops, void *stream);
+ * `sink_dev` receives 512*512 floats, operands as for lmh_calib_mfma; `*flops` (host, optional) the flops of the launch. */
+int lmh_calib_mix(void *sink_dev, const void *operands_dev, size_t operand_bytes, int iters, int mix, int waves_per_simd,
+                  double *flops, void *stream);
 
 /* ---- flash attention forward: replaces
  *   execute_op!(out, op::FlashAttentionOp, q, k, v)   reference src/Execution.jl:565-578

@@ -133,7 +133,7 @@ def load():
     L.lmh_calib_mfma.argtypes = [vp, vp, ctypes.c_size_t, ctypes.c_int, ctypes.POINTER(ctypes.c_double), vp]
     L.lmh_flash_attn_plan.argtypes = [ctypes.POINTER(AttnParams), ctypes.c_char_p, ctypes.c_size_t]
     L.lmh_flash_attn_plan.restype = ctypes.c_int
-    L.lmh_calib_mix.argtypes = [vp, vp, ctypes.c_size_t, ctypes.c_int, ctypes.c_int, ctypes.POINTER(ctypes.c_double), vp]
+    L.lmh_calib_mix.argtypes = [vp, vp, ctypes.c_size_t, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.POINTER(ctypes.c_double), vp]
     L.lmh_calib_mix.restype = ctypes.c_int
     L.lmh_calib_read.argtypes = [vp, ctypes.c_size_t, vp, vp]
     L.lmh_calib_read.restype = ctypes.c_int
@@ -305,10 +305,10 @@ def flash_attn_plan(params):
     return buf.value.decode()
 
 
-def calib_mix(sink, operands, operand_bytes, iters, mix, stream=None):
-    """Launch the synthetic instruction-mix stream `mix` (0..5); returns the flops of the launch."""
+def calib_mix(sink, operands, operand_bytes, iters, mix, waves_per_simd=2, stream=None):
+    """Launch the synthetic instruction-mix stream `mix` (0..5) at 2 or 4 waves per SIMD; returns the flops of the launch."""
     flops = ctypes.c_double(0.0)
-    check(load().lmh_calib_mix(sink, operands, operand_bytes, iters, mix, ctypes.byref(flops), stream))
+    check(load().lmh_calib_mix(sink, operands, operand_bytes, iters, mix, waves_per_simd, ctypes.byref(flops), stream))
     return flops.value
 
 

@@ -58,7 +58,7 @@ __global__ __launch_bounds__(256) void calib_copy_kernel(uint4 *__restrict__ dst
 }
 // An interleaved stream with a chosen instruction mix per MFMA: NV vector instructions (NE of them v_exp_f32, the
 // rest fused multiply-adds) and one 16-byte-per-lane LDS read every LDS_EVERY MFMAs (0 = none; the fragment read
-// feeds the A operand of the next LDS_EVERY MFMAs). Two waves per SIMD, operands from caller-supplied values. This
+// feeds the A operand of the next LDS_EVERY MFMAs). Two or four waves per SIMD, operands from caller-supplied values. This
 // is the best case of a kernel with that mix — no barriers, no staging, no dependencies between the MFMA and the
 // vector work — so its rate on the whole chip is the ceiling for an attention kernel of the same mix.
 template <int NV, int NE, int LDS_EVERY>
@@ -169,12 +169,15 @@ extern "C" int lmh_calib_mfma_xcds(void *sink, const void *operands, size_t oper
   return LMH_OK;
 }
 
-extern "C" int lmh_calib_mix(void *sink, const void *operands, size_t operand_bytes, int iters, int mix, double *flops, void *stream) {
+extern "C" int lmh_calib_mix(void *sink, const void *operands, size_t operand_bytes, int iters, int mix, int waves_per_simd,
+                             double *flops, void *stream) {
   using namespace lmh;
   if (!sink || !operands) return fail(LMH_E_NULL, "lmh_calib_mix: null pointer");
   if (operand_bytes < 32 || operand_bytes % 16 != 0 || (reinterpret_cast<uintptr_t>(operands) & 15u) || iters < 1)
     return fail(LMH_E_SHAPE, "lmh_calib_mix: operands must be >= 32 bytes, a multiple of 16, 16-byte aligned; iters >= 1");
-  const dim3 grid(256), block(512);  // one workgroup per CU, two waves per SIMD
+  if (waves_per_simd != 2 && waves_per_simd != 4)
+    return fail(LMH_E_UNSUPPORTED, "lmh_calib_mix: waves_per_simd must be 2 or 4, got %d", waves_per_simd);
+  const dim3 grid(128 * waves_per_simd), block(512);  // one or two workgroups of 8 waves per CU
   float *snk = reinterpret_cast<float *>(sink);
   const calib_half8_t *ops = reinterpret_cast<const calib_half8_t *>(operands);
   const int n_ops = (int)(operand_bytes / 16);
@@ -189,7 +192,7 @@ extern "C" int lmh_calib_mix(void *sink, const void *operands, size_t operand_by
     default: return fail(LMH_E_UNSUPPORTED, "lmh_calib_mix: mix %d is not one of 0..5", mix);
   }
   LMH_HIP_TRY(hipGetLastError());
-  if (flops) *flops = 256.0 * 8.0 * iters * 8.0 * (2.0 * 32 * 32 * 16);
+  if (flops) *flops = (double)grid.x * 8.0 * iters * 8.0 * (2.0 * 32 * 32 * 16);
   return LMH_OK;
 }
 

@@ -753,6 +753,9 @@ def test_calibration_kernels(lm, hip):
     flops = lm.binding.calib_mix(sink.ptr, ones.ptr, 1 << 13, 3, 0)
     assert flops == 256 * 8 * 3 * 8 * 2 * 32 * 32 * 16
     assert np.all(sink.to_host() == 64 * 16 * 2 * 3 + 8)
+    big = lm.HipArray((512 * 512,), "f32", hip).fill_bytes(0xFF)
+    assert lm.binding.calib_mix(big.ptr, ones.ptr, 1 << 13, 3, 0, 4) == 2 * flops  # two workgroups per CU
+    assert np.all(big.to_host() == 64 * 16 * 2 * 3 + 8)
     for mix in (2, 5):  # LDS fragments are ones too, so the matrix part is unchanged; the vector part is bounded
         sink.fill_bytes(0xFF)
         lm.binding.calib_mix(sink.ptr, ones.ptr, 1 << 13, 3, mix)
@@ -760,6 +763,8 @@ def test_calibration_kernels(lm, hip):
         assert np.all(np.isfinite(got)) and np.all(np.abs(got - 64 * 16 * 2 * 3) < 4096)
     with pytest.raises(lm.LuminalHipError):
         lm.binding.calib_mix(sink.ptr, ones.ptr, 1 << 13, 3, 6)
+    with pytest.raises(lm.LuminalHipError):
+        lm.binding.calib_mix(sink.ptr, ones.ptr, 1 << 13, 3, 0, 3)
 
 
 def test_compiled_decode_step_graph_serves_every_position(lm, hip, oracle):
