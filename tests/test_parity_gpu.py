@@ -563,6 +563,28 @@ def test_strided_tensors(lm, hip, oracle):
     assert rel_err(out.to_host(), oracle.flash_attn(q, k, v, causal=True)) <= 2e-3
 
 
+def test_strided_tensors_on_the_wide_workgroups(lm, hip, oracle):
+    # cross attention over K and V interleaved in one [B, H, Sk, 2, D] buffer, Q and the output as [B, Sq, H, D]
+    # (head stride D, row stride H*D): every stride differs from the contiguous one
+    B, H, Sq, Sk, D = 2, 20, 448, 800, 64
+    q, k, v = inputs(oracle, (B, H, Sq, D), (B, H, Sk, D), "f16", 8100)
+    dkv = lm.to_device(np.stack([k, v], axis=3), hip, "f16")
+    dq = lm.to_device(np.ascontiguousarray(q.transpose(0, 2, 1, 3)), hip, "f16")  # [B, Sq, H, D]
+    out = lm.HipArray((B, Sq, H, D), "f16", hip)
+    p = lm.binding.AttnParams()
+    p.out, p.q, p.k, p.v = out.ptr, dq.ptr, dkv.ptr, dkv.ptr + D * 2
+    p.B, p.Hq, p.Hkv, p.Sq, p.Sk, p.D = B, H, H, Sq, Sk, D
+    for arr in (p.k_stride, p.v_stride):
+        arr[0], arr[1], arr[2] = H * Sk * 2 * D, Sk * 2 * D, 2 * D
+    for arr in (p.q_stride, p.o_stride):
+        arr[0], arr[1], arr[2] = Sq * H * D, D, H * D
+    p.dtype, p.scale, p.causal, p.head_map = lm.binding.LMH_F16, lm.default_scale(D), 0, 0
+    assert "prefill_mfma_wide_kernel" in lm.binding.flash_attn_plan(p)
+    lm.binding.flash_attn_fwd(p)
+    got = out.to_host().transpose(0, 2, 1, 3)
+    assert rel_err(got, oracle.flash_attn(q, k, v, causal=False, nthreads=NT)) <= 2e-3
+
+
 def test_compiled_graph_reuses_buffers(lm, hip, oracle):
     # compile() pre-allocates one buffer per node and runs in place (reference src/Compiler.jl:218-255)
     B, H, S, D = 1, 4, 96, 64
