@@ -211,6 +211,22 @@ function execute_op!(out::HipArray{TO,4}, op::FlashAttentionOp, q::HipArray{T,4}
     return out
 end
 
+"""
+    flash_attention_plan(op, q, k, v) -> String
+
+Names the kernel (instantiation, workgroup count) that `execute_op!` would launch for these arrays; launches nothing.
+"""
+function flash_attention_plan(op::FlashAttentionOp, q::HipArray{T,4}, k::HipArray{T,4}, v::HipArray{T,4};
+                              head_map::Int32=HEADMAP_INTERLEAVED) where {T}
+    B, Hq, Sq, D = size(q)
+    _, Hkv, Sk, _ = size(k)
+    p = Ref(AttnParams(q.ptr, q.ptr, k.ptr, v.ptr, C_NULL, B, Hq, Hkv, Sq, Sk, D, Z3, Z3, Z3, Z3,
+                       dtype_code(T), op.scale, Int32(op.causal), head_map, Int32(0), C_NULL))
+    text = Vector{UInt8}(undef, 256)
+    check(ccall((:lmh_flash_attn_plan, libluminal_hip), Cint, (Ref{AttnParams}, Ptr{UInt8}, Csize_t), p, text, length(text)))
+    return GC.@preserve text unsafe_string(pointer(text))
+end
+
 function execute_op(op::FlashAttentionOp, q::HipArray, k::HipArray, v::HipArray)
     out = similar(q)                      # src/Execution.jl:252-255
     return execute_op!(out, op, q, k, v)
@@ -580,6 +596,6 @@ end
 
 export HIPDevice, HipArray, BF16Bits, release_capture!, enable_capture!, compile_hip, DecodeAttentionOp, decode_attention,
        RotaryEmbeddingOp, rotary_embedding, KVAppendOp, kv_cache_append, get_device, functional, rope!, kv_append!,
-       self_attention_core!, cached_self_attention_core!, self_attention_core, cached_self_attention_core
+       self_attention_core!, cached_self_attention_core!, self_attention_core, cached_self_attention_core, flash_attention_plan
 
 end # module
