@@ -1,0 +1,79 @@
+"""Seeded sweeps over shapes nobody picked by hand: every case is drawn from a fixed generator, run through the C ABI and
+compared with the CPU oracle to the contract's tolerance. The sweeps report which kernels the cases reached."""
+import numpy as np
+import pytest
+
+from conftest import TOL, rel_err
+from test_parity_gpu import inputs, run_decode, run_flash
+
+pytestmark = pytest.mark.gpu
+
+NT = 16
+HEADS = [(1, 1), (4, 4), (8, 2), (6, 3), (12, 4), (5, 1)]
+
+
+def poison_tail(k, v, lens):
+    kp, vp = k.copy(), v.copy()
+    for b, n in enumerate(lens):
+        kp[b, :, n:] = np.nan
+        vp[b, :, n:] = np.nan
+    return kp, vp
+
+
+def test_prefill_random_shapes(lm, hip, oracle):
+    reached = {}
+    for case in range(56):
+        rng = np.random.default_rng(91000 + case)
+        dtype = ["f32", "f16", "bf16"][case % 3]
+        D = int(rng.choice([8, 16, 24, 40, 64, 72, 80, 96, 104, 128, 136, 192]))
+        Hq, Hkv = HEADS[int(rng.integers(len(HEADS)))]
+        B = int(rng.integers(1, 4))
+        causal = bool(rng.integers(2))
+        Sq = int(rng.integers(1, 301))
+        Sk = Sq if causal else int(rng.integers(1, 701))
+        head_map = int(rng.integers(2))
+        lens = None if rng.integers(3) == 0 else rng.integers(1, Sk + 1, size=B).astype(np.int32)
+        plan = lm.flash_attention_plan((B, Hq, Sq, D), (B, Hkv, Sk, D), dtype, causal)
+        what = "case %d: %s B=%d Hq=%d Hkv=%d Sq=%d Sk=%d D=%d causal=%s head_map=%d kv_len=%s -> %s" % (
+            case, dtype, B, Hq, Hkv, Sq, Sk, D, causal, head_map, None if lens is None else lens.tolist(), plan)
+        print(what, flush=True)
+        q, k, v = inputs(oracle, (B, Hq, Sq, D), (B, Hkv, Sk, D), dtype, 92000 + 3 * case, float(rng.choice([0.5, 1.0, 2.0])))
+        kp, vp = (k, v) if lens is None else poison_tail(k, v, lens)
+        got = run_flash(lm, hip, q, kp, vp, dtype, causal, head_map=head_map, kv_len=lens)
+        want = oracle.flash_attn(q, k, v, causal=causal, head_map=head_map, kv_len=lens, nthreads=NT)
+        err = rel_err(got, want)
+        assert err <= TOL[dtype], "%s: rel err %.3g" % (what, err)
+        reached[plan.split("<")[0]] = reached.get(plan.split("<")[0], 0) + 1
+    print("kernels reached:", reached, flush=True)
+    assert {"prefill_f32_kernel", "prefill_mfma_kernel", "prefill_valu_kernel"} <= set(reached)
+
+
+def test_decode_random_shapes(lm, hip, oracle):
+    for case in range(48):
+        rng = np.random.default_rng(93000 + case)
+        dtype = ["f32", "f16", "bf16"][case % 3]
+        D = int(rng.choice([8, 40, 64, 96, 128, 256]))
+        Hq, Hkv = HEADS[int(rng.integers(len(HEADS)))]
+        B = int(rng.integers(1, 6))
+        Lmax = int(rng.integers(1, 3001))
+        splits = int(rng.choice([0, 0, 1, 2, 5]))
+        head_map = int(rng.integers(2))
+        lens = None if rng.integers(4) == 0 else rng.integers(0, Lmax + 1, size=B).astype(np.int32)
+        what = "case %d: %s B=%d Hq=%d Hkv=%d Lmax=%d D=%d splits=%d head_map=%d kv_len=%s" % (
+            case, dtype, B, Hq, Hkv, Lmax, D, splits, head_map, None if lens is None else lens.tolist())
+        print(what, flush=True)
+        q = oracle.round_to(oracle.gen_normal((B, Hq, D), 94000 + 3 * case), dtype)
+        k = oracle.round_to(oracle.gen_normal((B, Hkv, Lmax, D), 94001 + 3 * case), dtype)
+        v = oracle.round_to(oracle.gen_normal((B, Hkv, Lmax, D), 94002 + 3 * case), dtype)
+        kp, vp = (k, v) if lens is None else poison_tail(k, v, lens)
+        got = run_decode(lm, hip, q, kp, vp, dtype, kv_len=lens, head_map=head_map, num_splits=splits)
+        want_len = None if lens is None else np.maximum(lens, 1)
+        want = oracle.decode_attn(q, k, v, kv_len=want_len, head_map=head_map, nthreads=NT)
+        keep = np.arange(B) if lens is None else np.nonzero(lens > 0)[0]
+        assert np.isfinite(got).all(), what
+        if len(keep):
+            err = rel_err(got[keep], want[keep])
+            assert err <= TOL[dtype], "%s: rel err %.3g" % (what, err)
+        if lens is not None:
+            for b in np.nonzero(lens == 0)[0]:
+                assert np.all(got[b] == 0), what  # a sequence without keys is written as zeros
