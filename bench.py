@@ -505,7 +505,8 @@ def ceiling_leg(lm, dev):
     # the ceiling of a kernel with attention's instruction mix: synthetic interleaved streams on the whole chip
     mixes = ["MFMA only", "MFMA + 6 vector instr (1 exp)", "MFMA + 6 vector instr (1 exp) + 1 LDS fragment read",
              "MFMA + 6 vector instr (1 exp) + 1 LDS fragment read per 2 MFMAs", "MFMA + 4 vector instr (1 exp) + 1 LDS fragment read",
-             "MFMA + 4 vector instr (1 exp) + 1 LDS fragment read per 2 MFMAs"]
+             "MFMA + 4 vector instr (1 exp) + 1 LDS fragment read per 2 MFMAs",
+             "MFMA + 11 vector instr (the exp as a 6-instruction polynomial) + 1 LDS fragment read"]
     res["instruction_mix_streams"] = {}
     mix_sink = lm.HipArray((512 * 512,), "f32", dev)
     for mix, label in enumerate(mixes):

@@ -189,7 +189,8 @@ extern "C" int lmh_calib_mix(void *sink, const void *operands, size_t operand_by
     case 3: hipLaunchKernelGGL((calib_mix_kernel<6, 1, 2>), grid, block, 0, st, snk, ops, n_ops, iters); break;
     case 4: hipLaunchKernelGGL((calib_mix_kernel<4, 1, 1>), grid, block, 0, st, snk, ops, n_ops, iters); break;
     case 5: hipLaunchKernelGGL((calib_mix_kernel<4, 1, 2>), grid, block, 0, st, snk, ops, n_ops, iters); break;
-    default: return fail(LMH_E_UNSUPPORTED, "lmh_calib_mix: mix %d is not one of 0..5", mix);
+    case 6: hipLaunchKernelGGL((calib_mix_kernel<11, 0, 1>), grid, block, 0, st, snk, ops, n_ops, iters); break;
+    default: return fail(LMH_E_UNSUPPORTED, "lmh_calib_mix: mix %d is not one of 0..6", mix);
   }
   LMH_HIP_TRY(hipGetLastError());
   if (flops) *flops = (double)grid.x * 8.0 * iters * 8.0 * (2.0 * 32 * 32 * 16);

@@ -784,7 +784,7 @@ def test_calibration_kernels(lm, hip):
         got = sink.to_host()
         assert np.all(np.isfinite(got)) and np.all(np.abs(got - 64 * 16 * 2 * 3) < 4096)
     with pytest.raises(lm.LuminalHipError):
-        lm.binding.calib_mix(sink.ptr, ones.ptr, 1 << 13, 3, 6)
+        lm.binding.calib_mix(sink.ptr, ones.ptr, 1 << 13, 3, 7)
     with pytest.raises(lm.LuminalHipError):
         lm.binding.calib_mix(sink.ptr, ones.ptr, 1 << 13, 3, 0, 3)
 
