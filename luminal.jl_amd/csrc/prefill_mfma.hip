@@ -175,6 +175,15 @@ __global__ __launch_bounds__(64 * NW, WPS) void prefill_mfma_kernel(PrefillArgs 
     uint4 raw = make_uint4(0, 0, 0, 0);
     if (qi < a.Sq && 16 * ks + 8 * g < a.D) raw = *reinterpret_cast<const uint4 *>(qp + (int64_t)qi * a.qs[2] + 16 * ks + 8 * g);
     qreg[ks] = __builtin_bit_cast(vec8, raw);
+#ifdef LMH_FOLD_SCALE
+    // Measurement build, not the shipped path: scale * log2(e) multiplied into the Q fragments (rounded to the element
+    // type once more), the running max kept in log2 units and handed to the first QK^T MFMA of a block as its
+    // accumulator input, so that the MFMAs deliver the argument of exp2 and the per-score v_fma disappears. The extra
+    // rounding moves a logit by up to 2^-12 of its magnitude: 1.5e-4 of the output range at a row max of 4 (log2 units),
+    // 4.5e-4 at 16, 1.5e-3 at 45, over the 2e-3 budget at a few hundred (the large-logit parity tests fail).
+#pragma unroll
+    for (int e = 0; e < 8; e++) qreg[ks][e] = MT::cvt((float)qreg[ks][e] * (a.scale * kLog2e));
+#endif
   }
 
   floatx16_t oacc[DB];
@@ -185,6 +194,13 @@ __global__ __launch_bounds__(64 * NW, WPS) void prefill_mfma_kernel(PrefillArgs 
   float m_i = -INFINITY;  // running max of the raw (unscaled) scores of query qi
   float l_i = 0.f;        // this lane's half of the running sum
   const float c = a.scale * kLog2e;
+#ifdef LMH_FOLD_SCALE
+  float neg_mc = 0.f;     // minus the running max, in log2 units ...
+  floatx16_t neg_mc16;    // ... and as the accumulator input of a block's first MFMA (rewritten only when the max is raised)
+#pragma unroll
+  for (int i = 0; i < 16; i++) neg_mc16[i] = 0.f;
+  bool have_m = false;
+#endif
 
   // ---- tile staging: global memory -> LDS directly (buffer_load_dwordx4 ... lds), one tile ahead ----
   // A tile of BT rows x LD elements is BT * LD / 512 blocks of 1 KB. One wave-wide load fills one block:
@@ -297,7 +313,11 @@ __global__ __launch_bounds__(64 * NW, WPS) void prefill_mfma_kernel(PrefillArgs 
       for (int ks = 0; ks < KS; ks++)
 #pragma unroll
         for (int kb = 0; kb < KBG; kb++) {
+#ifdef LMH_FOLD_SCALE
+          sacc[kb0 + kb] = MT::mfma(kf[kb][ks], qreg[ks], ks == 0 ? neg_mc16 : sacc[kb0 + kb]);
+#else
           sacc[kb0 + kb] = MT::mfma(kf[kb][ks], qreg[ks], sacc[kb0 + kb]);
+#endif
         }
     }
 
@@ -320,6 +340,26 @@ __global__ __launch_bounds__(64 * NW, WPS) void prefill_mfma_kernel(PrefillArgs 
 #pragma unroll
       for (int i = 0; i < 16; i++) mx = fmaxf(mx, sacc[kb][i]);
     mx = max_over_wave_halves(mx);
+#ifdef LMH_FOLD_SCALE
+    // the scores are c s - c m already: raise m (and re-base this tile) where a row exceeds it by 2^8, and on the first tile
+    if (!have_m || __builtin_amdgcn_ballot_w64(mx > kLazyRescale) != 0) {
+      const float d = have_m ? fmaxf(mx, 0.f) : mx;
+      const float alpha = have_m ? __builtin_amdgcn_exp2f(-d) : 1.f;
+      have_m = true;
+      neg_mc -= d;
+#pragma unroll
+      for (int i = 0; i < 16; i++) neg_mc16[i] = neg_mc;
+      l_i *= alpha;
+#pragma unroll
+      for (int db = 0; db < DB; db++)
+#pragma unroll
+        for (int i = 0; i < 16; i++) oacc[db][i] *= alpha;
+#pragma unroll
+      for (int kb = 0; kb < NKB; kb++)
+#pragma unroll
+        for (int i = 0; i < 16; i++) sacc[kb][i] -= d;
+    }
+#else
     // m_i is finite after the first tile (key 0 is visible to every query); -inf before it.
     if (__builtin_amdgcn_ballot_w64((mx - m_i) * c > kLazyRescale) != 0) {  // wave-uniform
       const float m_new = fmaxf(m_i, mx);
@@ -331,6 +371,7 @@ __global__ __launch_bounds__(64 * NW, WPS) void prefill_mfma_kernel(PrefillArgs 
 #pragma unroll
         for (int i = 0; i < 16; i++) oacc[db][i] *= alpha;
     }
+#endif
     const float mc = m_i * c;
     vec8 pf[NKB][2], pf_lo[NKB][2];
 #pragma unroll
@@ -339,7 +380,11 @@ __global__ __launch_bounds__(64 * NW, WPS) void prefill_mfma_kernel(PrefillArgs 
       for (int t = 0; t < 2; t++) {
 #pragma unroll
         for (int e = 0; e < 8; e++) {
+#ifdef LMH_FOLD_SCALE
+          const float p = __builtin_amdgcn_exp2f(sacc[kb][8 * t + e]);
+#else
           const float p = __builtin_amdgcn_exp2f(sacc[kb][8 * t + e] * c - mc);
+#endif
           pf[kb][t][e] = MT::cvt(p);
           if (MT::kSplitP) pf_lo[kb][t][e] = MT::cvt(p - (float)pf[kb][t][e]);
         }
@@ -365,6 +410,9 @@ __global__ __launch_bounds__(64 * NW, WPS) void prefill_mfma_kernel(PrefillArgs 
     }
   }
 
+#ifdef LMH_FOLD_SCALE
+  m_i = have_m ? -neg_mc / c : -INFINITY;  // back to the units the merge below works in
+#endif
   // ---- key groups: fold group 1's (m, l, O) into group 0's; lane for lane the same layout ----
   if (KSPLIT > 1) {
     constexpr int NF = DB * 16 + 2;  // floats per lane
