@@ -193,3 +193,21 @@ def test_graph_recording_argument_errors(lm):
     assert e.value.code == b.LMH_E_NULL
     assert b.load().lmh_graph_destroy(None) == 0
     assert b.load().lmh_stream_destroy(None) == 0
+
+
+def test_plain_c_client_builds_against_the_public_header(tmp_path):
+    """tests/c_host/abi_client.c uses nothing but include/luminal_hip.h and the C library: it must compile as pedantic
+    C99 without a warning, link against the shared library and start. Without a GPU it stops after the device count
+    (exit status 77); with one it runs its checks (the GPU suite does that on the in-tree binary)."""
+    import importlib.util
+    import subprocess
+    here = os.path.dirname(os.path.abspath(__file__))
+    spec = importlib.util.spec_from_file_location("c_host_build", os.path.join(here, "c_host", "build.py"))
+    mod = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(mod)
+    # same rpath convention as the in-tree binary: place it two levels below the repository root
+    out_dir = os.path.join(here, "c_host")
+    binary = mod.build(os.path.join(out_dir, "abi_client"))
+    res = subprocess.run([binary], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=120)
+    assert "libluminal_hip version" in res.stdout, res.stdout
+    assert res.returncode in (0, 77), res.stdout

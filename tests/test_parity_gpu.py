@@ -753,6 +753,19 @@ def test_incremental_decode_equals_causal_prefill(lm, hip, oracle):
     assert cache.step_pos == S
 
 
+def test_plain_c_client_of_the_abi(hip):
+    """The C ABI driven from C, not Python: tests/c_host/abi_client (built beforehand by `__graft_entry__.build()` or
+    `python tests/c_host/build.py`) runs cross attention, causal GQA attention and split-KV decode in fp32 against its
+    own float64 softmax and exits 0 when all are within 1e-5."""
+    import os
+    import subprocess
+    binary = os.path.join(os.path.dirname(os.path.abspath(__file__)), "c_host", "abi_client")
+    assert os.path.exists(binary), "build tests/c_host/abi_client first (python tests/c_host/build.py)"
+    res = subprocess.run([binary], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=120)
+    print(res.stdout)
+    assert res.returncode == 0, res.stdout
+
+
 def test_calibration_kernels(lm, hip):
     # measurement aids: the copy kernel copies, the bare MFMA loop reports its flops and checks its arguments
     n = 1 << 16
