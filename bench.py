@@ -553,6 +553,34 @@ def other_configs(lm, dev, check=False, only="other"):
     return res
 
 
+def grid_leg(lm, dev):
+    """Flash attention over a grid of square shapes (fp16 and bf16, causal and not, D = 64 / 128): µs per launch, TFLOP/s
+    and the kernel each shape reaches. Not one of the contract's configurations: a map of where the launcher's rules put
+    which instantiation, and of how far small launches are from the large ones."""
+    rows = []
+    for dtype in ("f16", "bf16"):
+        for causal in (True, False):
+            for D in (64, 128):
+                for B, H in ((1, 8), (1, 32), (4, 32)):
+                    for S in (512, 1024, 2048, 4096, 8192):
+                        if B * H * S * S > 2 * 32 * 8192 * 8192:
+                            continue
+                        hq, hk, hv = (lm.synth.normal((B, H, S, D), 5000 + i, 0.5) for i in range(3))
+                        q, k, v = (lm.HipArray(x.shape, dtype, dev).copy_from_host(x) for x in (hq, hk, hv))
+                        o = lm.HipArray((B, H, S, D), dtype, dev)
+                        p = attn_params(lm, o, q, k, v, dtype, causal, lm.default_scale(D))
+                        steps = 30 if B * H * S * S < 2e9 else 8
+                        _, ev = time_steps(lambda: lm.binding.flash_attn_fwd(p), steps, 3, lm.binding)
+                        flops = 4.0 * B * H * D * (S * (S + 1) / 2 if causal else S * S)
+                        row = {"dtype": dtype, "causal": causal, "B": B, "H": H, "S": S, "D": D, "launch_us": ev * 1e3,
+                               "TFLOP/s": flops / (ev * 1e-3) / 1e12, "kernel": lm.binding.flash_attn_plan(p)}
+                        rows.append(row)
+                        log("[grid] %-4s %-6s B=%d H=%-2d S=%-4d D=%-3d %8.1f us %7.1f TFLOP/s (%4.1f%%)  %s" % (
+                            dtype, "causal" if causal else "full", B, H, S, D, row["launch_us"], row["TFLOP/s"],
+                            100 * row["TFLOP/s"] / PEAK_FP16_TFLOPS, row["kernel"]))
+    return rows
+
+
 def copy_leg(lm, dev, steps, warmup):
     """The calibration copy kernel alone (profile this with --pmc FETCH_SIZE / WRITE_SIZE)."""
     nbytes = 1 << 30
@@ -568,7 +596,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--only", choices=["all", "prefill", "decode", "other", "c1", "c3", "c4", "ops", "step", "copy", "ceiling"], default="all")
+    ap.add_argument("--only", choices=["all", "prefill", "decode", "other", "c1", "c3", "c4", "ops", "step", "copy", "ceiling", "grid"], default="all")
     ap.add_argument("--decode-splits", type=int, default=0, help="KV splits for the decode leg (0 = library heuristic)")
     ap.add_argument("--cpu-seconds", type=float, default=15.0, help="CPU-baseline budget per leg; 0 disables it")
     args = ap.parse_args()
@@ -597,6 +625,10 @@ def main():
         return
     if args.only == "ceiling":
         line["ceiling"] = ceiling_leg(lm, dev)
+        print(json.dumps(line))
+        return
+    if args.only == "grid":
+        line["shape_grid"] = grid_leg(lm, dev)
         print(json.dumps(line))
         return
     if args.only in ("all", "prefill"):
