@@ -77,3 +77,53 @@ def test_decode_random_shapes(lm, hip, oracle):
         if lens is not None:
             for b in np.nonzero(lens == 0)[0]:
                 assert np.all(got[b] == 0), what  # a sequence without keys is written as zeros
+
+
+def test_wide_workgroup_random_shapes(lm, hip, oracle):
+    """Shapes drawn until 24 of them reach the one-workgroup-per-CU kernel (the plan query says which do): row-block
+    counts, key-group counts, ragged lengths and head dims nobody picked by hand."""
+    rng = np.random.default_rng(95000)
+    done, tried = 0, 0
+    seen = set()
+    while done < 24 and tried < 4000:
+        tried += 1
+        dtype = ["f16", "bf16"][int(rng.integers(2))]
+        D = int(rng.choice([16, 32, 40, 64, 72, 88, 96]))
+        G = int(rng.choice([1, 1, 2, 4]))
+        Hkv = int(rng.integers(1, 33))
+        B = int(rng.integers(1, 9))
+        Hq = Hkv * G
+        Sq = int(rng.integers(64, 601))
+        Sk = int(rng.integers(640, 2501))
+        if B * Hq > 256 or B * Hq * Sq * Sk * D > 6e9:
+            continue
+        plan = lm.flash_attention_plan((B, Hq, Sq, D), (B, Hkv, Sk, D), dtype, False)
+        if "prefill_mfma_wide_kernel" not in plan:
+            continue
+        key = plan.split("workgroups per head")[1]
+        if key in seen and rng.integers(3) != 0:  # favour plans not seen yet
+            continue
+        seen.add(key)
+        head_map = int(rng.integers(2))
+        lens = None if rng.integers(2) == 0 else rng.integers(0, Sk + 1, size=B).astype(np.int32)
+        what = "case %d: %s B=%d Hq=%d Hkv=%d Sq=%d Sk=%d D=%d head_map=%d kv_len=%s -> %s" % (
+            done, dtype, B, Hq, Hkv, Sq, Sk, D, head_map, None if lens is None else lens.tolist(), plan)
+        print(what, flush=True)
+        q, k, v = inputs(oracle, (B, Hq, Sq, D), (B, Hkv, Sk, D), dtype, 96000 + 3 * done, float(rng.choice([0.5, 1.0, 1.5])))
+        kp, vp = (k, v) if lens is None else poison_tail(k, v, lens)
+        got = run_flash(lm, hip, q, kp, vp, dtype, False, head_map=head_map, kv_len=lens)
+        hq = np.unique(rng.integers(0, Hq, size=min(Hq, 6)))
+        kv_of = hq if Hq == Hkv else (hq // G if head_map == 1 else hq % Hkv)
+        want_len = None if lens is None else np.maximum(lens, 1)
+        want = oracle.flash_attn(q[:, hq], k[:, kv_of], v[:, kv_of], causal=False, kv_len=want_len, nthreads=NT)
+        keep = np.arange(B) if lens is None else np.nonzero(lens > 0)[0]
+        assert np.isfinite(got).all(), what
+        if len(keep):
+            err = rel_err(got[keep][:, hq], want[keep])
+            assert err <= TOL[dtype], "%s: rel err %.3g" % (what, err)
+        if lens is not None:
+            for b in np.nonzero(lens == 0)[0]:
+                assert np.all(got[b] == 0), what
+        done += 1
+    assert done == 24, "only %d shapes reached the wide kernel" % done
+    print("plans covered:", sorted(seen), flush=True)
