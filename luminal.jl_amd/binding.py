@@ -9,6 +9,7 @@ import os
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(HERE, "lib", "libluminal_hip.so")
+CALIB_LIB_PATH = os.path.join(HERE, "lib", "libluminal_hip_calib.so")
 
 LMH_F32, LMH_F16, LMH_BF16 = 0, 1, 2
 HEADMAP_INTERLEAVED, HEADMAP_BLOCKED = 0, 1
@@ -20,11 +21,10 @@ LMH_E_NULL, LMH_E_SHAPE, LMH_E_UNSUPPORTED, LMH_E_WORKSPACE, LMH_E_HIP, LMH_E_NO
 
 # every symbol include/luminal_hip.h declares
 EXPORTS = [
-    "lmh_version", "lmh_last_error", "lmh_device_count", "lmh_init", "lmh_device_name", "lmh_malloc", "lmh_free",
+    "lmh_version", "lmh_measurement_build", "lmh_last_error", "lmh_device_count", "lmh_init", "lmh_device_name", "lmh_malloc", "lmh_free",
     "lmh_memset", "lmh_memcpy_h2d", "lmh_memcpy_d2h", "lmh_memcpy_d2d", "lmh_sync", "lmh_event_create",
     "lmh_event_destroy", "lmh_event_record", "lmh_event_elapsed_ms", "lmh_flash_attn_fwd",
-    "lmh_decode_workspace_bytes", "lmh_decode_auto_splits", "lmh_decode_attn", "lmh_calib_copy", "lmh_calib_read", "lmh_calib_mfma",
-    "lmh_calib_mfma_xcds", "lmh_calib_mix", "lmh_flash_attn_plan", "lmh_rope",
+    "lmh_decode_workspace_bytes", "lmh_decode_auto_splits", "lmh_decode_attn", "lmh_flash_attn_plan", "lmh_rope",
     "lmh_kv_append", "lmh_stream_create", "lmh_stream_destroy", "lmh_graph_capture_begin", "lmh_graph_capture_end",
     "lmh_graph_launch", "lmh_graph_destroy", "lmh_static_scratch_bytes", "lmh_decode_static_splits",
     "lmh_decode_attn_static",
@@ -86,9 +86,14 @@ class KvAppendParams(ctypes.Structure):
     ]
 
 
+# every symbol include/luminal_hip_calib.h declares (libluminal_hip_calib.so: measurement kernels, loaded on demand)
+CALIB_EXPORTS = ["lmh_calib_last_error", "lmh_calib_copy", "lmh_calib_read", "lmh_calib_mfma", "lmh_calib_mfma_xcds",
+                 "lmh_calib_mix"]
+
 ROPE_HALF_SPLIT, ROPE_INTERLEAVED = 0, 1
 
 _lib = None
+_calib = None
 
 
 def load():
@@ -103,6 +108,12 @@ def load():
     L = ctypes.CDLL(LIB_PATH)
     vp = ctypes.c_void_p
     L.lmh_version.restype = ctypes.c_int
+    L.lmh_measurement_build.restype = ctypes.c_int
+    if L.lmh_measurement_build() and os.environ.get("LMH_MEASUREMENT_BUILD") != "1":
+        raise RuntimeError(
+            "%s was compiled with experiment switches (lmh_measurement_build() == 1): its kernels may compute wrong "
+            "results on purpose. Rebuild with `python luminal.jl_amd/build.py`, or set LMH_MEASUREMENT_BUILD=1 to "
+            "load it for a measurement." % LIB_PATH)
     L.lmh_last_error.restype = ctypes.c_char_p
     L.lmh_device_count.restype = ctypes.c_int
     L.lmh_init.argtypes = [ctypes.c_int]
@@ -129,16 +140,8 @@ def load():
     L.lmh_static_scratch_bytes.restype = ctypes.c_size_t
     L.lmh_decode_static_splits.restype = ctypes.c_int32
     L.lmh_decode_static_splits.argtypes = [ctypes.c_int32] * 5
-    L.lmh_calib_copy.argtypes = [vp, vp, ctypes.c_size_t, vp]
-    L.lmh_calib_mfma.argtypes = [vp, vp, ctypes.c_size_t, ctypes.c_int, ctypes.POINTER(ctypes.c_double), vp]
     L.lmh_flash_attn_plan.argtypes = [ctypes.POINTER(AttnParams), ctypes.c_char_p, ctypes.c_size_t]
     L.lmh_flash_attn_plan.restype = ctypes.c_int
-    L.lmh_calib_mix.argtypes = [vp, vp, ctypes.c_size_t, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.POINTER(ctypes.c_double), vp]
-    L.lmh_calib_mix.restype = ctypes.c_int
-    L.lmh_calib_read.argtypes = [vp, ctypes.c_size_t, vp, vp]
-    L.lmh_calib_read.restype = ctypes.c_int
-    L.lmh_calib_mfma_xcds.argtypes = [vp, vp, ctypes.c_size_t, ctypes.c_int, ctypes.c_int, ctypes.POINTER(ctypes.c_double), vp]
-    L.lmh_calib_mfma_xcds.restype = ctypes.c_int
     L.lmh_rope.argtypes = [ctypes.POINTER(RopeParams)]
     L.lmh_kv_append.argtypes = [ctypes.POINTER(KvAppendParams)]
     L.lmh_stream_create.argtypes = [ctypes.POINTER(vp)]
@@ -147,7 +150,7 @@ def load():
     L.lmh_graph_capture_end.argtypes = [vp, ctypes.POINTER(vp)]
     L.lmh_graph_launch.argtypes = [vp, vp]
     L.lmh_graph_destroy.argtypes = [vp]
-    for name in ("lmh_rope", "lmh_kv_append", "lmh_calib_copy", "lmh_calib_read", "lmh_calib_mfma", "lmh_init", "lmh_device_name", "lmh_malloc", "lmh_free", "lmh_memset", "lmh_memcpy_h2d",
+    for name in ("lmh_rope", "lmh_kv_append", "lmh_init", "lmh_device_name", "lmh_malloc", "lmh_free", "lmh_memset", "lmh_memcpy_h2d",
                  "lmh_memcpy_d2h", "lmh_memcpy_d2d", "lmh_sync", "lmh_event_create", "lmh_event_destroy",
                  "lmh_event_record", "lmh_event_elapsed_ms", "lmh_flash_attn_fwd", "lmh_decode_attn"):
         getattr(L, name).restype = ctypes.c_int
@@ -155,9 +158,36 @@ def load():
     return L
 
 
+def load_calib():
+    """Load libluminal_hip_calib.so, the measurement kernels (once). Raises if it has not been built."""
+    global _calib
+    if _calib is not None:
+        return _calib
+    if not os.path.exists(CALIB_LIB_PATH):
+        raise RuntimeError("libluminal_hip_calib.so is not built (%s missing); run `python luminal.jl_amd/build.py`." % CALIB_LIB_PATH)
+    L = ctypes.CDLL(CALIB_LIB_PATH)
+    vp = ctypes.c_void_p
+    dp = ctypes.POINTER(ctypes.c_double)
+    L.lmh_calib_last_error.restype = ctypes.c_char_p
+    L.lmh_calib_copy.argtypes = [vp, vp, ctypes.c_size_t, vp]
+    L.lmh_calib_read.argtypes = [vp, ctypes.c_size_t, vp, vp]
+    L.lmh_calib_mfma.argtypes = [vp, vp, ctypes.c_size_t, ctypes.c_int, dp, vp]
+    L.lmh_calib_mfma_xcds.argtypes = [vp, vp, ctypes.c_size_t, ctypes.c_int, ctypes.c_int, dp, vp]
+    L.lmh_calib_mix.argtypes = [vp, vp, ctypes.c_size_t, ctypes.c_int, ctypes.c_int, ctypes.c_int, dp, vp]
+    for name in CALIB_EXPORTS[1:]:
+        getattr(L, name).restype = ctypes.c_int
+    _calib = L
+    return L
+
+
 def check(rc):
     if rc != LMH_OK:
         raise LuminalHipError(rc, load().lmh_last_error().decode("utf-8", "replace"))
+
+
+def check_calib(rc):
+    if rc != LMH_OK:
+        raise LuminalHipError(rc, load_calib().lmh_calib_last_error().decode("utf-8", "replace"))
 
 
 def device_count():
@@ -284,17 +314,17 @@ def graph_destroy(graph_exec):
 
 
 def calib_copy(dst, src, nbytes, stream=None):
-    check(load().lmh_calib_copy(dst, src, nbytes, stream))
+    check_calib(load_calib().lmh_calib_copy(dst, src, nbytes, stream))
 
 
 def calib_read(src, nbytes, sink4, stream=None):
-    check(load().lmh_calib_read(src, nbytes, sink4, stream))
+    check_calib(load_calib().lmh_calib_read(src, nbytes, sink4, stream))
 
 
 def calib_mfma(sink, operands, operand_bytes, iters, stream=None):
     """Launch the bare MFMA loop; returns the flops of the launch."""
     flops = ctypes.c_double(0.0)
-    check(load().lmh_calib_mfma(sink, operands, operand_bytes, iters, ctypes.byref(flops), stream))
+    check_calib(load_calib().lmh_calib_mfma(sink, operands, operand_bytes, iters, ctypes.byref(flops), stream))
     return flops.value
 
 
@@ -308,14 +338,14 @@ def flash_attn_plan(params):
 def calib_mix(sink, operands, operand_bytes, iters, mix, waves_per_simd=2, stream=None):
     """Launch the synthetic instruction-mix stream `mix` (0..5) at 2 or 4 waves per SIMD; returns the flops of the launch."""
     flops = ctypes.c_double(0.0)
-    check(load().lmh_calib_mix(sink, operands, operand_bytes, iters, mix, waves_per_simd, ctypes.byref(flops), stream))
+    check_calib(load_calib().lmh_calib_mix(sink, operands, operand_bytes, iters, mix, waves_per_simd, ctypes.byref(flops), stream))
     return flops.value
 
 
 def calib_mfma_xcds(sink, operands, operand_bytes, iters, active_xcds, stream=None):
     """The bare MFMA loop on the first `active_xcds` XCDs only; returns the flops of one running workgroup."""
     flops = ctypes.c_double(0.0)
-    check(load().lmh_calib_mfma_xcds(sink, operands, operand_bytes, iters, active_xcds, ctypes.byref(flops), stream))
+    check_calib(load_calib().lmh_calib_mfma_xcds(sink, operands, operand_bytes, iters, active_xcds, ctypes.byref(flops), stream))
     return flops.value
 
 

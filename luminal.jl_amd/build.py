@@ -1,7 +1,12 @@
-"""Build libluminal_hip.so (hand-written HIP for gfx950) in-tree with hipcc.
+"""Build libluminal_hip.so (hand-written HIP for gfx950) and libluminal_hip_calib.so (measurement kernels the
+benchmark uses) in-tree with hipcc.
 
 Usage: python luminal.jl_amd/build.py            # rebuild everything
-The library lands in luminal.jl_amd/lib/ and is what the ctypes binding loads.
+The libraries land in luminal.jl_amd/lib/ and are what the ctypes binding loads.
+
+LMH_EXTRA_FLAGS (extra -D switches for kernel experiments) is refused unless LMH_MEASUREMENT_BUILD=1 is set too;
+the library is then compiled with -DLMH_MEASUREMENT_BUILD, answers 1 to lmh_measurement_build(), and the binding
+refuses to load it unless the same variable is set in the loading process.
 """
 import os
 import shutil
@@ -12,7 +17,11 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIBDIR = os.path.join(HERE, "lib")
 LIBNAME = "libluminal_hip.so"
-SOURCES = ["api.hip", "prefill_valu.hip", "prefill_mfma.hip", "prefill_f32.hip", "decode.hip", "decode_mfma.hip", "cache_ops.hip", "calib.hip"]
+CALIB_LIBNAME = "libluminal_hip_calib.so"
+LIBRARIES = {
+    LIBNAME: ["api.hip", "prefill_valu.hip", "prefill_mfma.hip", "prefill_f32.hip", "decode.hip", "decode_mfma.hip", "cache_ops.hip"],
+    CALIB_LIBNAME: ["calib.hip"],
+}
 
 # -packed-fp32-ops: keep the compiler from forming v_pk_{add,mul,fma}_f32 out of scalar fp32 code.
 HIPCC_FLAGS = [
@@ -20,8 +29,18 @@ HIPCC_FLAGS = [
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wno-unused-command-line-argument",
 ]
-# extra -D switches for one-off kernel experiments (never set by the tests, the bench or the driver)
-HIPCC_FLAGS += os.environ.get("LMH_EXTRA_FLAGS", "").split()
+
+
+def experiment_flags():
+    """Extra -D switches for one-off kernel experiments (never set by the tests, the bench or the driver)."""
+    extra = os.environ.get("LMH_EXTRA_FLAGS", "").split()
+    if not extra:
+        return []
+    if os.environ.get("LMH_MEASUREMENT_BUILD") != "1":
+        raise RuntimeError("LMH_EXTRA_FLAGS=%r is set: experiment switches change what the kernels compute. Unset it, or set "
+                           "LMH_MEASUREMENT_BUILD=1 to build a library that is marked as a measurement build." % " ".join(extra))
+    print("[build] MEASUREMENT BUILD with %s: not a product library" % " ".join(extra), flush=True)
+    return extra + ["-DLMH_MEASUREMENT_BUILD"]
 
 
 def hipcc_path():
@@ -31,25 +50,27 @@ def hipcc_path():
     raise RuntimeError("hipcc not found; the HIP extension cannot be built")
 
 
-def library_path():
-    return os.path.join(LIBDIR, LIBNAME)
+def library_path(name=LIBNAME):
+    return os.path.join(LIBDIR, name)
 
 
 def build_library(verbose=True):
-    """Compile every .hip source for gfx950 and link the shared library. Always recompiles."""
+    """Compile every .hip source for gfx950 and link the shared libraries. Always recompiles."""
     hipcc = hipcc_path()
+    flags = HIPCC_FLAGS + experiment_flags()
     os.makedirs(LIBDIR, exist_ok=True)
     objdir = os.path.join(LIBDIR, "obj")
     os.makedirs(objdir, exist_ok=True)
     procs = []
-    for src in SOURCES:
-        obj = os.path.join(objdir, src.replace(".hip", ".o"))
-        cmd = [hipcc] + HIPCC_FLAGS + ["-c", os.path.join(CSRC, src), "-o", obj]
-        if verbose:
-            print("[build]", " ".join(cmd), flush=True)
-        procs.append((src, obj, subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)))
-    objs = []
-    for src, obj, proc in procs:
+    for libname, sources in LIBRARIES.items():
+        for src in sources:
+            obj = os.path.join(objdir, src.replace(".hip", ".o"))
+            cmd = [hipcc] + flags + ["-c", os.path.join(CSRC, src), "-o", obj]
+            if verbose:
+                print("[build]", " ".join(cmd), flush=True)
+            procs.append((libname, src, obj, subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)))
+    objs = {name: [] for name in LIBRARIES}
+    for libname, src, obj, proc in procs:
         out, _ = proc.communicate()
         # the host pass does not know the gfx-only target feature; that note is expected
         out = "\n".join(l for l in out.splitlines() if "packed-fp32-ops" not in l)
@@ -57,15 +78,16 @@ def build_library(verbose=True):
             raise RuntimeError("hipcc failed on %s:\n%s" % (src, out))
         if verbose and out.strip():
             print(out)
-        objs.append(obj)
-    tmp = library_path() + ".tmp"
-    cmd = [hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", tmp] + objs
-    if verbose:
-        print("[build]", " ".join(cmd), flush=True)
-    res = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
-    if res.returncode != 0:
-        raise RuntimeError("link failed:\n" + res.stdout)
-    os.replace(tmp, library_path())
+        objs[libname].append(obj)
+    for libname in LIBRARIES:
+        tmp = library_path(libname) + ".tmp"
+        cmd = [hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", tmp] + objs[libname]
+        if verbose:
+            print("[build]", " ".join(cmd), flush=True)
+        res = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+        if res.returncode != 0:
+            raise RuntimeError("link of %s failed:\n%s" % (libname, res.stdout))
+        os.replace(tmp, library_path(libname))
     return library_path()
 
 

@@ -102,6 +102,14 @@ extern "C" {
 
 int lmh_version(void) { return LMH_VERSION; }
 
+int lmh_measurement_build(void) {
+#ifdef LMH_MEASUREMENT_BUILD
+  return 1;
+#else
+  return 0;
+#endif
+}
+
 const char *lmh_last_error(void) { return g_last_error; }
 
 int lmh_device_count(void) {
@@ -136,7 +144,7 @@ int lmh_init(int device) {
   // set-up for lmh_decode_attn_static: resolve this device's copy of the static scratch now, so that the
   // entry point itself never has to (a failure here is reported by that entry point, not by init)
   void *unused = nullptr;
-  (void)static_scratch_for_current_device(&unused);
+  if (static_scratch_for_current_device(&unused) != LMH_OK) g_last_error[0] = 0;  // init succeeded: leave no stale message
   return LMH_OK;
 }
 
@@ -396,7 +404,9 @@ static int decode_launch(const lmh_decode_params *p, const char *fn, int32_t num
   if (a.qs[0] < 0 || a.qs[1] < 0 || a.os[0] < 0 || a.os[1] < 0) return fail(LMH_E_SHAPE, "%s: negative stride", fn);
 
   // the matrix-core kernel addresses a (b, kv head) slice with 32-bit buffer offsets
-  const bool slice_fits = (int64_t)p->Lmax * a.ks[2] * 2 < 0x7ffffff0 && (int64_t)p->Lmax * a.vs[2] * 2 < 0x7ffffff0;
+  // (a block of 32 rows is addressed even when Lmax is smaller, so bound that too)
+  const int64_t rows = p->Lmax > 32 ? p->Lmax : 32;
+  const bool slice_fits = rows * a.ks[2] * 2 < 0x7ffffff0 && rows * a.vs[2] * 2 < 0x7ffffff0;
   a.mfma_ok = (p->scale > 0.f && aligned16(p->q) && a.qs[0] % 8 == 0 && a.qs[1] % 8 == 0 && slice_fits) ? 1 : 0;
   a.num_splits = num_splits;
   a.chunk = decode_chunk_for(p->Lmax, a.num_splits);

@@ -7,10 +7,33 @@
 // (all-zero operands sustain a much higher rate than random ones). Timing this kernel on the same
 // kind of data as the attention inputs gives the rate the matrix cores can actually sustain, the
 // ceiling an attention kernel is measured against besides the published figure.
-#include "common.hpp"
+//
+// These kernels are measurement aids, not part of the attention backend: they are built into their own library,
+// libluminal_hip_calib.so (include/luminal_hip_calib.h), which only the benchmark and its test load.
+#include <hip/hip_runtime.h>
+#include <stdarg.h>
+#include <stdint.h>
+#include <stdio.h>
+
+#include "../../include/luminal_hip_calib.h"
 
 namespace lmh {
 namespace {
+thread_local char g_calib_error[256] = "";
+int fail(int code, const char *fmt, ...) __attribute__((format(printf, 2, 3)));
+int fail(int code, const char *fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_calib_error, sizeof(g_calib_error), fmt, ap);
+  va_end(ap);
+  return code;
+}
+#define LMH_HIP_TRY(expr)                                                                                    \
+  do {                                                                                                       \
+    hipError_t lmh_e_ = (expr);                                                                              \
+    if (lmh_e_ != hipSuccess) return fail(LMH_E_HIP, "HIP error %d (%s) in %s", (int)lmh_e_, hipGetErrorString(lmh_e_), #expr); \
+  } while (0)
+
 typedef _Float16 calib_half8_t __attribute__((ext_vector_type(8)));
 typedef float calib_floatx16_t __attribute__((ext_vector_type(16)));
 constexpr int kCalibMfmaGrid = 512;    // two workgroups per CU
@@ -130,6 +153,8 @@ __global__ __launch_bounds__(256) void calib_read_kernel(const calib_u4_t *__res
 }
 }  // namespace
 }  // namespace lmh
+
+extern "C" const char *lmh_calib_last_error(void) { return lmh::g_calib_error; }
 
 extern "C" int lmh_calib_read(const void *src, size_t bytes, void *sink4, void *stream) {
   using namespace lmh;

@@ -27,6 +27,10 @@
 #include "common.hpp"
 #include "dtypes.hpp"
 
+#if (defined(LMH_FOLD_SCALE) || defined(LMH_ONLY_XCDS) || defined(LMH_WIDE_MARGIN)) && !defined(LMH_MEASUREMENT_BUILD)
+#error "LMH_FOLD_SCALE / LMH_ONLY_XCDS / LMH_WIDE_MARGIN are experiment switches: they need -DLMH_MEASUREMENT_BUILD, which marks the library"
+#endif
+
 namespace lmh {
 namespace {
 

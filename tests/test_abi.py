@@ -9,14 +9,15 @@ import pytest
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
 
-def header_functions():
-    text = open(os.path.join(ROOT, "include", "luminal_hip.h")).read()
+def header_functions(header="luminal_hip.h"):
+    text = open(os.path.join(ROOT, "include", header)).read()
     text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
     return sorted(set(re.findall(r"\b(lmh_[a-z0-9_]+)\s*\(", text)))
 
 
 def test_header_and_binding_list_the_same_symbols(lm):
     assert header_functions() == sorted(lm.binding.EXPORTS)
+    assert header_functions("luminal_hip_calib.h") == sorted(lm.binding.CALIB_EXPORTS)
 
 
 def test_library_exports_every_declared_symbol(lm):
@@ -24,6 +25,33 @@ def test_library_exports_every_declared_symbol(lm):
     for name in header_functions():
         assert hasattr(lib, name), name
     assert lib.lmh_version() == 103
+    calib = lm.binding.load_calib()
+    for name in header_functions("luminal_hip_calib.h"):
+        assert hasattr(calib, name), name
+
+
+def test_measurement_kernels_are_not_in_the_attention_library(lm):
+    """The attention library is the drop-in boundary: it exports nothing but what luminal_hip.h declares for the
+    reference's interfaces, and it is a product build (no experiment switches compiled in)."""
+    lib = lm.binding.load()
+    for name in lm.binding.CALIB_EXPORTS:
+        assert not hasattr(lib, name), name
+    assert lib.lmh_measurement_build() == 0
+
+
+def test_experiment_flags_need_the_measurement_marker(lm, monkeypatch):
+    import importlib.util
+    spec = importlib.util.spec_from_file_location("lmh_build_for_test", os.path.join(ROOT, "luminal.jl_amd", "build.py"))
+    build = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(build)
+    monkeypatch.delenv("LMH_EXTRA_FLAGS", raising=False)
+    monkeypatch.delenv("LMH_MEASUREMENT_BUILD", raising=False)
+    assert build.experiment_flags() == []
+    monkeypatch.setenv("LMH_EXTRA_FLAGS", "-DLMH_FOLD_SCALE")
+    with pytest.raises(RuntimeError, match="LMH_MEASUREMENT_BUILD"):
+        build.experiment_flags()
+    monkeypatch.setenv("LMH_MEASUREMENT_BUILD", "1")
+    assert build.experiment_flags() == ["-DLMH_FOLD_SCALE", "-DLMH_MEASUREMENT_BUILD"]
 
 
 def test_struct_layout_matches_header(lm):
