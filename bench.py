@@ -430,7 +430,50 @@ def ops_leg(lm, dev, res, caches=None):
         rstate["i"] += 1
 
     hbm_line("plain copy of the same 25 MB (reference for the line above)", copy_step, 2.0 * B * H * S * D * 2, n=36)
-    del xs
+
+    # The prompt path of an attention layer on the C2 shape (reference src/NN.jl:357-382: rotary embedding of q and k,
+    # then attention): three launches, against two with the queries rotated inside the attention kernel.
+    q, k = xs[0], xs[1]
+    v = lm.HipArray((B, H, S, D), "f16", dev).copy_from_host(lm.synth.normal((B, H, S, D), 2001, 0.5))
+    qr, kr = lm.HipArray((B, H, S, D), "f16", dev), lm.HipArray((B, H, S, D), "f16", dev)
+    o = lm.HipArray((B, H, S, D), "f16", dev)
+
+    def rope_params(dst, src):
+        rp = lm.binding.RopeParams()
+        rp.out, rp.x, rp.pos0, rp.prev_seq = dst.ptr, src.ptr, None, 0
+        rp.B, rp.H, rp.S, rp.D = B, H, S, D
+        rp.dtype, rp.base, rp.pairing, rp.stream = lm.binding.DTYPE_CODES["f16"], 10000.0, lm.binding.ROPE_HALF_SPLIT, None
+        return rp
+
+    rq, rk = rope_params(qr, q), rope_params(kr, k)
+    plain = attn_params(lm, o, qr, kr, v, "f16", True, lm.default_scale(D))
+    fused = attn_params(lm, o, q, kr, v, "f16", True, lm.default_scale(D))
+    fused.q_rope, fused.q_rope_pairing, fused.q_prev_seq, fused.q_rope_base = 1, lm.binding.ROPE_HALF_SPLIT, 0, 10000.0
+
+    def three_launches():
+        lm.binding.rope(rq)
+        lm.binding.rope(rk)
+        lm.binding.flash_attn_fwd(plain)
+
+    def two_launches():
+        lm.binding.rope(rk)
+        lm.binding.flash_attn_fwd(fused)
+
+    three_launches()
+    lm.binding.sync()
+    want = o.to_host()
+    two_launches()
+    lm.binding.sync()
+    same = bool(np.array_equal(o.to_host(), want))
+    line = {"same_bits_as_three_launches": same}
+    for name, fn in (("attention_alone_us", lambda: lm.binding.flash_attn_fwd(plain)),
+                     ("attention_rotating_q_us", lambda: lm.binding.flash_attn_fwd(fused)),
+                     ("rope_q_rope_k_attention_3_launches_us", three_launches), ("rope_k_attention_rotating_q_2_launches_us", two_launches)):
+        _, ev = time_steps(fn, 20, 5, lm.binding)
+        line[name] = ev * 1e3
+    res["prompt path fp16 B=1 H=32 S=4096 D=96 causal (rotary embedding of q and k + attention)"] = line
+    log("[other] prompt path: %s" % json.dumps(line))
+    del xs, q, k, v, qr, kr, o
 
     caches = caches or c4_caches(lm, dev)
     for T, label in ((4096, "whole prompt T=4096"), (1, "one decode step T=1")):

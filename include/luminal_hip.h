@@ -23,7 +23,7 @@
 extern "C" {
 #endif
 
-#define LMH_VERSION 103 /* major*10000 + minor*100 + patch */
+#define LMH_VERSION 104 /* major*10000 + minor*100 + patch */
 
 /* status codes */
 #define LMH_OK 0
@@ -50,6 +50,12 @@ extern "C" {
  * BLOCKED: hq / (Hq/Hkv) — the row-major (HuggingFace) convention. */
 #define LMH_HEADMAP_INTERLEAVED 0
 #define LMH_HEADMAP_BLOCKED 1
+
+/* which elements of a row the rotary embedding rotates together (lmh_rope, lmh_kv_append, lmh_attn_params.q_rope).
+ * HALF_SPLIT: (j, j + D/2), what the reference's column-major reshape to (D/2, 2) produces
+ *   (reference src/NN.jl:253-303). INTERLEAVED: (2j, 2j+1). */
+#define LMH_ROPE_HALF_SPLIT 0
+#define LMH_ROPE_INTERLEAVED 1
 
 /* ---- runtime plumbing: replaces CUDA.functional()/CuArray()/Array() in the reference's
  * device layer (reference src/Device.jl:31-74 get_device, :82-96 to_device, :103-105
@@ -128,6 +134,18 @@ typedef struct lmh_attn_params {
   int32_t head_map; /* LMH_HEADMAP_* */
   int32_t out_f32;  /* 0: out has element type `dtype`; 1: out is fp32 */
   void *stream;     /* hipStream_t, null = default stream */
+  /* Optional: the rotary embedding of the queries, which the reference applies directly in front of attention
+   * (reference src/NN.jl:357, apply_rotary_embeddings :253-303), done on the rows as the kernel loads them instead of
+   * by a launch of lmh_rope on q: row i of sequence b is rotated at position (q_pos0 ? q_pos0[b] : q_prev_seq) + i and
+   * rounded to `dtype`, exactly what lmh_rope would have stored; q itself is not modified. K is not rotated here
+   * (lmh_kv_append rotates it on its way into a cache, lmh_rope anywhere else). D must be even; head dims 64, 96 and
+   * 128 keep the matrix-core kernels, any other runs on the vector-ALU kernel. Last in the struct so that
+   * zero-initialised params of earlier callers keep their meaning. */
+  int32_t q_rope;         /* 0 / 1 */
+  int32_t q_rope_pairing; /* LMH_ROPE_* */
+  const int32_t *q_pos0;  /* optional device int32[B]: position of row 0 per sequence; null = q_prev_seq */
+  int32_t q_prev_seq;
+  float q_rope_base;      /* 10000 in the reference */
 } lmh_attn_params;
 
 int lmh_flash_attn_fwd(const lmh_attn_params *p);
@@ -195,10 +213,7 @@ int lmh_decode_attn_static(const lmh_decode_params *p);
 /* ---- rotary position embedding: replaces the ~25-node subgraph of
  *   apply_rotary_embeddings(input, prev_seq; base)    reference src/NN.jl:253-303
  * out[b,h,s,:] = rotate(x[b,h,s,:], position = (pos0 ? pos0[b] : prev_seq) + s); out may alias x.
- * pairing LMH_ROPE_HALF_SPLIT rotates (j, j + D/2), which is what the reference's column-major
- * reshape to (D/2, 2) produces; LMH_ROPE_INTERLEAVED rotates (2j, 2j+1). D must be even. ---- */
-#define LMH_ROPE_HALF_SPLIT 0
-#define LMH_ROPE_INTERLEAVED 1
+ * pairing: LMH_ROPE_* (above). D must be even. ---- */
 typedef struct lmh_rope_params {
   void *out;           /* [B,H,S,D] device */
   const void *x;       /* [B,H,S,D] device */

@@ -47,6 +47,8 @@ class AttnParams(ctypes.Structure):
         ("o_stride", ctypes.c_int64 * 3),
         ("dtype", ctypes.c_int32), ("scale", ctypes.c_float), ("causal", ctypes.c_int32),
         ("head_map", ctypes.c_int32), ("out_f32", ctypes.c_int32), ("stream", ctypes.c_void_p),
+        ("q_rope", ctypes.c_int32), ("q_rope_pairing", ctypes.c_int32), ("q_pos0", ctypes.c_void_p),
+        ("q_prev_seq", ctypes.c_int32), ("q_rope_base", ctypes.c_float),
     ]
 
 

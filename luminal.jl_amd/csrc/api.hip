@@ -298,12 +298,23 @@ int lmh_flash_attn_fwd(const lmh_attn_params *p) {
     return fail(LMH_E_UNSUPPORTED, "lmh_flash_attn_fwd: unknown head_map %d", p->head_map);
   if (p->D > 256) return fail(LMH_E_UNSUPPORTED, "lmh_flash_attn_fwd: head dim %d > 256 is not supported", p->D);
   if (!(p->scale == p->scale)) return fail(LMH_E_SHAPE, "lmh_flash_attn_fwd: scale is NaN");
+  if (p->q_rope) {
+    if (p->D % 2 != 0) return fail(LMH_E_SHAPE, "lmh_flash_attn_fwd: head dim %d must be even for the rotary embedding", p->D);
+    if (p->q_rope_pairing != LMH_ROPE_HALF_SPLIT && p->q_rope_pairing != LMH_ROPE_INTERLEAVED)
+      return fail(LMH_E_UNSUPPORTED, "lmh_flash_attn_fwd: unknown q_rope_pairing %d", p->q_rope_pairing);
+    if (!(p->q_rope_base > 0.f)) return fail(LMH_E_SHAPE, "lmh_flash_attn_fwd: q_rope_base must be positive");
+  }
 
   PrefillArgs a;
   a.out = p->out; a.q = p->q; a.k = p->k; a.v = p->v; a.kv_len = p->kv_len;
   a.B = p->B; a.Hq = p->Hq; a.Hkv = p->Hkv; a.Sq = p->Sq; a.Sk = p->Sk; a.D = p->D;
   a.scale = p->scale; a.causal = p->causal ? 1 : 0; a.head_map = p->head_map;
   a.out_f32 = (p->out_f32 != 0 || p->dtype == LMH_F32) ? 1 : 0;
+  a.q_rope = p->q_rope ? 1 : 0;
+  a.q_interleaved = p->q_rope_pairing == LMH_ROPE_INTERLEAVED;
+  a.q_pos0 = p->q_rope ? p->q_pos0 : nullptr;
+  a.q_prev_seq = p->q_prev_seq;
+  a.q_log2_base = p->q_rope ? log2f(p->q_rope_base) : 0.f;
   auto fill = [&](int64_t *dst, const int64_t *src, int64_t H, int64_t S) {
     if (all_zero(src, 3)) {
       dst[0] = H * S * p->D; dst[1] = S * p->D; dst[2] = p->D;
@@ -329,6 +340,7 @@ int lmh_flash_attn_fwd(const lmh_attn_params *p) {
   // (offsets from 0x7ffffff0 up are what the half-precision kernel uses as "out of range")
   constexpr int64_t kMaxSliceBytes = 0x7ffffff0;
   mfma_ok = mfma_ok && (int64_t)p->Sk * a.ks[2] * esz < kMaxSliceBytes && (int64_t)p->Sk * a.vs[2] * esz < kMaxSliceBytes;
+  mfma_ok = mfma_ok && (!p->q_rope || prefill_mfma_rope_ok(p->D));  // the rotation in registers needs a head dim that fills its tiling
   for (int i = 0; i < 3 && mfma_ok; i++)
     mfma_ok = (a.qs[i] % vec == 0) && (a.ks[i] % vec == 0) && (a.vs[i] % vec == 0) && (a.os[i] % vec == 0);
   if (mfma_ok && p->dtype == LMH_F32) return launch_prefill_f32_mfma(a, (hipStream_t)p->stream);

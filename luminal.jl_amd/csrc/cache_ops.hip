@@ -17,38 +17,10 @@
 // the one-element-per-thread kernels.
 #include "common.hpp"
 #include "dtypes.hpp"
+#include "rope.hpp"
 
 namespace lmh {
 namespace {
-
-// sin and cos of an fp32 angle (radians, any magnitude an fp32 position reaches) on the hardware's
-// v_sin_f32 / v_cos_f32, which take revolutions. The library sincosf costs ~100 instructions per angle (its
-// large-argument path alone is a table walk) and made the rotary kernels compute-bound at 46 % of the
-// memory roofline. Here the angle is reduced by whole turns with 2 pi split into its fp32 head and the
-// remainder (two fused multiply-adds: the first is exact up to the rounding of a result no larger than
-// ~pi, whatever the number of turns), so |r| <= pi to ~3e-7 rad, and r / 2 pi goes to the hardware.
-__device__ inline void sincos_angle(float angle, float *sn, float *cs) {
-  constexpr float kInv2Pi = 0.15915493667125702f;
-  constexpr float k2PiHead = 6.2831854820251465f;      // fp32(2 pi)
-  constexpr float k2PiTail = -1.7484555314695172e-07f;  // 2 pi - fp32(2 pi)
-  const float turns = rintf(angle * kInv2Pi);
-  float r = fmaf(-turns, k2PiHead, angle);
-  r = fmaf(-turns, k2PiTail, r);
-  const float x = r * kInv2Pi;
-  *sn = __builtin_amdgcn_sinf(x);
-  *cs = __builtin_amdgcn_cosf(x);
-}
-
-template <typename E>
-__device__ inline void rope_pair(float x0, float x1, float pos, int j, int D, float log2_base, float *o0, float *o1) {
-  // inv_freq = 1 / exp2((2j/D) * log2(base)), evaluated as the reference does (src/NN.jl:262-263)
-  const float freq = (float)j * 2.0f / (float)D;
-  const float inv_freq = 1.0f / exp2f(freq * log2_base);
-  float sn, cs;
-  sincos_angle(pos * inv_freq, &sn, &cs);
-  *o0 = x0 * cs - x1 * sn;
-  *o1 = x0 * sn + x1 * cs;
-}
 
 template <typename E>
 __global__ __launch_bounds__(256) void rope_kernel(RopeArgs a) {
@@ -66,7 +38,7 @@ __global__ __launch_bounds__(256) void rope_kernel(RopeArgs a) {
     const raw *xp = reinterpret_cast<const raw *>(a.x) + b * a.xs[0] + h * a.xs[1] + (int64_t)s * a.xs[2];
     raw *op = reinterpret_cast<raw *>(a.out) + b * a.os[0] + h * a.os[1] + (int64_t)s * a.os[2];
     float o0, o1;
-    rope_pair<E>(E::ld(xp[d0]), E::ld(xp[d1]), pos, j, a.D, a.log2_base, &o0, &o1);
+    rope_pair(E::ld(xp[d0]), E::ld(xp[d1]), pos, j, a.D, a.log2_base, &o0, &o1);
     op[d0] = E::st(o0);
     op[d1] = E::st(o1);
   }
@@ -89,7 +61,7 @@ __global__ __launch_bounds__(256) void kv_append_kernel(KvAppendArgs a) {
       const int d1 = a.interleaved ? 2 * j + 1 : j + half;
       raw *qp = reinterpret_cast<raw *>(a.q) + (bh * a.T + t) * a.D;
       float o0, o1;
-      rope_pair<E>(E::ld(qp[d0]), E::ld(qp[d1]), (float)((a.pos ? a.pos[b] : a.pos_all) + t), j, a.D, a.log2_base, &o0, &o1);
+      rope_pair(E::ld(qp[d0]), E::ld(qp[d1]), (float)((a.pos ? a.pos[b] : a.pos_all) + t), j, a.D, a.log2_base, &o0, &o1);
       qp[d0] = E::st(o0);
       qp[d1] = E::st(o1);
       continue;
@@ -114,7 +86,7 @@ __global__ __launch_bounds__(256) void kv_append_kernel(KvAppendArgs a) {
       const float x0 = E::ld(first ? kn[d] : kn[dp]);
       const float x1 = E::ld(first ? kn[dp] : kn[d]);
       float o0, o1;
-      rope_pair<E>(x0, x1, (float)row, j, a.D, a.log2_base, &o0, &o1);
+      rope_pair(x0, x1, (float)row, j, a.D, a.log2_base, &o0, &o1);
       kc[d] = E::st(first ? o0 : o1);
     }
   }
@@ -132,18 +104,20 @@ template <typename E>
 __device__ inline void rotate_chunks(Chunk<E> &c0, Chunk<E> &c1, const float *sn, const float *cs) {
 #pragma unroll
   for (int i = 0; i < E::kVec; i++) {
-    const float x0 = E::ld(c0.e[i]), x1 = E::ld(c1.e[i]);
-    c0.e[i] = E::st(x0 * cs[i] - x1 * sn[i]);
-    c1.e[i] = E::st(x0 * sn[i] + x1 * cs[i]);
+    float o0, o1;
+    rope_rotate(E::ld(c0.e[i]), E::ld(c1.e[i]), sn[i], cs[i], &o0, &o1);
+    c0.e[i] = E::st(o0);
+    c1.e[i] = E::st(o1);
   }
 }
 template <typename E>
 __device__ inline void rotate_interleaved(Chunk<E> &c, const float *sn, const float *cs) {
 #pragma unroll
   for (int i = 0; i < E::kVec / 2; i++) {
-    const float x0 = E::ld(c.e[2 * i]), x1 = E::ld(c.e[2 * i + 1]);
-    c.e[2 * i] = E::st(x0 * cs[i] - x1 * sn[i]);
-    c.e[2 * i + 1] = E::st(x0 * sn[i] + x1 * cs[i]);
+    float o0, o1;
+    rope_rotate(E::ld(c.e[2 * i]), E::ld(c.e[2 * i + 1]), sn[i], cs[i], &o0, &o1);
+    c.e[2 * i] = E::st(o0);
+    c.e[2 * i + 1] = E::st(o1);
   }
 }
 template <typename E>
@@ -151,9 +125,7 @@ __device__ inline void sincos_pairs(float pos, int j0, int n, int D, float log2_
 #pragma unroll
   for (int i = 0; i < E::kVec; i++) {
     if (i >= n) break;
-    const float freq = (float)(j0 + i) * 2.0f / (float)D;
-    const float inv_freq = 1.0f / exp2f(freq * log2_base);
-    sincos_angle(pos * inv_freq, &sn[i], &cs[i]);
+    sincos_angle(pos * rope_inv_freq(j0 + i, D, log2_base), &sn[i], &cs[i]);
   }
 }
 

@@ -37,6 +37,13 @@ struct PrefillArgs {
   int32_t causal;
   int32_t head_map;
   int32_t out_f32;  // out is fp32 whatever the input element type
+  // Rotary embedding of the query rows on their way into the kernel (q_rope != 0): row i of sequence b is rotated at
+  // position (q_pos0 ? q_pos0[b] : q_prev_seq) + i and rounded to the element type, as lmh_rope would have stored it.
+  int32_t q_rope;
+  int32_t q_interleaved;  // 0: pairs (j, j + D/2) as the reference; 1: pairs (2j, 2j+1)
+  const int32_t *q_pos0;
+  int32_t q_prev_seq;
+  float q_log2_base;
 };
 
 // Decode launch arguments.
@@ -96,6 +103,9 @@ __host__ __device__ inline int q_head_of(int kvh, int g, int Hq, int Hkv, int he
 
 // Launchers: validate nothing (api.hip already did), pick an instantiation, enqueue on `stream`.
 // Return LMH_OK or LMH_E_UNSUPPORTED / LMH_E_HIP.
+// The matrix-core kernels rotate Q in registers, which needs the partner of every element in the same lane: head dims
+// that fill a tiling exactly (64, 96, 128).
+inline bool prefill_mfma_rope_ok(int D) { return D == 64 || D == 96 || D == 128; }
 bool prefill_mfma_supported(int dtype, int D);
 int launch_prefill_mfma(const PrefillArgs &a, int dtype, hipStream_t stream);
 bool prefill_f32_mfma_supported(int dtype, int D);

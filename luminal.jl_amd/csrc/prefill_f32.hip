@@ -19,6 +19,7 @@
 // fp16, so the ~70 vector instructions and ~80 LDS reads per tile hide behind 64-128 MFMAs of 64 cycles.
 #include "common.hpp"
 #include "dtypes.hpp"
+#include "rope.hpp"
 
 namespace lmh {
 namespace {
@@ -161,6 +162,39 @@ __global__ __launch_bounds__(256, (KSPLIT > 1 ? 1 : D <= 96 ? 3 : 2)) void prefi
   const int v_frag_off = 4 * g * LDV + n;  // + (8 * (i / 4) + i % 4) * LDV + 32 * db
 
   if (n_kv_tiles > 0) load_tile(0, 0);
+  // Rotary embedding of the query fragments in registers (PrefillArgs::q_rope; the head dim equals the tiling). Lane
+  // (n, g) holds elements 8 j + 4 g + e: the partner j' + D/2 of element j' is fragment j + D/16 of the same lane, the
+  // interleaved pairs are neighbours. inv_freq is computed once per workgroup into the second K buffer, which nothing
+  // writes before the loop's first barrier.
+  if (a.q_rope) {
+    float *table = &Ks2[1][0];
+    if (tid < D / 2) table[tid] = rope_inv_freq(tid, D, a.q_log2_base);
+    __syncthreads();
+    const float pos = (float)((a.q_pos0 ? a.q_pos0[b] : a.q_prev_seq) + qi);
+    if (!a.q_interleaved) {
+#pragma unroll
+      for (int j = 0; j < KJ / 2; j++)
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+          float sn, cs, o0, o1;
+          sincos_angle(pos * table[8 * j + 4 * g + e], &sn, &cs);
+          rope_rotate(qf[j][e], qf[j + KJ / 2][e], sn, cs, &o0, &o1);
+          qf[j][e] = o0;
+          qf[j + KJ / 2][e] = o1;
+        }
+    } else {
+#pragma unroll
+      for (int j = 0; j < KJ; j++)
+#pragma unroll
+        for (int e = 0; e < 4; e += 2) {
+          float sn, cs, o0, o1;
+          sincos_angle(pos * table[(8 * j + 4 * g + e) / 2], &sn, &cs);
+          rope_rotate(qf[j][e], qf[j][e + 1], sn, cs, &o0, &o1);
+          qf[j][e] = o0;
+          qf[j][e + 1] = o1;
+        }
+    }
+  }
   // The compiler does not model the asm loads or the asm wait below: make it wait for Q here, not inside the loop.
 #pragma unroll
   for (int j = 0; j < KJ; j++) asm volatile("" :: "v"(qf[j]));

@@ -26,6 +26,7 @@
 //     causal, issues the long rows first.
 #include "common.hpp"
 #include "dtypes.hpp"
+#include "rope.hpp"
 
 #if (defined(LMH_FOLD_SCALE) || defined(LMH_ONLY_XCDS) || defined(LMH_WIDE_MARGIN)) && !defined(LMH_MEASUREMENT_BUILD)
 #error "LMH_FOLD_SCALE / LMH_ONLY_XCDS / LMH_WIDE_MARGIN are experiment switches: they need -DLMH_MEASUREMENT_BUILD, which marks the library"
@@ -100,6 +101,43 @@ struct MfmaBF16 {
     return acc;
   }
 };
+
+
+// Rotary embedding of the wave's query fragments in registers (PrefillArgs::q_rope). Lane (n, g) holds elements
+// 16 ks + 8 g + e of its row; with the head dim equal to the tiling, the partner j + D/2 of element j sits in
+// fragment ks + D/32 of the same lane (the interleaved pairs are neighbours inside a fragment). inv_freq does not
+// depend on the row: the workgroup computes its D/2 values once into `table` (LDS that nothing else uses before the
+// next barrier) and every lane multiplies them by its own position. Every thread of the workgroup must call this.
+template <typename MT, int D>
+__device__ inline void rotate_q_fragments(typename MT::vec8 (&qreg)[D / 16], const PrefillArgs &a, int b, int qi, int g, float *table) {
+  constexpr int KS = D / 16, HK = D / 32;
+  if ((int)threadIdx.x < D / 2) table[threadIdx.x] = rope_inv_freq(threadIdx.x, D, a.q_log2_base);
+  __syncthreads();
+  const float pos = (float)((a.q_pos0 ? a.q_pos0[b] : a.q_prev_seq) + qi);
+  if (!a.q_interleaved) {
+#pragma unroll
+    for (int ks = 0; ks < HK; ks++)
+#pragma unroll
+      for (int e = 0; e < 8; e++) {
+        float sn, cs, o0, o1;
+        sincos_angle(pos * table[16 * ks + 8 * g + e], &sn, &cs);
+        rope_rotate((float)qreg[ks][e], (float)qreg[ks + HK][e], sn, cs, &o0, &o1);
+        qreg[ks][e] = MT::cvt(o0);
+        qreg[ks + HK][e] = MT::cvt(o1);
+      }
+  } else {
+#pragma unroll
+    for (int ks = 0; ks < KS; ks++)
+#pragma unroll
+      for (int e = 0; e < 8; e += 2) {
+        float sn, cs, o0, o1;
+        sincos_angle(pos * table[(16 * ks + 8 * g + e) / 2], &sn, &cs);
+        rope_rotate((float)qreg[ks][e], (float)qreg[ks][e + 1], sn, cs, &o0, &o1);
+        qreg[ks][e] = MT::cvt(o0);
+        qreg[ks][e + 1] = MT::cvt(o1);
+      }
+  }
+}
 
 // NW waves per workgroup, 32 query rows each, walking the same 64-key tiles (KSPLIT = 1).
 // NW = 8 (256 query rows) stages every K/V tile once per 256 rows instead of once per 128: 3-8 % faster
@@ -278,6 +316,8 @@ __global__ __launch_bounds__(64 * NW, WPS) void prefill_mfma_kernel(PrefillArgs 
   // + (kb*32 + 16*t [+8]) * LDV + db*32
 
   if (n_kv_tiles > 0) load_tile(0, 0);
+  // (the second K buffer is not written before the loop's first barrier: room for the inv_freq table)
+  if (a.q_rope) rotate_q_fragments<MT, D>(qreg, a, b, qi, g, reinterpret_cast<float *>(&Ks2[1][0]));
   // The compiler does not model the asm loads or the asm wait below. Make it wait for Q here;
   // otherwise it puts its own vmcnt(0) in front of the first MFMA inside the loop, after the
   // prefetch of the next tile has been issued.
@@ -607,6 +647,7 @@ __global__ __launch_bounds__(1024, 4) void prefill_mfma_wide_kernel(PrefillArgs 
   const int v_frag_off = (kg * 32 + 4 * g + (i16 >> 2)) * LDV + 16 * ((lane >> 4) & 1) + 4 * (i16 & 3);
 
   if (n_kv_tiles > 0) load_tile(0, 0);
+  if (a.q_rope) rotate_q_fragments<MT, D>(qreg, a, b, qi, g, reinterpret_cast<float *>(&lds[K_BUF]));
 #pragma unroll
   for (int ks = 0; ks < KS; ks++) asm volatile("" :: "v"(qreg[ks]));
 

@@ -11,6 +11,7 @@
 // and read as float4 (the 16 row-groups of a wave read the same address -> LDS broadcast).
 #include "common.hpp"
 #include "dtypes.hpp"
+#include "rope.hpp"
 
 namespace lmh {
 namespace {
@@ -55,6 +56,10 @@ __global__ __launch_bounds__(256) void prefill_valu_kernel(PrefillArgs a) {
     for (int e = 0; e < 4; e++) {
       int d = (c * 4 + t) * 4 + e;
       tmp[e] = (row_valid && d < D) ? E::ld(qp[d]) : 0.f;
+      // rotary embedding on the way in (PrefillArgs::q_rope), rounded to the element type as lmh_rope stores it
+      if (a.q_rope && row_valid && d < D)
+        tmp[e] = E::ld(E::st(rope_element(qp, d, D, (float)((a.q_pos0 ? a.q_pos0[b] : a.q_prev_seq) + qi), a.q_log2_base,
+                                          a.q_interleaved != 0, [](raw x) { return E::ld(x); })));
     }
     qf[c] = make_float4(tmp[0], tmp[1], tmp[2], tmp[3]);
     of[c] = make_float4(0.f, 0.f, 0.f, 0.f);

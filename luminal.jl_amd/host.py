@@ -217,13 +217,24 @@ class InputTensor(Op):
 
 
 class FlashAttentionOp(Op):
-    """Fused flash attention node (reference src/Ops.jl:104-107), plus the GQA head map."""
+    """Fused flash attention node (reference src/Ops.jl:104-107), plus the GQA head map. Inputs (q, k, v), then
+    optionally kv_len (int32[B], `has_kv_len`) and q_pos0 (int32[B], `has_q_pos0`). With `q_rope_base` the kernel
+    rotates the query rows as it loads them (apply_rotary_embeddings on the queries, reference src/NN.jl:357, without
+    a launch of its own): row i of sequence b at position (q_pos0 ? q_pos0[b] : q_prev_seq) + i."""
 
-    def __init__(self, scale, causal, head_map=HEADMAP_INTERLEAVED, out_dtype=None):
+    def __init__(self, scale, causal, head_map=HEADMAP_INTERLEAVED, out_dtype=None, has_kv_len=False,
+                 q_rope_base=None, q_prev_seq=0, q_rope_interleaved=False, has_q_pos0=False):
         self.scale = float(np.float32(scale))
         self.causal = bool(causal)
         self.head_map = head_map
         self.out_dtype = out_dtype  # None = q's element type; "f32" = full-precision result
+        self.has_kv_len = bool(has_kv_len)
+        self.q_rope_base = None if q_rope_base is None else float(q_rope_base)
+        self.q_prev_seq = int(q_prev_seq)
+        self.q_rope_interleaved = bool(q_rope_interleaved)
+        self.has_q_pos0 = bool(has_q_pos0)
+        if self.has_q_pos0 and self.q_rope_base is None:
+            raise ValueError("q_pos0 is the position input of the rotary embedding: give q_rope_base as well")
 
 
 class DecodeAttentionOp(Op):
@@ -295,14 +306,23 @@ def tensor(graph, shape, dtype="f32"):
     return add_op(graph, InputTensor(), [], tuple(shape), dtype)
 
 
-def flash_attention(q, k, v, scale=None, causal=False, head_map=HEADMAP_INTERLEAVED, out_dtype=None):
+def flash_attention(q, k, v, scale=None, causal=False, head_map=HEADMAP_INTERLEAVED, out_dtype=None, kv_len=None,
+                    q_rope_base=None, q_prev_seq=0, q_pos0=None, q_rope_interleaved=False):
     """q, k, v: (Batch, Head, Seq, HeadDim). Output has q's shape; scale defaults to 1/sqrt(D)
-    computed in fp32 (reference src/HighLevelOps.jl:377-388)."""
+    computed in fp32 (reference src/HighLevelOps.jl:377-388). kv_len (int32[B] tensor) limits sequence b to its
+    first kv_len[b] keys; q_rope_base asks for the rotary embedding of the queries inside the kernel, at positions
+    q_prev_seq + i or q_pos0[b] + i (q_pos0 an int32[B] tensor)."""
     if scale is None:
         scale = np.float32(1.0) / np.sqrt(np.float32(q.shape[-1]))
     inputs = [(q.id, q.index, q.shape), (k.id, k.index, k.shape), (v.id, v.index, v.shape)]
-    return add_op(q.graph_ref, FlashAttentionOp(np.float32(scale), causal, head_map, out_dtype), inputs, q.shape,
-                  out_dtype or q.graph_ref.dtypes[q.id])
+    if kv_len is not None:
+        inputs.append((kv_len.id, kv_len.index, kv_len.shape))
+    if q_pos0 is not None:
+        inputs.append((q_pos0.id, q_pos0.index, q_pos0.shape))
+    op = FlashAttentionOp(np.float32(scale), causal, head_map, out_dtype, has_kv_len=kv_len is not None,
+                          q_rope_base=q_rope_base, q_prev_seq=q_prev_seq, q_rope_interleaved=q_rope_interleaved,
+                          has_q_pos0=q_pos0 is not None)
+    return add_op(q.graph_ref, op, inputs, q.shape, out_dtype or q.graph_ref.dtypes[q.id])
 
 
 def decode_attention(q, k_cache, v_cache, kv_len, scale=None, head_map=HEADMAP_INTERLEAVED, num_splits=0,
@@ -349,10 +369,39 @@ def self_attention_core(q, k, v, causal=True, prev_seq=0, rope_base=None, scale=
     node that reads the Hkv key/value heads directly (`head_map` INTERLEAVED is the head order repeat_kv produces,
     src/NN.jl:305-317) instead of materialising G copies. rope_base=None skips the rotary embedding (Whisper's
     attention layers, reference src/Whisper.jl:263-272 and :310-312, with causal=False for cross attention)."""
-    if rope_base is not None:
+    if rope_base is None:
+        return flash_attention(q, k, v, scale=scale, causal=causal, head_map=head_map, out_dtype=out_dtype)
+    k = rotary_embedding(k, prev_seq, rope_base)
+    if q.shape[-1] not in FUSED_ROPE_HEAD_DIMS:  # the vector-ALU kernel would serve the fused form: keep the rotary node
         q = rotary_embedding(q, prev_seq, rope_base)
-        k = rotary_embedding(k, prev_seq, rope_base)
-    return flash_attention(q, k, v, scale=scale, causal=causal, head_map=head_map, out_dtype=out_dtype)
+        return flash_attention(q, k, v, scale=scale, causal=causal, head_map=head_map, out_dtype=out_dtype)
+    # the queries are rotated inside the attention kernel: no node (and no launch) of their own
+    return flash_attention(q, k, v, scale=scale, causal=causal, head_map=head_map, out_dtype=out_dtype,
+                           q_rope_base=rope_base, q_prev_seq=prev_seq)
+
+
+# head dims for which the matrix-core attention kernels rotate the queries in registers
+FUSED_ROPE_HEAD_DIMS = (64, 96, 128)
+
+
+def prompt_self_attention_core(q, k_new, v_new, k_cache, v_cache, pos, kv_len, rope_base=None, scale=None,
+                               head_map=HEADMAP_INTERLEAVED, out_dtype=None):
+    """The prompt pass of a cached attention layer as two fused nodes (the reference runs SelfAttention on the prompt,
+    src/NN.jl:352-382, and fills its caches by slice + concat, src/Whisper.jl:552-570): q (B,Hq,T,D) and k_new, v_new
+    (B,Hkv,T,D) are the prompt's projections; the append node writes rows pos[b] .. pos[b]+T-1 of the caches with K
+    rotated on the way in, the attention node reads the caches' first kv_len[b] rows and rotates the queries as it
+    loads them. The causal mask aligns query row i with cache row i, so the prompt must start its cache: pos[b] = 0
+    and kv_len[b] = T (later chunks of a prompt are out of scope). Returns (out (B,Hq,T,D), k_cache, v_cache)."""
+    if rope_base is not None:
+        k_cache, v_cache = kv_cache_append(k_cache, v_cache, k_new, v_new, pos, rope_k=True, base=rope_base)
+    else:
+        k_cache, v_cache = kv_cache_append(k_cache, v_cache, k_new, v_new, pos)
+    fused = rope_base is not None and q.shape[-1] in FUSED_ROPE_HEAD_DIMS
+    if rope_base is not None and not fused:
+        q = rotary_embedding(q, 0, rope_base, pos0=pos)
+    out = flash_attention(q, k_cache, v_cache, scale=scale, causal=True, head_map=head_map, out_dtype=out_dtype,
+                          kv_len=kv_len, q_rope_base=rope_base if fused else None, q_pos0=pos if fused else None)
+    return out, k_cache, v_cache
 
 
 def cached_self_attention_core(q, k_new, v_new, k_cache, v_cache, pos, kv_len, rope_base=None, scale=None,
@@ -425,7 +474,15 @@ def execute_op_inplace(out, op, *inputs, stream=None, workspaces=None):
     is where decode attention takes its split-KV scratch from (default: one buffer shared by all eager calls)."""
     if isinstance(op, FlashAttentionOp):
         q, k, v = inputs[:3]
-        kv_len = inputs[3] if len(inputs) > 3 else None
+        rest = list(inputs[3:])
+        if not (op.has_kv_len or op.has_q_pos0) and len(rest) == 1:  # eager callers pass kv_len as a fourth array
+            kv_len, q_pos0 = rest[0], None
+        else:
+            if len(rest) != int(op.has_kv_len) + int(op.has_q_pos0):
+                raise ValueError("FlashAttentionOp takes (q, k, v%s%s); got %d inputs" %
+                                 (", kv_len" if op.has_kv_len else "", ", q_pos0" if op.has_q_pos0 else "", len(inputs)))
+            kv_len = rest.pop(0) if op.has_kv_len else None
+            q_pos0 = rest.pop(0) if op.has_q_pos0 else None
         _require_hip(out, q, k, v)
         if len(q.shape) != 4 or len(k.shape) != 4 or k.shape != v.shape:
             raise ValueError("flash attention expects q (B,H,S,D) and k, v (B,Hkv,Sk,D); got %s %s %s" %
@@ -445,6 +502,12 @@ def execute_op_inplace(out, op, *inputs, stream=None, workspaces=None):
         p.scale, p.causal, p.head_map = op.scale, int(op.causal), op.head_map
         p.out_f32 = int(out.dtype == "f32")
         p.stream = stream
+        if op.q_rope_base is not None:
+            p.q_rope = 1
+            p.q_rope_pairing = binding.ROPE_INTERLEAVED if op.q_rope_interleaved else binding.ROPE_HALF_SPLIT
+            p.q_pos0 = q_pos0.ptr if q_pos0 is not None else None
+            p.q_prev_seq = op.q_prev_seq
+            p.q_rope_base = op.q_rope_base
         binding.flash_attn_fwd(p)
         return out
     if isinstance(op, DecodeAttentionOp):
@@ -748,7 +811,7 @@ __all__ = [
     "AbstractDevice", "CPUDevice", "HIPDevice", "HipArray", "get_device", "to_device", "from_device", "Graph",
     "GraphTensor", "tensor", "add_op", "FlashAttentionOp", "DecodeAttentionOp", "flash_attention", "decode_attention",
     "RotaryEmbeddingOp", "KVAppendOp", "rotary_embedding", "kv_cache_append", "self_attention_core",
-    "cached_self_attention_core", "execute_op", "execute_op_inplace", "execute", "compile", "CompiledGraph", "execute_with_capture", "release_capture", "HEADMAP_INTERLEAVED",
+    "cached_self_attention_core", "prompt_self_attention_core", "FUSED_ROPE_HEAD_DIMS", "execute_op", "execute_op_inplace", "execute", "compile", "CompiledGraph", "execute_with_capture", "release_capture", "HEADMAP_INTERLEAVED",
     "HEADMAP_BLOCKED", "LuminalHipError", "apply_rotary_embeddings", "kv_append", "KVCacheState", "encode", "decode", "f32_to_bf16_bits", "bf16_bits_to_f32", "default_scale",
     "flash_attention_plan",
 ]

@@ -179,7 +179,10 @@ struct AttnParams
     q_stride::NTuple{3,Int64}; k_stride::NTuple{3,Int64}; v_stride::NTuple{3,Int64}; o_stride::NTuple{3,Int64}
     dtype::Int32; scale::Float32; causal::Int32; head_map::Int32; out_f32::Int32
     stream::Ptr{Cvoid}
+    q_rope::Int32; q_rope_pairing::Int32; q_pos0::Ptr{Int32}; q_prev_seq::Int32; q_rope_base::Float32
 end
+# the trailing fields of AttnParams for "no rotary embedding of the queries"
+const NO_Q_ROPE = (Int32(0), Int32(0), Ptr{Int32}(C_NULL), Int32(0), 0.0f0)
 
 struct DecodeParams
     out::Ptr{Cvoid}; q::Ptr{Cvoid}; k_cache::Ptr{Cvoid}; v_cache::Ptr{Cvoid}; kv_len::Ptr{Int32}
@@ -201,12 +204,20 @@ const Z2 = (Int64(0), Int64(0))
 # FlashAttentionOp on device arrays
 # ------------------------------------------------------------------------------------------
 function execute_op!(out::HipArray{TO,4}, op::FlashAttentionOp, q::HipArray{T,4}, k::HipArray{T,4}, v::HipArray{T,4};
-                     head_map::Int32=HEADMAP_INTERLEAVED) where {TO,T}
+                     head_map::Int32=HEADMAP_INTERLEAVED, kv_len::Union{Nothing,HipArray{Int32,1}}=nothing,
+                     q_rope_base=nothing, q_prev_seq::Integer=0,
+                     q_pos0::Union{Nothing,HipArray{Int32,1}}=nothing) where {TO,T}
     B, Hq, Sq, D = size(q)
     _, Hkv, Sk, _ = size(k)
     size(out) == size(q) || error("FlashAttentionOp: output shape $(size(out)) differs from q shape $(size(q))")
-    p = Ref(AttnParams(out.ptr, q.ptr, k.ptr, v.ptr, C_NULL, B, Hq, Hkv, Sq, Sk, D, Z3, Z3, Z3, Z3,
-                       dtype_code(T), op.scale, Int32(op.causal), head_map, Int32(TO === Float32 && T !== Float32), current_stream()))
+    # q_rope_base: the kernel rotates the query rows as it loads them (apply_rotary_embeddings on the queries,
+    # src/NN.jl:357), row i of sequence b at position (q_pos0 === nothing ? q_prev_seq : q_pos0[b]) + i
+    rope = q_rope_base === nothing ? NO_Q_ROPE :
+           (Int32(1), Int32(0), q_pos0 === nothing ? Ptr{Int32}(C_NULL) : Ptr{Int32}(q_pos0.ptr), Int32(q_prev_seq), Float32(q_rope_base))
+    p = Ref(AttnParams(out.ptr, q.ptr, k.ptr, v.ptr, kv_len === nothing ? Ptr{Int32}(C_NULL) : Ptr{Int32}(kv_len.ptr),
+                       B, Hq, Hkv, Sq, Sk, D, Z3, Z3, Z3, Z3,
+                       dtype_code(T), op.scale, Int32(op.causal), head_map, Int32(TO === Float32 && T !== Float32), current_stream(),
+                       rope...))
     check(ccall((:lmh_flash_attn_fwd, libluminal_hip), Cint, (Ref{AttnParams},), p))
     return out
 end
@@ -221,7 +232,7 @@ function flash_attention_plan(op::FlashAttentionOp, q::HipArray{T,4}, k::HipArra
     B, Hq, Sq, D = size(q)
     _, Hkv, Sk, _ = size(k)
     p = Ref(AttnParams(q.ptr, q.ptr, k.ptr, v.ptr, C_NULL, B, Hq, Hkv, Sq, Sk, D, Z3, Z3, Z3, Z3,
-                       dtype_code(T), op.scale, Int32(op.causal), head_map, Int32(0), C_NULL))
+                       dtype_code(T), op.scale, Int32(op.causal), head_map, Int32(0), C_NULL, NO_Q_ROPE...))
     text = Vector{UInt8}(undef, 256)
     check(ccall((:lmh_flash_attn_plan, libluminal_hip), Cint, (Ref{AttnParams}, Ptr{UInt8}, Csize_t), p, text, length(text)))
     return GC.@preserve text unsafe_string(pointer(text))
@@ -417,15 +428,38 @@ execute_op(op::KVAppendOp, kc::HipArray, rest::HipArray...) = execute_op!(kc, op
 # (src/NN.jl:305-317). Whisper's layers (src/Whisper.jl:263-272, :310-312) are the same call without
 # rotary embedding, cross attention with causal=false.
 # ------------------------------------------------------------------------------------------
+# head dims for which the matrix-core attention kernels rotate the queries in registers
+const FUSED_ROPE_HEAD_DIMS = (64, 96, 128)
+
 function self_attention_core!(out::HipArray, q::HipArray{T,4}, k::HipArray{T,4}, v::HipArray{T,4}; causal::Bool=true,
                               prev_seq::Integer=0, rope_base=nothing, scale=nothing,
                               head_map::Int32=HEADMAP_INTERLEAVED) where {T}
-    if rope_base !== nothing
-        rope!(q; prev_seq=prev_seq, base=rope_base)
-        rope!(k; prev_seq=prev_seq, base=rope_base)
-    end
     s = isnothing(scale) ? 1.0f0 / sqrt(Float32(size(q, 4))) : Float32(scale)
+    rope_base === nothing && return execute_op!(out, FlashAttentionOp(s, causal), q, k, v; head_map=head_map)
+    rope!(k; prev_seq=prev_seq, base=rope_base)
+    if size(q, 4) in FUSED_ROPE_HEAD_DIMS   # q is rotated inside the attention kernel: no launch (and no write) of its own
+        return execute_op!(out, FlashAttentionOp(s, causal), q, k, v; head_map=head_map, q_rope_base=rope_base, q_prev_seq=prev_seq)
+    end
+    rope!(q; prev_seq=prev_seq, base=rope_base)
     return execute_op!(out, FlashAttentionOp(s, causal), q, k, v; head_map=head_map)
+end
+
+"""
+The prompt pass of a cached attention layer in two launches (the reference runs SelfAttention on the prompt,
+src/NN.jl:352-382, and fills its caches by slice + concat, src/Whisper.jl:552-570): the prompt's K/V rows go into the
+caches at rows pos[b] .. (K rotated on the way in), then attention reads the caches' first kv_len[b] rows and rotates
+the queries as it loads them. The causal mask aligns query row i with cache row i: the prompt starts its cache
+(pos[b] = 0, kv_len[b] = T).
+"""
+function prompt_self_attention_core!(out::HipArray, q::HipArray{T,4}, k_new::HipArray{T,4}, v_new::HipArray{T,4},
+                                     kc::HipArray{T,4}, vc::HipArray{T,4}, pos::HipArray{Int32,1}, kv_len::HipArray{Int32,1};
+                                     rope_base=nothing, scale=nothing, head_map::Int32=HEADMAP_INTERLEAVED) where {T}
+    kv_append!(kc, vc, k_new, v_new, pos; rope_k=(rope_base !== nothing), base=something(rope_base, 10000.0f0))
+    s = isnothing(scale) ? 1.0f0 / sqrt(Float32(size(q, 4))) : Float32(scale)
+    fused = rope_base !== nothing && size(q, 4) in FUSED_ROPE_HEAD_DIMS
+    rope_base !== nothing && !fused && rope!(q; base=rope_base, pos0=pos)
+    return execute_op!(out, FlashAttentionOp(s, true), q, kc, vc; head_map=head_map, kv_len=kv_len,
+                       q_rope_base=(fused ? rope_base : nothing), q_pos0=(fused ? pos : nothing))
 end
 
 """
@@ -450,13 +484,41 @@ end
 # The same two cores as graph builders (GraphTensor in, GraphTensor out), for model code that builds a Luminal graph.
 function self_attention_core(q::GraphTensor, k::GraphTensor, v::GraphTensor; causal::Bool=true, prev_seq::Integer=0,
                              rope_base=nothing, scale=nothing)
-    if rope_base !== nothing
-        q = rotary_embedding(q; prev_seq=prev_seq, base=rope_base)
-        k = rotary_embedding(k; prev_seq=prev_seq, base=rope_base)
-    end
     # FlashAttentionOp reads the Hkv key/value heads in the order repeat_kv produces (src/NN.jl:305-317)
+    rope_base === nothing && return Luminal.flash_attention(q, k, v; scale=scale, causal=causal)
+    k = rotary_embedding(k; prev_seq=prev_seq, base=rope_base)
+    D = Int(eval_dim(realized_dims(q.shape)[end]))
+    if D in FUSED_ROPE_HEAD_DIMS
+        return rope_flash_attention(q, k, v; scale=scale, causal=causal, prev_seq=prev_seq, base=rope_base)
+    end
+    q = rotary_embedding(q; prev_seq=prev_seq, base=rope_base)
     return Luminal.flash_attention(q, k, v; scale=scale, causal=causal)
 end
+
+"""
+FlashAttentionOp whose queries are rotated inside the kernel: the reference's op carries (scale, causal) only
+(src/Ops.jl:104-107), so the fused form is a node type of the glue. Inputs (q, k, v) like FlashAttentionOp.
+"""
+struct RopeFlashAttentionOp <: Op
+    scale::Float32
+    causal::Bool
+    prev_seq::Int32
+    base::Float32
+end
+
+function rope_flash_attention(q::GraphTensor, k::GraphTensor, v::GraphTensor; scale=nothing, causal::Bool=false,
+                              prev_seq::Integer=0, base::Real=10000.0f0)
+    if isnothing(scale)
+        scale = 1.0f0 / sqrt(Float32(eval_dim(realized_dims(q.shape)[end])))   # src/HighLevelOps.jl:378-381
+    end
+    inputs = [(q.id, 0, q.shape), (k.id, 0, k.shape), (v.id, 0, v.shape)]
+    return add_op!(q.graph_ref, RopeFlashAttentionOp(Float32(scale), causal, Int32(prev_seq), Float32(base)), inputs, q.shape)
+end
+
+function execute_op!(out::HipArray{TO,4}, op::RopeFlashAttentionOp, q::HipArray{T,4}, k::HipArray{T,4}, v::HipArray{T,4}) where {TO,T}
+    return execute_op!(out, FlashAttentionOp(op.scale, op.causal), q, k, v; q_rope_base=op.base, q_prev_seq=op.prev_seq)
+end
+execute_op(op::RopeFlashAttentionOp, q::HipArray, k::HipArray, v::HipArray) = execute_op!(similar(q), op, q, k, v)
 
 "Returns (out, k_cache): `out` has q's shape (B,Hq,1,D); `k_cache` is the append node (the updated cache)."
 function cached_self_attention_core(q::GraphTensor, k_new::GraphTensor, v_new::GraphTensor, k_cache::GraphTensor,
@@ -480,7 +542,7 @@ end
 #            lengths default to Int32) and, optionally, for op nodes (default: the type of their first
 #            input; Float32 on a half-precision attention node asks for the fp32 result).
 # ------------------------------------------------------------------------------------------
-const DeviceOp = Union{FlashAttentionOp,DecodeAttentionOp,RotaryEmbeddingOp,KVAppendOp}
+const DeviceOp = Union{FlashAttentionOp,RopeFlashAttentionOp,DecodeAttentionOp,RotaryEmbeddingOp,KVAppendOp}
 is_input_node(op) = op isa Luminal.Function && op.name == "InputTensor"
 
 function compile_hip(graph::Luminal.Graph; eltypes::AbstractDict=Dict{Int,DataType}())
@@ -596,6 +658,7 @@ end
 
 export HIPDevice, HipArray, BF16Bits, release_capture!, enable_capture!, compile_hip, DecodeAttentionOp, decode_attention,
        RotaryEmbeddingOp, rotary_embedding, KVAppendOp, kv_cache_append, get_device, functional, rope!, kv_append!,
-       self_attention_core!, cached_self_attention_core!, self_attention_core, cached_self_attention_core, flash_attention_plan
+       self_attention_core!, cached_self_attention_core!, self_attention_core, cached_self_attention_core, flash_attention_plan,
+       RopeFlashAttentionOp, rope_flash_attention, prompt_self_attention_core!
 
 end # module

@@ -164,17 +164,18 @@ def test_glue_graph_nodes_have_builders_and_executors():
     # a builder that calls add_op!, an in-place executor and an allocating one; compile_hip knows all four ops
     text = glue_text()
     for op, builder in (("DecodeAttentionOp", "decode_attention"), ("RotaryEmbeddingOp", "rotary_embedding"),
-                        ("KVAppendOp", "kv_cache_append")):
+                        ("KVAppendOp", "kv_cache_append"), ("RopeFlashAttentionOp", "rope_flash_attention")):
         assert re.search(r"^struct %s <: Op$" % op, text, flags=re.M), op
         body = re.search(r"^function %s\(.*?^end$" % builder, text, flags=re.M | re.S)
         assert body and "add_op!(" in body.group(0) and op + "(" in body.group(0), builder
         assert re.search(r"^function execute_op!\(out::HipArray\{\w+,\d\}, op::%s," % op, text, flags=re.M), op
         assert re.search(r"^execute_op\(op::%s, " % op, text, flags=re.M), op
-    assert re.search(r"^const DeviceOp = Union\{FlashAttentionOp,DecodeAttentionOp,RotaryEmbeddingOp,KVAppendOp\}$", text,
-                     flags=re.M)
+    assert re.search(r"^const DeviceOp = Union\{FlashAttentionOp,RopeFlashAttentionOp,DecodeAttentionOp,RotaryEmbeddingOp,KVAppendOp\}$",
+                     text, flags=re.M)
     exported = re.search(r"^export (.*?)\n\n", text, flags=re.M | re.S).group(1)
     for name in ("compile_hip", "HipArray", "HIPDevice", "rotary_embedding", "kv_cache_append", "decode_attention",
-                 "cached_self_attention_core", "self_attention_core", "enable_capture!"):
+                 "cached_self_attention_core", "self_attention_core", "enable_capture!", "rope_flash_attention",
+                 "prompt_self_attention_core!"):
         assert name in re.split(r"[,\s]+", exported), name
 
 

@@ -109,9 +109,35 @@ def test_self_attention_core_without_rope_is_one_flash_node(lm):
     assert len(g.nodes) == n + 1 and isinstance(g.nodes[out.id].op, lm.FlashAttentionOp)
     assert g.nodes[out.id].op.causal is False and out.shape == q.shape
     out2 = lm.self_attention_core(q, k, v, causal=True, prev_seq=3, rope_base=10000.0)
+    # head dim 64: K gets a rotary node, the queries are rotated inside the attention kernel
     kinds = [type(x.op).__name__ for x in g.nodes[n + 1:]]
-    assert kinds == ["RotaryEmbeddingOp", "RotaryEmbeddingOp", "FlashAttentionOp"]
-    assert g.nodes[n + 1].op.prev_seq == 3 and g.nodes[out2.id].op.causal is True
+    assert kinds == ["RotaryEmbeddingOp", "FlashAttentionOp"]
+    assert g.nodes[n + 1].op.prev_seq == 3 and g.nodes[n + 1].inputs[0][0] == k.id
+    att = g.nodes[out2.id].op
+    assert att.causal is True and att.q_rope_base == 10000.0 and att.q_prev_seq == 3 and not att.has_q_pos0
+    # a head dim the kernels do not rotate in registers keeps both rotary nodes
+    g3 = lm.Graph()
+    q3, k3, v3 = (lm.tensor(g3, (1, 4, 32, 80), "f16") for _ in range(3))
+    out3 = lm.self_attention_core(q3, k3, v3, rope_base=10000.0)
+    kinds = [type(x.op).__name__ for x in g3.nodes[3:]]
+    assert kinds == ["RotaryEmbeddingOp", "RotaryEmbeddingOp", "FlashAttentionOp"] and g3.nodes[out3.id].op.q_rope_base is None
+
+
+def test_prompt_core_is_append_plus_attention_over_the_cache(lm):
+    g = lm.Graph()
+    B, Hq, Hkv, T, D, Lmax = 2, 8, 2, 16, 128, 64
+    q, kn, vn = lm.tensor(g, (B, Hq, T, D), "bf16"), lm.tensor(g, (B, Hkv, T, D), "bf16"), lm.tensor(g, (B, Hkv, T, D), "bf16")
+    kc, vc = lm.tensor(g, (B, Hkv, Lmax, D), "bf16"), lm.tensor(g, (B, Hkv, Lmax, D), "bf16")
+    pos, kv_len = lm.tensor(g, (B,), "i32"), lm.tensor(g, (B,), "i32")
+    n = len(g.nodes)
+    out, kc2, vc2 = lm.prompt_self_attention_core(q, kn, vn, kc, vc, pos, kv_len, rope_base=10000.0)
+    app, att = g.nodes[n:]
+    assert isinstance(app.op, lm.KVAppendOp) and app.op.rope_k and not app.op.rope_q
+    assert isinstance(att.op, lm.FlashAttentionOp) and att.op.causal and att.op.has_kv_len and att.op.has_q_pos0
+    assert [r[0] for r in att.inputs] == [q.id, kc2.id, kc2.id, kv_len.id, pos.id] and att.inputs[2][1] == 1
+    assert out.shape == q.shape
+    with pytest.raises(ValueError):
+        lm.FlashAttentionOp(0.1, True, has_q_pos0=True)  # positions without a rotary base
 
 
 def test_execute_with_capture_without_a_hip_device_just_runs(lm):
