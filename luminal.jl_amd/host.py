@@ -16,8 +16,15 @@ Additions the reference has only as un-fused subgraphs:
   DecodeAttentionOp / decode_attention           reference src/Whisper.jl:584-620, :628-645
   GQA (Hkv < Hq) inside the fused ops            reference src/NN.jl:305-317, :362-366
 
+Around the attention path, a model graph also holds the nodes of the layer that calls it (projections, reshapes,
+permutes: reference src/NN.jl:343-361, :383-386). Those have no kernel here; they run through a host fallback
+(HostOp: download the inputs, the reference's CPU semantics in numpy, upload the result), so that a whole
+attention layer executes on a HIPDevice with attention itself on the GPU:
+  MatMul, Permute, Reshape, Add, Expand          reference src/Execution.jl:216-250, src/HighLevelOps.jl:173-266
+  Linear, SelfAttention                          reference src/NN.jl:11-38, :319-387
+
 Arrays here are row-major [B, H, S, D] (numpy order), which is the layout the C ABI takes. There
-is no CPU execution path in this backend: running an attention op on host arrays raises.
+is no CPU execution path for the attention ops: running one on host arrays raises.
 """
 import ctypes
 import math
@@ -270,6 +277,65 @@ class KVAppendOp(Op):
         self.rope_q = bool(rope_q)
 
 
+class HostOp(Op):
+    """A node of the reference's graph that has no kernel in libluminal_hip.so. On a HIPDevice it runs through the host:
+    inputs are downloaded, `compute` applies the reference's CPU semantics in fp32 numpy (reference
+    src/Execution.jl:216-250), the result is uploaded in `out_dtype`. The logical meaning is the reference's; where
+    that depends on Julia's column-major element order (Reshape) the numpy form says so."""
+    out_dtype = "f32"
+
+    def compute(self, *arrays):
+        raise NotImplementedError
+
+
+class MatMulOp(HostOp):
+    """MatMul (reference src/Execution.jl:12-90 batch_matmul): (..., M, K) x (K, N) or x (..., K, N)."""
+
+    def compute(self, a, b):
+        if a.shape[-1] != b.shape[-2]:
+            raise ValueError("Matmul dimension mismatch: A is %s, B is %s" % (a.shape, b.shape))
+        return np.matmul(a, b)
+
+
+class PermuteOp(HostOp):
+    """Permute(dims) = permutedims (reference src/Execution.jl:229); dims are 0-based here."""
+
+    def __init__(self, dims):
+        self.dims = tuple(int(d) for d in dims)
+
+    def compute(self, a):
+        return np.transpose(a, self.dims)
+
+
+class ReshapeOp(HostOp):
+    """Reshape(shape) = Base.reshape on a column-major array (reference src/Execution.jl:228): the elements keep
+    their column-major order, which in numpy is order='F'. Splitting hidden into (heads, head_dim) this way makes the
+    head index the fast one: hidden index = head + n_heads * d (reference src/NN.jl:347)."""
+
+    def __init__(self, shape):
+        self.shape = tuple(int(d) for d in shape)
+
+    def compute(self, a):
+        return np.reshape(a, self.shape, order="F")
+
+
+class AddOp(HostOp):
+    """Add with the lower-rank operand given leading singleton axes (reference src/Execution.jl:207-216)."""
+
+    def compute(self, a, b):
+        return a + b
+
+
+class ExpandOp(HostOp):
+    """Expand(dim, size): a new axis at `dim` (0-based), repeated `size` times (reference src/Execution.jl:238-248)."""
+
+    def __init__(self, dim, size):
+        self.dim, self.size = int(dim), int(size)
+
+    def compute(self, a):
+        return np.repeat(np.expand_dims(a, self.dim), self.size, axis=self.dim)
+
+
 class Node:
     def __init__(self, op, inputs):
         self.op = op
@@ -304,6 +370,91 @@ def tensor(graph, shape, dtype="f32"):
     if isinstance(shape, np.ndarray):
         shape = shape.shape
     return add_op(graph, InputTensor(), [], tuple(shape), dtype)
+
+
+def _host_node(op, inputs, shape, dtype):
+    op.out_dtype = dtype
+    g = inputs[0].graph_ref
+    return add_op(g, op, [(t.id, t.index, t.shape) for t in inputs], shape, dtype)
+
+
+def matmul(a, b, dtype="f32"):
+    """(..., M, K) * (..., K, N) -> (..., M, N) (reference src/HighLevelOps.jl:252-266)."""
+    if len(a.shape) < 2 or len(b.shape) < 2:
+        raise ValueError("Matmul inputs must be at least 2D")
+    return _host_node(MatMulOp(), [a, b], tuple(a.shape[:-1]) + (b.shape[-1],), dtype)
+
+
+def permute(a, dims, dtype=None):
+    """reference src/HighLevelOps.jl:183-192; dims 0-based."""
+    return _host_node(PermuteOp(dims), [a], tuple(a.shape[d] for d in dims), dtype or a.graph_ref.dtypes[a.id])
+
+
+def reshape(a, new_shape, dtype=None):
+    """reference src/HighLevelOps.jl:173-181: column-major element order, see ReshapeOp."""
+    if int(np.prod(new_shape, dtype=np.int64)) != int(np.prod(a.shape, dtype=np.int64)):
+        raise ValueError("reshape: %s does not hold the elements of %s" % (tuple(new_shape), a.shape))
+    return _host_node(ReshapeOp(new_shape), [a], tuple(new_shape), dtype or a.graph_ref.dtypes[a.id])
+
+
+def add(a, b):
+    shape = np.broadcast_shapes(a.shape, b.shape)
+    return _host_node(AddOp(), [a, b], tuple(shape), "f32")
+
+
+def expand(a, dim, size):
+    """reference src/HighLevelOps.jl:194-200; dim 0-based."""
+    shape = list(a.shape)
+    shape.insert(dim, size)
+    return _host_node(ExpandOp(dim, size), [a], tuple(shape), a.graph_ref.dtypes[a.id])
+
+
+class Linear:
+    """y = x W^T + b with W (out_features, in_features) (reference src/NN.jl:11-38)."""
+
+    def __init__(self, in_features, out_features, graph, bias=True):
+        self.weight = tensor(graph, (out_features, in_features))
+        self.bias = tensor(graph, (out_features,)) if bias else None
+
+    def __call__(self, x):
+        out = matmul(x, permute(self.weight, (1, 0)))
+        if self.bias is not None:
+            b = self.bias
+            for size in reversed(out.shape[:-1]):  # (the reference expands over the batch axis only; same values)
+                b = expand(b, 0, size)
+            out = add(out, b)
+        return out
+
+
+class SelfAttention:
+    """SelfAttention (reference src/NN.jl:319-387) with the layer's own nodes kept — projections, the split of hidden
+    into heads (a column-major reshape, so the head index is the fast one), the permutes — and everything between them
+    (rotary embedding of Q and K, repeat_kv, scaled causal softmax attention, src/NN.jl:356-382) replaced by
+    self_attention_core: GQA without copies of K/V, the queries rotated inside the attention kernel. `attn_dtype` is
+    the element type attention runs in (the reference is fp32 only); the projections stay fp32 on the host."""
+
+    def __init__(self, hidden, n_heads, n_kv_heads, graph, attn_dtype="f32"):
+        if hidden % n_heads or n_heads % n_kv_heads:
+            raise ValueError("hidden must be a multiple of n_heads, n_heads of n_kv_heads")
+        self.n_heads, self.n_kv_heads, self.head_dim = n_heads, n_kv_heads, hidden // n_heads
+        self.attn_dtype = attn_dtype
+        self.q_proj = Linear(hidden, hidden, graph, bias=False)
+        self.k_proj = Linear(hidden, n_kv_heads * self.head_dim, graph, bias=False)
+        self.v_proj = Linear(hidden, n_kv_heads * self.head_dim, graph, bias=False)
+        self.o_proj = Linear(hidden, hidden, graph, bias=False)
+
+    def __call__(self, x, prev_seq=0, rope_base=10000.0):
+        batch, seq, hidden = x.shape
+        dt = self.attn_dtype
+
+        def heads(proj, n):  # (B, S, n*D) -> (B, n, S, D), uploaded in the element type attention reads
+            return permute(reshape(proj(x), (batch, seq, n, self.head_dim)), (0, 2, 1, 3), dtype=dt)
+
+        queries, keys, values = heads(self.q_proj, self.n_heads), heads(self.k_proj, self.n_kv_heads), heads(self.v_proj, self.n_kv_heads)
+        out = self_attention_core(queries, keys, values, causal=True, prev_seq=prev_seq, rope_base=rope_base,
+                                  out_dtype="f32")
+        out = reshape(permute(out, (0, 2, 1, 3)), (batch, seq, hidden))
+        return self.o_proj(out)
 
 
 def flash_attention(q, k, v, scale=None, causal=False, head_map=HEADMAP_INTERLEAVED, out_dtype=None, kv_len=None,
@@ -469,9 +620,25 @@ def flash_attention_plan(q_shape, kv_shape, dtype, causal=False, scale=None, out
     return binding.flash_attn_plan(p)
 
 
+def _host_fallback(op, inputs):
+    """The reference's CPU semantics for a node without a kernel: download, compute in fp32 numpy, hand back the host
+    result (the caller uploads it)."""
+    host = [x.to_host() if isinstance(x, HipArray) else np.asarray(x, dtype=np.float32) for x in inputs]
+    return np.ascontiguousarray(op.compute(*host), dtype=np.float32)
+
+
 def execute_op_inplace(out, op, *inputs, stream=None, workspaces=None):
     """execute_op!(out, op, inputs...) (reference src/Execution.jl:565-578) for the attention ops. `workspaces`
     is where decode attention takes its split-KV scratch from (default: one buffer shared by all eager calls)."""
+    if isinstance(op, HostOp):
+        if stream is not None:
+            raise RuntimeError("%s runs through the host and cannot be part of a recorded HIP graph" % type(op).__name__)
+        _require_hip(out)
+        res = _host_fallback(op, inputs)
+        if res.shape != out.shape:
+            raise ValueError("%s: result shape %s differs from the node's %s" % (type(op).__name__, res.shape, out.shape))
+        binding.sync()  # the inputs were produced by kernels on the null stream; the download above waited for them
+        return out.copy_from_host(res)
     if isinstance(op, FlashAttentionOp):
         q, k, v = inputs[:3]
         rest = list(inputs[3:])
@@ -556,6 +723,12 @@ def execute_op_inplace(out, op, *inputs, stream=None, workspaces=None):
 
 def execute_op(op, *inputs):
     """Allocating form: out = similar(q); execute_op!(out, ...) (reference src/Execution.jl:252-255)."""
+    if isinstance(op, HostOp):
+        dev = next((x.device for x in inputs if isinstance(x, HipArray)), None)
+        if dev is None:
+            raise TypeError("%s: no input is on a HIP device" % type(op).__name__)
+        res = _host_fallback(op, inputs)
+        return HipArray(res.shape, op.out_dtype, dev).copy_from_host(res)
     q = inputs[0]
     _require_hip(q)
     if isinstance(op, KVAppendOp):
@@ -647,7 +820,8 @@ class CompiledGraph:
     inputs into their buffers, runs the steps in place and returns the buffer list; nothing is
     allocated per call. After capture() the steps go through execute_with_capture: one HIP graph launch."""
 
-    def __init__(self, steps, results, workspaces=None, device=None):
+    def __init__(self, steps, results, workspaces=None, device=None, host_steps=0):
+        self.host_steps = host_steps  # nodes served by the host fallback
         self.steps = steps
         self.results = results
         self.workspaces = workspaces  # decode scratch owned by this graph: its address never changes
@@ -679,6 +853,9 @@ class CompiledGraph:
     def capture(self):
         """From the next call on, run the step list as one recorded HIP graph. Buffer addresses are fixed and
         per-step values (positions, lengths) are device tensors, so one recording is valid for every call."""
+        if self.host_steps:
+            raise RuntimeError("this graph has %d nodes that run through the host (projections, reshapes): only graphs "
+                               "of device ops can be recorded" % self.host_steps)
         self.use_capture = True
         return self
 
@@ -710,7 +887,8 @@ def compile(graph, device=None):
         args = [_pick(results, ref) for ref in node.inputs]
         steps.append(lambda stream, out=results[node_id], op=node.op, args=args:
                      execute_op_inplace(out, op, *args, stream=stream, workspaces=workspaces))
-    return CompiledGraph(steps, results, workspaces, device)
+    host_steps = sum(isinstance(node.op, HostOp) for node in graph.nodes)
+    return CompiledGraph(steps, results, workspaces, device, host_steps)
 
 
 # ---------------------------------------------------------------------------------------------
@@ -811,7 +989,8 @@ __all__ = [
     "AbstractDevice", "CPUDevice", "HIPDevice", "HipArray", "get_device", "to_device", "from_device", "Graph",
     "GraphTensor", "tensor", "add_op", "FlashAttentionOp", "DecodeAttentionOp", "flash_attention", "decode_attention",
     "RotaryEmbeddingOp", "KVAppendOp", "rotary_embedding", "kv_cache_append", "self_attention_core",
-    "cached_self_attention_core", "prompt_self_attention_core", "FUSED_ROPE_HEAD_DIMS", "execute_op", "execute_op_inplace", "execute", "compile", "CompiledGraph", "execute_with_capture", "release_capture", "HEADMAP_INTERLEAVED",
+    "cached_self_attention_core", "prompt_self_attention_core", "FUSED_ROPE_HEAD_DIMS", "HostOp", "MatMulOp", "PermuteOp", "ReshapeOp", "AddOp", "ExpandOp", "matmul", "permute",
+    "reshape", "add", "expand", "Linear", "SelfAttention", "execute_op", "execute_op_inplace", "execute", "compile", "CompiledGraph", "execute_with_capture", "release_capture", "HEADMAP_INTERLEAVED",
     "HEADMAP_BLOCKED", "LuminalHipError", "apply_rotary_embeddings", "kv_append", "KVCacheState", "encode", "decode", "f32_to_bf16_bits", "bf16_bits_to_f32", "default_scale",
     "flash_attention_plan",
 ]

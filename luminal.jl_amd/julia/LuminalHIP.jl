@@ -15,6 +15,11 @@
 #     (length, reshape, similar, copyto!: src/Execution.jl:92-97, :253; src/Compiler.jl:82-90)
 #   * compile_hip(graph): Luminal.compile (src/Compiler.jl:181-255) with the node buffers on the device,
 #     returning Luminal's own CompiledGraph
+#   * a host fallback for every other op of Luminal's (MatMul, Reshape, Permute, Add ... src/Execution.jl:216-250):
+#     on HipArray arguments it downloads them, runs Luminal's own CPU method and uploads the result, so a model
+#     graph executes on a HIPDevice with attention on the GPU and the rest where the reference computes it
+#   * self_attention(sa, x, prev_seq): Luminal.NN.SelfAttention's own projections and reshapes
+#     (src/NN.jl:343-361, :383-386) around the fused attention core instead of src/NN.jl:362-382
 # and calls the C ABI of include/luminal_hip.h through `ccall`. There are no AMDGPU.jl kernels here.
 #
 # Layout: Luminal tensors are column-major (B,H,S,D) arrays (B fastest). The library takes
@@ -23,6 +28,7 @@
 module LuminalHIP
 
 using Luminal
+using InteractiveUtils: subtypes
 import Luminal: AbstractDevice, Op, FlashAttentionOp, GraphTensor, add_op!, realized_dims, eval_dim, realize_view,
                 to_device, from_device, execute_op, execute_op!, execute_with_capture
 # Luminal exports an Op called `Function`; the Julia type is always written Base.Function here.
@@ -142,6 +148,8 @@ function Base.reshape(a::HipArray{T}, dims::NTuple{N,Int}) where {T,N}
     if [d for d in dims if d != 1] == [d for d in a.dims if d != 1]
         return HipArray{T,N}(a.ptr, dims, owner(a))
     end
+    cache_capturing() && error("reshape of a HipArray from $(a.dims) to $(dims) regroups axes: it goes through the host and " *
+                               "cannot be part of a recorded HIP graph")
     return to_device(Base.reshape(from_device(a), dims), HIPDevice())
 end
 "true when `v` is `a` itself or a view of `a`'s memory (what compile_hip requires of captured step arguments)"
@@ -532,6 +540,58 @@ function cached_self_attention_core(q::GraphTensor, k_new::GraphTensor, v_new::G
 end
 
 # ------------------------------------------------------------------------------------------
+# Host fallback: the ops around attention in a model graph (projections, reshapes, permutes, elementwise:
+# src/Execution.jl:216-250) have no kernel in libluminal_hip.so. When one of them meets a HipArray — which is what
+# the interpreter hands it on a HIPDevice (src/Execution.jl:630-656) — the arguments are downloaded, Luminal's own
+# CPU method runs (the call below dispatches to it: the arguments are Arrays by then), and the result is uploaded.
+# Slow and correct: a model runs end to end with attention on the GPU. Luminal's methods take untyped arguments, so
+# the fallback methods are generated per op type and per pattern of HipArray positions (one untyped method per op
+# type would be ambiguous with Luminal's own).
+# ------------------------------------------------------------------------------------------
+host_value(x::HipArray{BF16Bits}) = Float32.(from_device(x))
+host_value(x::HipArray) = from_device(x)
+host_value(x) = x
+function host_fallback(op::Op, args...)
+    cache_capturing() && error("$(typeof(op)) runs through the host and cannot be recorded into a HIP graph")
+    res = execute_op(op, map(host_value, args)...)
+    return res isa AbstractArray ? to_device(Array(res), HIPDevice()) : res
+end
+cache_capturing() = _stream[] != C_NULL
+
+const FIXED_FALLBACK_ARITIES = 1:3
+const DeviceOp = Union{FlashAttentionOp,RopeFlashAttentionOp,DecodeAttentionOp,RotaryEmbeddingOp,KVAppendOp}
+is_device_op_type(T) = T <: DeviceOp
+for T in subtypes(Op)
+    (is_device_op_type(T) || parentmodule(T) === @__MODULE__) && continue
+    for n in FIXED_FALLBACK_ARITIES, pattern in 1:(2^n - 1)       # every non-empty set of HipArray positions
+        sig = [(pattern >> (k - 1)) & 1 == 1 ? :($(Symbol(:a, k))::HipArray) : Symbol(:a, k) for k in 1:n]
+        names = [Symbol(:a, k) for k in 1:n]
+        @eval execute_op(op::$T, $(sig...)) = host_fallback(op, $(names...))
+    end
+    # ops with a variable number of inputs (FusedElementwiseOp, Function): a HipArray anywhere among four or more
+    @eval execute_op(op::$T, a1, a2, a3, a4, rest...) =
+        any(x -> x isa HipArray, (a1, a2, a3, a4, rest...)) ? host_fallback(op, a1, a2, a3, a4, rest...) :
+        invoke(execute_op, Tuple{$T,Vararg{Any}}, op, a1, a2, a3, a4, rest...)
+end
+
+"""
+    self_attention(sa::Luminal.NN.SelfAttention, x, prev_seq; rope_base=10000f0)
+
+The reference layer (src/NN.jl:343-387) with its own nodes kept — the four projections, the split of `hidden` into
+heads (a column-major Reshape: the head index is the fast one), the permutes — and everything between them (rotary
+embedding of Q and K, repeat_kv, scaled causal softmax attention, src/NN.jl:356-382) replaced by
+self_attention_core: the fused op reads the Hkv key/value heads directly and rotates the queries inside the kernel.
+"""
+function self_attention(sa::Luminal.NN.SelfAttention, x::GraphTensor, prev_seq::Int; rope_base=10000.0f0)
+    batch, seq, hidden = realized_dims(x.shape)
+    heads(proj, n) = Luminal.permute(Luminal.reshape(proj(x), [batch, seq, n, sa.head_dim]), [1, 3, 2, 4])
+    queries, keys, values = heads(sa.q_proj, sa.n_heads), heads(sa.k_proj, sa.n_kv_heads), heads(sa.v_proj, sa.n_kv_heads)
+    out = self_attention_core(queries, keys, values; causal=true, prev_seq=prev_seq, rope_base=rope_base)
+    out = Luminal.reshape(Luminal.permute(out, [1, 3, 2, 4]), [batch, seq, hidden])
+    return sa.o_proj(out)
+end
+
+# ------------------------------------------------------------------------------------------
 # compile_hip(graph): Luminal.compile (src/Compiler.jl:181-255) for graphs of the operators above, with the
 # node buffers on the device. Luminal.compile itself cannot serve: it allocates host `zeros` for every
 # non-CUDA device (:224-228) and its step closures capture those host arrays at compile time (:250-255), so
@@ -542,7 +602,6 @@ end
 #            lengths default to Int32) and, optionally, for op nodes (default: the type of their first
 #            input; Float32 on a half-precision attention node asks for the fp32 result).
 # ------------------------------------------------------------------------------------------
-const DeviceOp = Union{FlashAttentionOp,RopeFlashAttentionOp,DecodeAttentionOp,RotaryEmbeddingOp,KVAppendOp}
 is_input_node(op) = op isa Luminal.Function && op.name == "InputTensor"
 
 function compile_hip(graph::Luminal.Graph; eltypes::AbstractDict=Dict{Int,DataType}())
@@ -570,13 +629,14 @@ function compile_hip(graph::Luminal.Graph; eltypes::AbstractDict=Dict{Int,DataTy
         elseif op isa DeviceOp
             eltype_of[node_id] = get(eltypes, node_id, eltype_of[node.inputs[1][1]])
             results[node_id] = zeros_hip(eltype_of[node_id], dims)
-        else
-            error("compile_hip: node $node_id is a $(typeof(op)), which has no executor in libluminal_hip.so; this " *
-                  "backend covers the attention path (FlashAttentionOp, DecodeAttentionOp, RotaryEmbeddingOp, KVAppendOp)")
+        else                                     # served by the host fallback: a Float32 buffer the step uploads into
+            eltype_of[node_id] = Float32
+            results[node_id] = zeros_hip(Float32, dims)
         end
     end
     # 2. one in-place step per op; arguments are views of the persistent buffers, captured once (:250-255)
     steps = Base.Function[]
+    n_host = 0
     for (node_id, node) in enumerate(graph.nodes)
         op = node.op
         is_input_node(op) && continue
@@ -586,13 +646,25 @@ function compile_hip(graph::Luminal.Graph; eltypes::AbstractDict=Dict{Int,DataTy
                 error("compile_hip: input $k of node $node_id is a reshape that regroups axes; not supported on device buffers")
         end
         target_buf = results[node_id]
-        push!(steps, (results, device) -> execute_op!(target_buf, op, step_args...))
+        if op isa DeviceOp
+            push!(steps, (results, device) -> execute_op!(target_buf, op, step_args...))
+        else                                     # download, Luminal's CPU method, upload into the node's buffer
+            n_host += 1
+            push!(steps, (results, device) -> copyto!(target_buf, Array(execute_op(op, map(host_value, step_args)...))))
+        end
     end
-    return Luminal.CompiledGraph(steps, results, Dict{Symbol,Any}())
+    cache = Dict{Symbol,Any}()
+    n_host > 0 && (cache[:hip_host_steps] = n_host)
+    return Luminal.CompiledGraph(steps, results, cache)
 end
 
 "From the next call on, run the compiled steps as one recorded HIP graph (see execute_with_capture below)."
-enable_capture!(cg::Luminal.CompiledGraph) = (cg.cache[:hip_capture] = true; cg)
+function enable_capture!(cg::Luminal.CompiledGraph)
+    get(cg.cache, :hip_host_steps, 0) == 0 ||
+        error("enable_capture!: $(cg.cache[:hip_host_steps]) steps of this graph run through the host; only graphs of device ops can be recorded")
+    cg.cache[:hip_capture] = true
+    return cg
+end
 
 # ------------------------------------------------------------------------------------------
 # execute_with_capture(device, f, cache) (src/Device.jl:108-121; called by the compiled step closure,
@@ -659,6 +731,6 @@ end
 export HIPDevice, HipArray, BF16Bits, release_capture!, enable_capture!, compile_hip, DecodeAttentionOp, decode_attention,
        RotaryEmbeddingOp, rotary_embedding, KVAppendOp, kv_cache_append, get_device, functional, rope!, kv_append!,
        self_attention_core!, cached_self_attention_core!, self_attention_core, cached_self_attention_core, flash_attention_plan,
-       RopeFlashAttentionOp, rope_flash_attention, prompt_self_attention_core!
+       RopeFlashAttentionOp, rope_flash_attention, prompt_self_attention_core!, self_attention, host_fallback
 
 end # module

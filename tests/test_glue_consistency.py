@@ -130,7 +130,15 @@ ARRAY_PROTOCOL = [
     ("execute_op!(target_buf, op, step_args...)", "src/Compiler.jl", 254, "execute_op!(target_buf, op, step_args...)",
      r"push!\(steps, \(results, device\) -> execute_op!\(target_buf, op, step_args\.\.\.\)\)"),
     ("CompiledGraph(steps, results, cache)", "src/Compiler.jl", 75, "struct CompiledGraph",
-     r"return Luminal\.CompiledGraph\(steps, results, Dict\{Symbol,Any\}\(\)\)"),
+     r"return Luminal\.CompiledGraph\(steps, results, cache\)"),
+    # every other op the interpreter dispatches (src/Execution.jl:216-250) meets HipArray arguments on a HIPDevice:
+    # a fallback method generated for each op type of Luminal's, for each pattern of HipArray positions
+    ("execute_op(op::Add, a, b) and the other untyped CPU methods", "src/Execution.jl", 216, "execute_op(op::Add, a, b)",
+     r"^for T in subtypes\(Op\)$"),
+    ("execute_op(op::MatMul, a, b)", "src/Execution.jl", 231, "execute_op(op::MatMul, a, b)",
+     r"@eval execute_op\(op::\$T, \$\(sig\.\.\.\)\) = host_fallback\(op, \$\(names\.\.\.\)\)"),
+    ("execute_op(op::Reshape, a)", "src/Execution.jl", 228, "execute_op(op::Reshape, a)",
+     r"^function host_fallback\(op::Op, args\.\.\.\)"),
 ]
 EXTRA_METHODS = [  # used by the glue's own executors on HipArray arguments
     r"^Base\.size\(a::HipArray\)", r"^Base\.size\(a::HipArray, i::Integer\)", r"^Base\.ndims\(::HipArray\{T,N\}\)",
@@ -277,3 +285,31 @@ def test_glue_ccalls_pass_as_many_arguments_as_the_header_declares():
         assert len(declared) == len(types), "ccall of %s: header declares %d parameters" % (name, len(declared))
         seen += 1
     assert seen >= 20
+
+
+def test_glue_host_fallback_and_layer_builder():
+    """The fallback downloads, calls Luminal's own CPU method and uploads; compile_hip gives nodes without a kernel a
+    host step instead of refusing them, and such graphs cannot be recorded; self_attention keeps the reference layer's
+    projections and reshapes (reference src/NN.jl:343-361, :383-386) around self_attention_core."""
+    text = glue_text()
+    body = re.search(r"^function host_fallback\(op::Op, args\.\.\.\).*?^end$", text, flags=re.M | re.S).group(0)
+    assert "execute_op(op, map(host_value, args)...)" in body and "to_device(" in body and "cache_capturing()" in body
+    assert re.search(r"^host_value\(x::HipArray\) = from_device\(x\)$", text, flags=re.M)
+    # the generated methods skip the ops that have kernels and the glue's own op types
+    loop = re.search(r"^for T in subtypes\(Op\)\n(.*?)^end$", text, flags=re.M | re.S).group(1)
+    assert "is_device_op_type(T) || parentmodule(T) === @__MODULE__" in loop and "pattern in 1:(2^n - 1)" in loop
+    comp = re.search(r"^function compile_hip\(.*?^end$", text, flags=re.M | re.S).group(0)
+    assert "copyto!(target_buf, Array(execute_op(op, map(host_value, step_args)...)))" in comp
+    assert "has no executor" not in comp and ":hip_host_steps" in comp
+    cap = re.search(r"^function enable_capture!\(.*?^end$", text, flags=re.M | re.S).group(0)
+    assert ":hip_host_steps" in cap and "error(" in cap
+    layer = re.search(r"^function self_attention\(sa::Luminal\.NN\.SelfAttention, x::GraphTensor, prev_seq::Int;.*?^end$", text,
+                      flags=re.M | re.S).group(0)
+    for piece in ("sa.q_proj", "sa.k_proj", "sa.v_proj", "sa.o_proj", "Luminal.reshape(proj(x), [batch, seq, n, sa.head_dim])",
+                  "[1, 3, 2, 4]", "self_attention_core(queries, keys, values; causal=true, prev_seq=prev_seq, rope_base=rope_base)",
+                  "[batch, seq, hidden]"):
+        assert piece in layer, piece
+    if os.path.isdir(REFERENCE):  # the layer's own lines in the reference say the same
+        nn = open(os.path.join(REFERENCE, "src/NN.jl")).read()
+        assert "Luminal.reshape(sa.q_proj(x), [batch, seq, sa.n_heads, sa.head_dim])" in nn
+        assert "Luminal.permute(queries, [1, 3, 2, 4])" in nn and "Luminal.reshape(out, [batch, seq, hidden])" in nn

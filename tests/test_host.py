@@ -186,3 +186,58 @@ def test_kernel_plan_of_the_benchmark_configurations(lm):
     assert plan((2, 4, 100, 64), (2, 4, 100, 64), "f16", False, scale=-1.0).startswith("prefill_valu_kernel<f16")
     with pytest.raises(lm.LuminalHipError):
         plan((2, 4, 100, 264), (2, 4, 100, 264), "f16", False)
+
+
+def test_host_ops_follow_the_reference_semantics(lm):
+    # Reshape is Base.reshape on a column-major array (reference src/Execution.jl:228): splitting 6 into (2, 3) makes the
+    # first new axis the fast one
+    a = np.arange(12, dtype=np.float32).reshape(2, 6)
+    r = lm.ReshapeOp((2, 2, 3)).compute(a)
+    assert r[0, 1, 0] == a[0, 1] and r[0, 0, 1] == a[0, 2] and r[1, 1, 2] == a[1, 5]
+    assert np.array_equal(lm.PermuteOp((1, 0)).compute(a), a.T)
+    e = lm.ExpandOp(1, 3).compute(a)  # (2, 3, 6), every copy equal (reference src/Execution.jl:238-248)
+    assert e.shape == (2, 3, 6) and np.array_equal(e[:, 2], a)
+    b3 = np.ones((4, 2, 6), np.float32)
+    assert lm.MatMulOp().compute(b3, a.T).shape == (4, 2, 2)  # ND x 2D (reference src/Execution.jl:12-90)
+    with pytest.raises(ValueError, match="mismatch"):
+        lm.MatMulOp().compute(a, a)
+    assert np.array_equal(lm.AddOp().compute(b3, a[0]), b3 + a[0])
+    # on host arrays the fallback has no device to work for: the attention backend has no CPU path
+    with pytest.raises(TypeError):
+        lm.execute_op(lm.MatMulOp(), a, a.T)
+
+
+def test_self_attention_layer_graph_and_its_semantics_against_the_reference_replay(lm, oracle):
+    """The layer's graph is the reference's own nodes around one fused core; and that decomposition — heads split by a
+    column-major reshape, rotary pairs (j, j + D/2), KV head of query head hq = hq % Hkv — reproduces the reference
+    layer replayed literally in float64 (repeat_kv, additive mask, softmax), here with the oracle as the core."""
+    from layer_reference import reference_layer_f64
+    B, S, hidden, n_heads, n_kv_heads, prev_seq = 2, 24, 64, 4, 2, 3
+    D = hidden // n_heads
+    g = lm.Graph()
+    tx = lm.tensor(g, (B, S, hidden))
+    layer = lm.SelfAttention(hidden, n_heads, n_kv_heads, g)
+    out = layer(tx, prev_seq)
+    kinds = [type(n.op).__name__ for n in g.nodes[5:]]
+    assert kinds == ["PermuteOp", "MatMulOp", "ReshapeOp", "PermuteOp"] * 3 + ["RotaryEmbeddingOp", "RotaryEmbeddingOp",
+                                                                              "FlashAttentionOp", "PermuteOp", "ReshapeOp",
+                                                                              "PermuteOp", "MatMulOp"]
+    assert out.shape == (B, S, hidden)
+    x = oracle.gen_normal((B, S, hidden), 31)
+    ws = [oracle.gen_normal(shape, 32 + i, 1.0 / np.sqrt(hidden)) for i, shape in
+          enumerate([(hidden, hidden), (n_kv_heads * D, hidden), (n_kv_heads * D, hidden), (hidden, hidden)])]
+    want = reference_layer_f64(x, *ws, n_heads, n_kv_heads, prev_seq)
+
+    def heads(w, n):
+        h = lm.ReshapeOp((B, S, n, D)).compute(lm.MatMulOp().compute(x, lm.PermuteOp((1, 0)).compute(w)))
+        return np.ascontiguousarray(lm.PermuteOp((0, 2, 1, 3)).compute(h))
+
+    q, k, v = heads(ws[0], n_heads), heads(ws[1], n_kv_heads), heads(ws[2], n_kv_heads)
+    att = oracle.flash_attn(oracle.rope(q, prev_seq=prev_seq), oracle.rope(k, prev_seq=prev_seq), v, causal=True)
+    merged = lm.ReshapeOp((B, S, hidden)).compute(lm.PermuteOp((0, 2, 1, 3)).compute(att))
+    got = lm.MatMulOp().compute(merged, ws[3].T)
+    assert np.abs(got - want).max() / np.abs(want).max() <= 2e-5
+    # the row-major (HuggingFace) conventions would not: blocked head map, or a row-major head split
+    att_blocked = oracle.flash_attn(oracle.rope(q, prev_seq=prev_seq), oracle.rope(k, prev_seq=prev_seq), v, causal=True, head_map=1)
+    wrong = lm.MatMulOp().compute(lm.ReshapeOp((B, S, hidden)).compute(lm.PermuteOp((0, 2, 1, 3)).compute(att_blocked)), ws[3].T)
+    assert np.abs(wrong - want).max() / np.abs(want).max() > 1e-2
