@@ -33,6 +33,7 @@ extern "C" {
 #define LMH_E_WORKSPACE (-4)   /* decode workspace missing, too small or not 16-byte aligned */
 #define LMH_E_HIP (-5)         /* a HIP runtime call failed */
 #define LMH_E_NODEVICE (-6)    /* no usable gfx950 device */
+#define LMH_E_BUSY (-7)        /* the static scratch is still in use by a call on another stream */
 
 /* element type of q/k/v/out; accumulation is always fp32 */
 #define LMH_F32 0
@@ -200,8 +201,13 @@ int lmh_decode_attn(const lmh_decode_params *p);
  *     array is rejected with LMH_E_WORKSPACE.
  *   - Every call on one GPU shares that GPU's array, which keeps the last call's contents. Nothing in it
  *     has to start at zero (each call writes every slot it later reads), so none is cleared; calls that
- *     overlap in time on one GPU (two streams, two host threads) race on it and must be serialised by the
- *     caller.
+ *     overlap in time on one GPU race on it and must be ordered by the caller. One stream orders its own
+ *     calls. A call on a second (non-null) stream while the previous user is still running is refused with
+ *     LMH_E_BUSY (the library records an event behind every eager call and queries it; no allocation). Calls
+ *     recorded into a HIP graph cannot be checked this way: a replay must not overlap another user of the array.
+ *   - The array is part of the library's code object: every process that loads the library holds
+ *     LMH_STATIC_SCRATCH_BYTES of device memory on each GPU it initialises, whether or not this entry point is
+ *     ever called.
  *   - lmh_init(device) resolves the array's address on that device; a device that was never passed to
  *     lmh_init resolves it on its first call here, which may load the code object (do that before a capture).
  * No hipMalloc, hipFree or other allocating call is made. ---- */

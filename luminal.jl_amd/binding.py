@@ -17,7 +17,7 @@ DTYPE_CODES = {"f32": LMH_F32, "f16": LMH_F16, "bf16": LMH_BF16}
 DTYPE_BYTES = {"f32": 4, "f16": 2, "bf16": 2}
 
 LMH_OK = 0
-LMH_E_NULL, LMH_E_SHAPE, LMH_E_UNSUPPORTED, LMH_E_WORKSPACE, LMH_E_HIP, LMH_E_NODEVICE = -1, -2, -3, -4, -5, -6
+LMH_E_NULL, LMH_E_SHAPE, LMH_E_UNSUPPORTED, LMH_E_WORKSPACE, LMH_E_HIP, LMH_E_NODEVICE, LMH_E_BUSY = -1, -2, -3, -4, -5, -6, -7
 
 # every symbol include/luminal_hip.h declares
 EXPORTS = [

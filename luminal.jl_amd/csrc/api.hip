@@ -72,6 +72,14 @@ constexpr int kMaxDevices = 64;
 // hipGetSymbolAddress, never an address a kernel can use.
 void *g_scratch_ptr[kMaxDevices];
 std::mutex g_scratch_mutex;
+// Who used the scratch last on each GPU: an event recorded behind that call's kernels and the stream it ran on. The next
+// call on another stream asks the event whether the earlier call has finished, and refuses to race with it.
+struct ScratchUse {
+  hipEvent_t done = nullptr;
+  hipStream_t stream = nullptr;
+  bool pending = false;
+};
+ScratchUse g_scratch_use[kMaxDevices];
 
 // Looks the address up once per device, with that device current, and returns it in *out.
 int static_scratch_for_current_device(void **out) {
@@ -87,10 +95,66 @@ int static_scratch_for_current_device(void **out) {
     const hipError_t e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
     if (e != hipSuccess) return hip_fail(e, "hipGetSymbolAddress(scratch)");
     if (!ptr) return fail(LMH_E_HIP, "static scratch: hipGetSymbolAddress returned a null address");
+    hipEvent_t ev = nullptr;  // part of the same one-time set-up: the entry point itself creates nothing
+    const hipError_t ee = hipEventCreateWithFlags(&ev, hipEventDisableTiming);
+    if (ee != hipSuccess) return hip_fail(ee, "hipEventCreateWithFlags(static scratch)");
+    g_scratch_use[dev].done = ev;
     g_scratch_ptr[dev] = ptr;
   }
   *out = g_scratch_ptr[dev];
   return LMH_OK;
+}
+
+// True while `stream` is recording a HIP graph (then nothing may be queried or recorded on its behalf).
+bool stream_is_capturing(hipStream_t stream) {
+  hipStreamCaptureStatus st = hipStreamCaptureStatusNone;
+  if (hipStreamIsCapturing(stream, &st) != hipSuccess) {
+    (void)hipGetLastError();
+    return true;  // cannot tell: behave as under capture (no event calls)
+  }
+  return st != hipStreamCaptureStatusNone;
+}
+
+// Before a call that uses the scratch: refuse when the previous user, on another stream, is still running. Two calls on
+// one stream are ordered by the stream; the null stream and the streams of lmh_stream_create order themselves against
+// each other, so only two different non-null streams can overlap. Calls recorded into a graph are not seen here.
+int static_scratch_claim(hipStream_t stream, const char *fn) {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) {
+    (void)hipGetLastError();
+    return LMH_OK;
+  }
+  if (stream_is_capturing(stream)) return LMH_OK;
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  ScratchUse &u = g_scratch_use[dev];
+  if (u.pending && u.stream != stream && u.stream != nullptr && stream != nullptr) {
+    const hipError_t q = hipEventQuery(u.done);
+    if (q == hipErrorNotReady)
+      return fail(LMH_E_BUSY, "%s: the previous call that uses this GPU's static scratch is still running on another stream; "
+                              "calls that share the scratch must not overlap (order them, or use lmh_decode_attn with a workspace)", fn);
+    if (q != hipSuccess) (void)hipGetLastError();
+  }
+  return LMH_OK;
+}
+
+// After the kernels of such a call were enqueued.
+void static_scratch_mark(hipStream_t stream) {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) {
+    (void)hipGetLastError();
+    return;
+  }
+  if (stream_is_capturing(stream)) return;
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  ScratchUse &u = g_scratch_use[dev];
+  if (!u.done) return;
+  if (hipEventRecord(u.done, stream) != hipSuccess) {
+    (void)hipGetLastError();
+    u.pending = false;
+    return;
+  }
+  u.stream = stream;
+  u.pending = true;
 }
 
 }  // namespace
@@ -491,10 +555,14 @@ int lmh_decode_attn_static(const lmh_decode_params *p) {
   if (splits > 1) {
     const int rc_ws = static_scratch_for_current_device(&ws);
     if (rc_ws != LMH_OK) return rc_ws;
+    const int rc_claim = static_scratch_claim((hipStream_t)p->stream, fn);
+    if (rc_claim != LMH_OK) return rc_claim;
   }
   // Nothing in the scratch has to start at zero: every partial slot the merge kernel reads was written by
   // the split kernel of the same call (a result, or the "empty" marker), so no clearing is enqueued.
-  return decode_launch(p, fn, splits, ws, LMH_STATIC_SCRATCH_BYTES);
+  const int rc_launch = decode_launch(p, fn, splits, ws, LMH_STATIC_SCRATCH_BYTES);
+  if (rc_launch == LMH_OK && splits > 1) static_scratch_mark((hipStream_t)p->stream);
+  return rc_launch;
 }
 
 // --------------------------------------------------------------------------------------------

@@ -91,3 +91,70 @@ def test_static_scratch_decode_rejects_what_does_not_fit(lm, hip):
     with pytest.raises(lm.LuminalHipError) as e:
         b.decode_attn_static(_params(lm, out, dq, dk, dk, dl, "f16", 32))
     assert e.value.code == b.LMH_E_WORKSPACE and "static scratch" in str(e.value)
+
+
+def test_static_scratch_decode_recorded_into_a_hip_graph(lm, hip, oracle):
+    """What the entry point is for: under stream capture nothing can be allocated. One recording of a split-KV call
+    (several splits, so the static array is in use) is replayed for two sets of lengths, with eager work and
+    synchronisations in between, and every replay is held to the oracle and to the eager call."""
+    b = lm.binding
+    B, Hq, Hkv, Lmax, D, dtype = 4, 16, 4, 2048, 128, "bf16"
+    q = oracle.round_to(oracle.gen_normal((B, Hq, D), 9500), dtype)
+    k = oracle.round_to(oracle.gen_normal((B, Hkv, Lmax, D), 9501), dtype)
+    v = oracle.round_to(oracle.gen_normal((B, Hkv, Lmax, D), 9502), dtype)
+    dq, dk, dv = (lm.to_device(x, hip, dtype) for x in (q, k, v))
+    lens = [np.array([2048, 1500, 700, 33], np.int32), np.array([5, 2048, 1, 1024], np.int32)]
+    dl = lm.to_device(lens[0], hip)
+    splits = b.decode_static_splits(B, Hq, Hkv, Lmax, D)
+    assert splits > 1
+    out = lm.HipArray((B, Hq, D), "f32", hip)
+    b.init(0)  # resolves the array's address and creates the guard event: set-up stays outside the recording
+    stream = b.stream_create()
+    p = _params(lm, out, dq, dk, dv, dl, dtype, 0)
+    p.stream = stream
+    b.graph_capture_begin(stream)
+    try:
+        b.decode_attn_static(p)
+    finally:
+        graph = b.graph_capture_end(stream)
+    eager_out = lm.HipArray((B, Hq, D), "f32", hip)
+    for rep in range(4):
+        cur = lens[rep % 2]
+        dl.copy_from_host(cur)
+        out.fill_bytes(0xFF)
+        b.graph_launch(graph, stream)
+        b.sync(stream)
+        got = out.to_host()
+        want = oracle.decode_attn(q, k, v, kv_len=cur, nthreads=16)
+        assert rel_err(got, want) <= TOL[dtype], rep
+        # an eager call on the null stream in between (it shares the array; ordered by the synchronisations)
+        b.decode_attn_static(_params(lm, eager_out, dq, dk, dv, dl, dtype, 0))
+        np.testing.assert_array_equal(eager_out.to_host(), got)
+    b.graph_destroy(graph)
+    b.stream_destroy(stream)
+
+
+def test_static_scratch_decode_refuses_to_overlap_on_two_streams(lm, hip):
+    """Calls that share the array must not overlap: a call on a second stream while the first is still running is
+    refused with LMH_E_BUSY; once the first has finished the same call goes through."""
+    b = lm.binding
+    B, Hq, Hkv, Lmax, D = 8, 32, 8, 32768, 128  # ~1 GB of cache reads: a few hundred microseconds of kernel
+    dq = lm.HipArray((B, Hq, D), "bf16", hip).fill_bytes(0)
+    dk = lm.HipArray((B, Hkv, Lmax, D), "bf16", hip).fill_bytes(0)
+    dl = lm.to_device(np.full(B, Lmax, np.int32), hip)
+    out1, out2 = lm.HipArray((B, Hq, D), "f32", hip), lm.HipArray((B, Hq, D), "f32", hip)
+    s1, s2 = b.stream_create(), b.stream_create()
+    p1, p2 = _params(lm, out1, dq, dk, dk, dl, "bf16", 0), _params(lm, out2, dq, dk, dk, dl, "bf16", 0)
+    p1.stream, p2.stream = s1, s2
+    b.sync()
+    for _ in range(3):
+        b.decode_attn_static(p1)  # queued back to back on one stream: ordered, never refused
+    with pytest.raises(lm.LuminalHipError) as e:
+        b.decode_attn_static(p2)
+    assert e.value.code == b.LMH_E_BUSY and "static scratch" in str(e.value)
+    b.sync(s1)
+    b.decode_attn_static(p2)
+    b.sync(s2)
+    np.testing.assert_array_equal(out1.to_host(), out2.to_host())
+    b.stream_destroy(s1)
+    b.stream_destroy(s2)
