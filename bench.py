@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the attention hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--only all|prefill|decode|other|c1|c3|c4|ops|step|copy|ceiling]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--only all|prefill|decode|other|c1|nomask|c3|c4|ops|step|copy|ceiling|grid]
 
 A step is one pass of the hot path over one batch of synthetic input, inputs resident in HBM:
   prefill leg (the headline `value`): causal flash attention, Phi-3-mini shape
@@ -162,6 +162,8 @@ def prefill_leg(lm, dev, steps, warmup, cpu_seconds):
         % (wall_ms * 1e3, ev_ms * 1e3, kern_tflops, 100 * kern_tflops / PEAK_FP16_TFLOPS, PEAK_FP16_TFLOPS))
     each = per_launch_us(fn, 20, lm.binding)
     sustained = mfma_sustained(lm, dev, dq)
+    on_zeros = zero_operand_launch_us(lm, dev, p, (B, H, S, D), "f16", steps, warmup)
+    log("[prefill] the same launch on all-zero Q, K, V (same instruction stream, no switching in the data paths): %.1f us" % on_zeros)
     res = {
         "ms_per_step": wall_ms, "value": tflops,
         "roofline": {"bound": "mfma", "achieved": kern_tflops, "peak": PEAK_FP16_TFLOPS, "unit": "TFLOP/s",
@@ -171,7 +173,11 @@ def prefill_leg(lm, dev, steps, warmup, cpu_seconds):
                      # what a bare MFMA loop sustains on this GPU right now (clock management under load):
                      # on all-zero operands and on the Q tensor of this workload
                      "mfma_sustained_tflops": sustained,
-                     "frac_of_sustained": kern_tflops / sustained["workload_operands"]},
+                     "frac_of_sustained": kern_tflops / sustained["workload_operands"],
+                     # the same launch (same kernel, grid and instruction stream) on all-zero Q, K and V: what is left
+                     # of the difference to launch_us once the handful of rescales is discounted is the clock the
+                     # chip grants under the data's switching activity
+                     "launch_us_on_zero_operands": on_zeros},
     }
     if cpu_seconds > 0:
         # CPU baseline = the oracle on a head subset of the same workload, all host threads; the same
@@ -205,6 +211,16 @@ def prefill_leg(lm, dev, steps, warmup, cpu_seconds):
                                              "sample": "head 0 of %d, all %d query rows, %.1f s" % (H, S, t1)}
         log("[prefill] CPU oracle, 1 thread: head 0 in %.1f s = %.5f TFLOP/s" % (t1, flops / H / t1 / 1e12))
     return res
+
+
+def zero_operand_launch_us(lm, dev, p, shape, dtype, steps, warmup):
+    """HIP-event time per launch of the attention launch `p` with its Q, K and V replaced by all-zero tensors."""
+    zq, zk, zv = (lm.HipArray(shape, dtype, dev).fill_bytes(0) for _ in range(3))
+    zo = lm.HipArray(shape, "f32" if p.out_f32 else dtype, dev)  # (the launch's own output stays as it is)
+    pz = lm.binding.AttnParams.from_buffer_copy(p)
+    pz.q, pz.k, pz.v, pz.out = zq.ptr, zk.ptr, zv.ptr, zo.ptr
+    _, ev = time_steps(lambda: lm.binding.flash_attn_fwd(pz), steps, warmup, lm.binding)
+    return ev * 1e3
 
 
 def mfma_sustained(lm, dev, operands):
@@ -330,6 +346,35 @@ def c1_leg(lm, dev, res, check):
     name = "C2 shape in fp32 (causal B=1 H=32 S=4096 D=96)"
     flash_config(lm, dev, res, name, 1, 32, 32, 4096, 4096, 96, "f32", True, 4.0 * 32 * 96 * 4096 * 4097 / 2, 2000, mul=0.5)
     res[name]["frac_of_fp32_mfma_peak"] = res[name]["TFLOP/s"] / PEAK_FP32_TFLOPS
+
+
+def nomask_leg(lm, dev, res, check):
+    """The C2 shape without the causal mask (an extra line, not one of the five configurations): every workgroup walks
+    all 4096 keys, so the launch is 32 equal tiles per CU and shows the loop's steady state without the diagonal."""
+    name = "C2 shape without the mask (fp16 B=1 H=32 S=4096 D=96)"
+    B, H, S, D = 1, 32, 4096, 96
+    hq, hk, hv = (lm.synth.normal((B, H, S, D), 2000 + i, 0.5) for i in range(3))
+    q, k, v = (lm.HipArray(x.shape, "f16", dev).copy_from_host(x) for x in (hq, hk, hv))
+    o = lm.HipArray((B, H, S, D), "f16", dev)
+    p = attn_params(lm, o, q, k, v, "f16", False, lm.default_scale(D))
+    fn = lambda: lm.binding.flash_attn_fwd(p)
+    flops = 4.0 * B * H * D * S * S
+    _, ev = time_steps(fn, 40, 5, lm.binding)
+    res[name] = {"launch_us": ev * 1e3, "TFLOP/s": flops / (ev * 1e-3) / 1e12, "frac_of_mfma_peak": flops / (ev * 1e-3) / 1e12 / PEAK_FP16_TFLOPS,
+                 "kernel": lm.binding.flash_attn_plan(p),
+                 "launch_us_on_zero_operands": zero_operand_launch_us(lm, dev, p, (B, H, S, D), "f16", 40, 5)}
+    log("[other] %s: %.1f us, %.1f TFLOP/s; on zero operands %.1f us; %s" % (name, ev * 1e3, res[name]["TFLOP/s"],
+                                                                           res[name]["launch_us_on_zero_operands"], res[name]["kernel"]))
+    if check:
+        import oracle
+        heads = slice(0, 4)
+        qh, kh, vh = (np.asarray(x.to_host(), np.float32)[:, heads] for x in (q, k, v))
+        want = oracle.flash_attn(qh, kh, vh, scale=lm.default_scale(D), causal=False, nthreads=oracle.max_threads())
+        err = rel_err(np.asarray(o.to_host(), np.float32)[:, heads], want)
+        res[name]["parity"] = {"max_rel_err": err, "tolerance": 2e-3, "checked": "heads 0..3 vs CPU oracle"}
+        log("[other] %s: GPU vs oracle rel err %.2e" % (name, err))
+        if err > 2e-3:
+            raise SystemExit("parity check failed on %s: rel err %.3g > 2e-3" % (name, err))
 
 
 def c3_leg(lm, dev, res, check):
@@ -580,11 +625,13 @@ def ceiling_leg(lm, dev):
 def other_configs(lm, dev, check=False, only="other"):
     """Short timings of the remaining contract configurations. With `check`, C1, C3 and C4 are also compared with the
     CPU oracle on the whole output (the parity gate of the five configurations: C2 and C5 are checked in their own
-    legs). `only` = "other" runs everything, or one of c1 / c3 / c4 / ops / step (a profile of one kernel)."""
+    legs). `only` = "other" runs everything, or one of c1 / nomask / c3 / c4 / ops / step (a profile of one kernel)."""
     res = {}
     caches = None
     if only in ("other", "c1"):
         c1_leg(lm, dev, res, check)
+    if only in ("other", "nomask"):
+        nomask_leg(lm, dev, res, check)
     if only in ("other", "c3"):
         c3_leg(lm, dev, res, check)
     if only in ("other", "c4"):
@@ -639,7 +686,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--only", choices=["all", "prefill", "decode", "other", "c1", "c3", "c4", "ops", "step", "copy", "ceiling", "grid"], default="all")
+    ap.add_argument("--only", choices=["all", "prefill", "decode", "other", "c1", "nomask", "c3", "c4", "ops", "step", "copy", "ceiling", "grid"], default="all")
     ap.add_argument("--decode-splits", type=int, default=0, help="KV splits for the decode leg (0 = library heuristic)")
     ap.add_argument("--cpu-seconds", type=float, default=15.0, help="CPU-baseline budget per leg; 0 disables it")
     args = ap.parse_args()
@@ -683,7 +730,7 @@ def main():
             line["cpu_baseline_single_thread"] = r["cpu_baseline_single_thread"]
     if args.only in ("all", "decode"):
         line["decode"] = decode_leg(lm, dev, args.steps, args.warmup, args.cpu_seconds, args.decode_splits)
-    if args.only in ("all", "other", "c1", "c3", "c4", "ops", "step"):
+    if args.only in ("all", "other", "c1", "nomask", "c3", "c4", "ops", "step"):
         line["other_configs"] = other_configs(lm, dev, check=args.cpu_seconds > 0, only="other" if args.only == "all" else args.only)
     gate = [("C2", line.get("parity"))] + [("C5", line.get("decode", {}).get("parity"))] + \
         [(k.split()[0], v.get("parity")) for k, v in line.get("other_configs", {}).items() if isinstance(v, dict) and "parity" in v]

@@ -23,6 +23,13 @@ LIBRARIES = {
     CALIB_LIBNAME: ["calib.hip"],
 }
 
+# Sources that only a measurement build contains: switch in LMH_EXTRA_FLAGS -> (source, flags for that file alone).
+# -amdgpu-mfma-vgpr-form: with one wave per SIMD the compiler otherwise keeps every MFMA result in the accumulation
+# registers and moves the scores out of them one by one.
+MEASUREMENT_SOURCES = {
+    "-DLMH_W64_KERNEL": ("prefill_mfma_w64.hip", ["-mllvm", "-amdgpu-mfma-vgpr-form"]),
+}
+
 # -packed-fp32-ops: keep the compiler from forming v_pk_{add,mul,fma}_f32 out of scalar fp32 code.
 HIPCC_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fno-gpu-rdc",
@@ -62,14 +69,20 @@ def build_library(verbose=True):
     objdir = os.path.join(LIBDIR, "obj")
     os.makedirs(objdir, exist_ok=True)
     procs = []
-    for libname, sources in LIBRARIES.items():
+    file_flags = {}
+    libraries = {name: list(sources) for name, sources in LIBRARIES.items()}
+    for switch, (src, src_flags) in MEASUREMENT_SOURCES.items():
+        if switch in flags:
+            libraries[LIBNAME].append(src)
+            file_flags[src] = src_flags
+    for libname, sources in libraries.items():
         for src in sources:
             obj = os.path.join(objdir, src.replace(".hip", ".o"))
-            cmd = [hipcc] + flags + ["-c", os.path.join(CSRC, src), "-o", obj]
+            cmd = [hipcc] + flags + file_flags.get(src, []) + ["-c", os.path.join(CSRC, src), "-o", obj]
             if verbose:
                 print("[build]", " ".join(cmd), flush=True)
             procs.append((libname, src, obj, subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)))
-    objs = {name: [] for name in LIBRARIES}
+    objs = {name: [] for name in libraries}
     for libname, src, obj, proc in procs:
         out, _ = proc.communicate()
         # the host pass does not know the gfx-only target feature; that note is expected
@@ -79,7 +92,7 @@ def build_library(verbose=True):
         if verbose and out.strip():
             print(out)
         objs[libname].append(obj)
-    for libname in LIBRARIES:
+    for libname in libraries:
         tmp = library_path(libname) + ".tmp"
         cmd = [hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", tmp] + objs[libname]
         if verbose:

@@ -108,6 +108,11 @@ __host__ __device__ inline int q_head_of(int kvh, int g, int Hq, int Hkv, int he
 inline bool prefill_mfma_rope_ok(int D) { return D == 64 || D == 96 || D == 128; }
 bool prefill_mfma_supported(int dtype, int D);
 int launch_prefill_mfma(const PrefillArgs &a, int dtype, hipStream_t stream);
+#ifdef LMH_W64_KERNEL
+// measurement builds only (prefill_mfma_w64.hip): the hand-pipelined 64-columns-per-wave kernel and the launches it takes
+bool prefill_w64_takes(const PrefillArgs &a, int dtype);
+int launch_prefill_w64(const PrefillArgs &a, hipStream_t stream);
+#endif
 bool prefill_f32_mfma_supported(int dtype, int D);
 int launch_prefill_f32_mfma(const PrefillArgs &a, hipStream_t stream);
 int launch_prefill_valu(const PrefillArgs &a, int dtype, hipStream_t stream);

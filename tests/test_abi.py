@@ -52,6 +52,12 @@ def test_experiment_flags_need_the_measurement_marker(lm, monkeypatch):
         build.experiment_flags()
     monkeypatch.setenv("LMH_MEASUREMENT_BUILD", "1")
     assert build.experiment_flags() == ["-DLMH_FOLD_SCALE", "-DLMH_MEASUREMENT_BUILD"]
+    # kernels that only a measurement build contains: not among the product sources, refuse to compile without the marker
+    product = {src for sources in build.LIBRARIES.values() for src in sources}
+    for switch, (src, _) in build.MEASUREMENT_SOURCES.items():
+        assert src not in product
+        text = open(os.path.join(ROOT, "luminal.jl_amd", "csrc", src)).read()
+        assert "#error" in text and switch[2:] in text and "LMH_MEASUREMENT_BUILD" in text
 
 
 def test_struct_layout_matches_header(lm):
