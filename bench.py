@@ -146,7 +146,7 @@ def rel_err(got, want):
 
 
 # -------------------------------------------------------------------------------------------------
-def prefill_leg(lm, dev, steps, warmup, cpu_seconds):
+def prefill_leg(lm, dev, steps, warmup, cpu_seconds, zero_operands=True):
     B, H, S, D = 1, 32, 4096, 96
     host = [lm.synth.normal((B, H, S, D), 2000 + i, 0.5).astype(np.float16) for i in range(3)]  # seeds of the C2 parity test
     dq, dk, dv = (lm.HipArray((B, H, S, D), "f16", dev).copy_from_host(x) for x in host)
@@ -162,8 +162,9 @@ def prefill_leg(lm, dev, steps, warmup, cpu_seconds):
         % (wall_ms * 1e3, ev_ms * 1e3, kern_tflops, 100 * kern_tflops / PEAK_FP16_TFLOPS, PEAK_FP16_TFLOPS))
     each = per_launch_us(fn, 20, lm.binding)
     sustained = mfma_sustained(lm, dev, dq)
-    on_zeros = zero_operand_launch_us(lm, dev, p, (B, H, S, D), "f16", steps, warmup)
-    log("[prefill] the same launch on all-zero Q, K, V (same instruction stream, no switching in the data paths): %.1f us" % on_zeros)
+    on_zeros = zero_operand_launch_us(lm, dev, p, (B, H, S, D), "f16", steps, warmup) if zero_operands else None
+    if zero_operands:
+        log("[prefill] the same launch on all-zero Q, K, V (same instruction stream, no switching in the data paths): %.1f us" % on_zeros)
     res = {
         "ms_per_step": wall_ms, "value": tflops,
         "roofline": {"bound": "mfma", "achieved": kern_tflops, "peak": PEAK_FP16_TFLOPS, "unit": "TFLOP/s",
@@ -348,7 +349,7 @@ def c1_leg(lm, dev, res, check):
     res[name]["frac_of_fp32_mfma_peak"] = res[name]["TFLOP/s"] / PEAK_FP32_TFLOPS
 
 
-def nomask_leg(lm, dev, res, check):
+def nomask_leg(lm, dev, res, check, zero_operands=True):
     """The C2 shape without the causal mask (an extra line, not one of the five configurations): every workgroup walks
     all 4096 keys, so the launch is 32 equal tiles per CU and shows the loop's steady state without the diagonal."""
     name = "C2 shape without the mask (fp16 B=1 H=32 S=4096 D=96)"
@@ -362,9 +363,9 @@ def nomask_leg(lm, dev, res, check):
     _, ev = time_steps(fn, 40, 5, lm.binding)
     res[name] = {"launch_us": ev * 1e3, "TFLOP/s": flops / (ev * 1e-3) / 1e12, "frac_of_mfma_peak": flops / (ev * 1e-3) / 1e12 / PEAK_FP16_TFLOPS,
                  "kernel": lm.binding.flash_attn_plan(p),
-                 "launch_us_on_zero_operands": zero_operand_launch_us(lm, dev, p, (B, H, S, D), "f16", 40, 5)}
-    log("[other] %s: %.1f us, %.1f TFLOP/s; on zero operands %.1f us; %s" % (name, ev * 1e3, res[name]["TFLOP/s"],
-                                                                           res[name]["launch_us_on_zero_operands"], res[name]["kernel"]))
+                 "launch_us_on_zero_operands": zero_operand_launch_us(lm, dev, p, (B, H, S, D), "f16", 40, 5) if zero_operands else None}
+    log("[other] %s: %.1f us, %.1f TFLOP/s; on zero operands %s us; %s" % (name, ev * 1e3, res[name]["TFLOP/s"],
+                                                                         res[name]["launch_us_on_zero_operands"], res[name]["kernel"]))
     if check:
         import oracle
         heads = slice(0, 4)
@@ -622,7 +623,7 @@ def ceiling_leg(lm, dev):
     return res
 
 
-def other_configs(lm, dev, check=False, only="other"):
+def other_configs(lm, dev, check=False, only="other", zero_operands=True):
     """Short timings of the remaining contract configurations. With `check`, C1, C3 and C4 are also compared with the
     CPU oracle on the whole output (the parity gate of the five configurations: C2 and C5 are checked in their own
     legs). `only` = "other" runs everything, or one of c1 / nomask / c3 / c4 / ops / step (a profile of one kernel)."""
@@ -631,7 +632,7 @@ def other_configs(lm, dev, check=False, only="other"):
     if only in ("other", "c1"):
         c1_leg(lm, dev, res, check)
     if only in ("other", "nomask"):
-        nomask_leg(lm, dev, res, check)
+        nomask_leg(lm, dev, res, check, zero_operands)
     if only in ("other", "c3"):
         c3_leg(lm, dev, res, check)
     if only in ("other", "c4"):
@@ -689,6 +690,9 @@ def main():
     ap.add_argument("--only", choices=["all", "prefill", "decode", "other", "c1", "nomask", "c3", "c4", "ops", "step", "copy", "ceiling", "grid"], default="all")
     ap.add_argument("--decode-splits", type=int, default=0, help="KV splits for the decode leg (0 = library heuristic)")
     ap.add_argument("--cpu-seconds", type=float, default=15.0, help="CPU-baseline budget per leg; 0 disables it")
+    ap.add_argument("--no-zero-operands", action="store_true",
+                    help="leave out the second timing of the prefill / nomask launch on all-zero tensors (for counter and "
+                         "kernel-trace runs, whose per-kernel averages should cover the workload's launches only)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: the attention path shards over (batch, KV head) with no exchange and "
@@ -722,7 +726,7 @@ def main():
         print(json.dumps(line))
         return
     if args.only in ("all", "prefill"):
-        r = prefill_leg(lm, dev, args.steps, args.warmup, args.cpu_seconds)
+        r = prefill_leg(lm, dev, args.steps, args.warmup, args.cpu_seconds, zero_operands=not args.no_zero_operands)
         line["value"], line["ms_per_step"] = r["value"], r["ms_per_step"]
         line["roofline"] = r["roofline"]
         if "cpu_baseline" in r:
@@ -731,7 +735,8 @@ def main():
     if args.only in ("all", "decode"):
         line["decode"] = decode_leg(lm, dev, args.steps, args.warmup, args.cpu_seconds, args.decode_splits)
     if args.only in ("all", "other", "c1", "nomask", "c3", "c4", "ops", "step"):
-        line["other_configs"] = other_configs(lm, dev, check=args.cpu_seconds > 0, only="other" if args.only == "all" else args.only)
+        line["other_configs"] = other_configs(lm, dev, check=args.cpu_seconds > 0, only="other" if args.only == "all" else args.only,
+                                              zero_operands=not args.no_zero_operands)
     gate = [("C2", line.get("parity"))] + [("C5", line.get("decode", {}).get("parity"))] + \
         [(k.split()[0], v.get("parity")) for k, v in line.get("other_configs", {}).items() if isinstance(v, dict) and "parity" in v]
     gate = [(n, p) for n, p in gate if p]

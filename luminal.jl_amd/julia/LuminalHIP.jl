@@ -489,6 +489,68 @@ function cached_self_attention_core!(out::HipArray{TO,3}, q::HipArray{T,4}, k_ne
     return execute_op!(out, DecodeAttentionOp(s, head_map), q3, kc, vc, kv_len)
 end
 
+# ------------------------------------------------------------------------------------------
+# Device-resident decode cache: the self-attention half of KVCacheState (src/Whisper.jl:519-540; one (K, V) pair of
+# (B, Hkv, max_seq, D) per layer, zero-filled) with the step of decode_step! (src/Whisper.jl:761-801) that concerns it.
+# The reference keeps the caches on the host, feeds them to the step graph as inputs and replaces them by the graph's
+# new-cache outputs every step (:775-797); here they stay on the device, a step writes its rows in place, and every
+# sequence carries its own length (the reference has one step_pos for the batch).
+# ------------------------------------------------------------------------------------------
+mutable struct HipKVCache{T}
+    max_seq::Int
+    self_cache::Vector{Tuple{HipArray{T,4},HipArray{T,4}}}   # per layer, as in KVCacheState
+    kv_len_host::Vector{Int32}                               # rows in use, per sequence (the same in every layer)
+    pos::HipArray{Int32,1}                                   # device copy of kv_len_host before a step ...
+    kv_len::HipArray{Int32,1}                                # ... and after it
+end
+
+"HipKVCache{T}(batch, n_layers, n_kv_heads, head_dim; max_seq): zeroed caches for a new decode session (KVCacheState(...), src/Whisper.jl:527-540)."
+function HipKVCache{T}(batch::Int, n_layers::Int, n_kv_heads::Int, head_dim::Int; max_seq::Int) where {T}
+    caches = [(zeros_hip(T, (batch, n_kv_heads, max_seq, head_dim)), zeros_hip(T, (batch, n_kv_heads, max_seq, head_dim)))
+              for _ in 1:n_layers]
+    return HipKVCache{T}(max_seq, caches, zeros(Int32, batch), zeros_hip(Int32, (batch,)), zeros_hip(Int32, (batch,)))
+end
+
+"The reference's single position (KVCacheState.step_pos): the longest sequence's length."
+step_pos(c::HipKVCache) = Int(maximum(c.kv_len_host))
+
+"""
+begin_step!(cache, n_new): uploads the rows the next `n_new` tokens of every sequence will occupy (pos = the lengths so
+far, kv_len = pos .+ n_new) and returns (pos, kv_len). Call it once per step, before the layers; `advance!` afterwards.
+"""
+function begin_step!(c::HipKVCache, n_new::Integer=1)
+    step_pos(c) + n_new <= c.max_seq || error("KV cache is full (max_seq = $(c.max_seq))")
+    copyto!(c.pos, c.kv_len_host)
+    copyto!(c.kv_len, c.kv_len_host .+ Int32(n_new))
+    return c.pos, c.kv_len
+end
+
+"advance!(cache, n_new): the step is done in every layer (cache.step_pos += 1, src/Whisper.jl:799)."
+function advance!(c::HipKVCache, n_new::Integer=1)
+    c.kv_len_host .+= Int32(n_new)
+    return c
+end
+
+"""
+One layer of a decode step (whisper_self_attn_cached, src/Whisper.jl:584-620): this step's q (B,Hq,1,D) and k_new, v_new
+(B,Hkv,1,D) against layer `layer`'s caches, between begin_step! and advance!. With `rope_base` the new K rows and q are
+rotated at their positions (src/NN.jl:356-358). Returns out (B,Hq,D).
+"""
+function decode_layer!(out::HipArray{TO,3}, c::HipKVCache{T}, layer::Integer, q::HipArray{T,4}, k_new::HipArray{T,4},
+                       v_new::HipArray{T,4}; rope_base=nothing, scale=nothing, head_map::Int32=HEADMAP_INTERLEAVED) where {TO,T}
+    kc, vc = c.self_cache[layer]
+    return cached_self_attention_core!(out, q, k_new, v_new, kc, vc, c.pos, c.kv_len; rope_base=rope_base, scale=scale,
+                                       head_map=head_map)
+end
+
+"The prompt pass of layer `layer` (T tokens per sequence into empty caches), between begin_step!(cache, T) and advance!(cache, T)."
+function prompt_layer!(out::HipArray, c::HipKVCache{T}, layer::Integer, q::HipArray{T,4}, k_new::HipArray{T,4},
+                       v_new::HipArray{T,4}; rope_base=nothing, scale=nothing, head_map::Int32=HEADMAP_INTERLEAVED) where {T}
+    kc, vc = c.self_cache[layer]
+    return prompt_self_attention_core!(out, q, k_new, v_new, kc, vc, c.pos, c.kv_len; rope_base=rope_base, scale=scale,
+                                       head_map=head_map)
+end
+
 # The same two cores as graph builders (GraphTensor in, GraphTensor out), for model code that builds a Luminal graph.
 function self_attention_core(q::GraphTensor, k::GraphTensor, v::GraphTensor; causal::Bool=true, prev_seq::Integer=0,
                              rope_base=nothing, scale=nothing)
@@ -731,6 +793,7 @@ end
 export HIPDevice, HipArray, BF16Bits, release_capture!, enable_capture!, compile_hip, DecodeAttentionOp, decode_attention,
        RotaryEmbeddingOp, rotary_embedding, KVAppendOp, kv_cache_append, get_device, functional, rope!, kv_append!,
        self_attention_core!, cached_self_attention_core!, self_attention_core, cached_self_attention_core, flash_attention_plan,
-       RopeFlashAttentionOp, rope_flash_attention, prompt_self_attention_core!, self_attention, host_fallback
+       RopeFlashAttentionOp, rope_flash_attention, prompt_self_attention_core!, self_attention, host_fallback,
+       HipKVCache, step_pos, begin_step!, advance!, decode_layer!, prompt_layer!
 
 end # module

@@ -270,7 +270,7 @@ def _split_top_level(s):
 def test_glue_ccalls_pass_as_many_arguments_as_the_header_declares():
     code = _strip_julia(glue_text())
     protos = {name: args for name, args in re.findall(r"\b(lmh_\w+)\s*\(([^)]*)\)\s*;", header_text())}
-    seen = 0
+    seen, names = 0, set()
     for m in re.finditer(r"ccall\(", code):
         i, depth = m.end(), 1
         while depth:
@@ -283,8 +283,37 @@ def test_glue_ccalls_pass_as_many_arguments_as_the_header_declares():
         assert len(types) == len(values), "ccall of %s: %d types, %d values" % (name, len(types), len(values))
         declared = [a for a in protos[name].split(",") if a.strip() and a.strip() != "void"]
         assert len(declared) == len(types), "ccall of %s: header declares %d parameters" % (name, len(declared))
+        # ... of the same kinds, in the same order, and the same return type
+        for decl, jl in zip(declared, types):
+            assert jl.strip() in _julia_spellings(decl), "ccall of %s: header parameter %r passed as %s" % (name, decl.strip(), jl.strip())
+        ret = re.search(r"([\w ]+?[ *]+)%s\s*\(" % name, header_text()).group(1)
+        assert parts[1].strip() in _julia_spellings(ret + "x"), "ccall of %s returns %r in the header, %s in the glue" % (name, ret, parts[1])
         seen += 1
+        names.add(name)
     assert seen >= 20
+    assert {"lmh_flash_attn_fwd", "lmh_flash_attn_plan", "lmh_decode_attn", "lmh_decode_attn_static", "lmh_rope", "lmh_kv_append"} <= names
+
+
+def _julia_spellings(c_decl):
+    """The ccall type spellings that fit one C parameter declaration (`const lmh_attn_params *p`, `size_t bytes` ...)."""
+    d = " ".join(c_decl.replace("*", " * ").split())
+    m = re.match(r"(?:const )?(\w+)((?: \*)*) \w+$", d)
+    assert m, c_decl
+    base, stars = m.group(1), m.group(2).count("*")
+    struct = {"lmh_attn_params": "AttnParams", "lmh_decode_params": "DecodeParams", "lmh_rope_params": "RopeParams",
+              "lmh_kv_append_params": "KvAppendParams"}
+    if base in struct:
+        assert stars == 1
+        return {"Ref{%s}" % struct[base]}
+    if stars == 0:
+        return {"int": {"Cint", "Int32"}, "int32_t": {"Int32", "Cint"}, "size_t": {"Csize_t"}, "float": {"Float32", "Cfloat"}}[base]
+    if base == "void":
+        return {"Ptr{Cvoid}"} if stars == 1 else {"Ref{Ptr{Cvoid}}", "Ptr{Ptr{Cvoid}}"}
+    if base == "char":
+        return {"Ptr{UInt8}", "Cstring"}
+    if base == "float":
+        return {"Ref{Float32}", "Ptr{Float32}"}
+    raise AssertionError("no Julia spelling known for %r" % c_decl)
 
 
 def test_glue_host_fallback_and_layer_builder():
@@ -313,3 +342,28 @@ def test_glue_host_fallback_and_layer_builder():
         nn = open(os.path.join(REFERENCE, "src/NN.jl")).read()
         assert "Luminal.reshape(sa.q_proj(x), [batch, seq, sa.n_heads, sa.head_dim])" in nn
         assert "Luminal.permute(queries, [1, 3, 2, 4])" in nn and "Luminal.reshape(out, [batch, seq, hidden])" in nn
+
+
+def test_glue_device_cache_mirrors_the_reference_cache_holder():
+    """HipKVCache keeps what KVCacheState keeps for self attention (reference src/Whisper.jl:519-540: max_seq, one (K, V)
+    pair per layer, zero-filled (B, H, max_seq, D)) and its step functions hand the cores exactly the keywords they take."""
+    text = glue_text()
+    st = re.search(r"^mutable struct HipKVCache\{T\}\n(.*?)^end$", text, flags=re.M | re.S).group(1)
+    for field in ("max_seq::Int", "self_cache::Vector{Tuple{HipArray{T,4},HipArray{T,4}}}", "kv_len_host::Vector{Int32}",
+                  "pos::HipArray{Int32,1}", "kv_len::HipArray{Int32,1}"):
+        assert field in st, field
+    ctor = re.search(r"^function HipKVCache\{T\}\(.*?^end$", text, flags=re.M | re.S).group(0)
+    assert ctor.count("zeros_hip(T, (batch, n_kv_heads, max_seq, head_dim))") == 2 and "for _ in 1:n_layers" in ctor
+    for fn, core in (("decode_layer!", "cached_self_attention_core!"), ("prompt_layer!", "prompt_self_attention_core!")):
+        body = re.search(r"^function %s\(.*?^end$" % re.escape(fn), text, flags=re.M | re.S).group(0)
+        call = re.search(r"%s\((.*?)\)\nend" % re.escape(core), body, flags=re.S).group(1)
+        sig = re.search(r"^function %s\((.*?)\) where" % re.escape(core), text, flags=re.M | re.S).group(1)
+        positional, keywords = sig.split(";")
+        assert len(_split_top_level(call.split(";")[0])) == len(_split_top_level(positional)), fn
+        for kw in re.findall(r"(\w+)=", call.split(";")[1]):
+            assert re.search(r"\b%s(::\w+)?=" % kw, keywords), (fn, kw)
+    begin = re.search(r"^function begin_step!\(.*?^end$", text, flags=re.M | re.S).group(0)
+    assert "copyto!(c.pos, c.kv_len_host)" in begin and "c.kv_len_host .+ Int32(n_new)" in begin and "error(" in begin
+    if os.path.isdir(REFERENCE):
+        wh = open(os.path.join(REFERENCE, "src/Whisper.jl")).read()
+        assert "self_cache::Vector{Tuple{Array{Float32,4}, Array{Float32,4}}}" in wh and "cache.step_pos += 1" in wh
