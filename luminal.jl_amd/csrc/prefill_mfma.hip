@@ -24,6 +24,8 @@
 //     lie entirely above its diagonal, and only diagonal tiles pay for masking;
 //   * blockIdx -> work mapping keeps all query tiles of a head on one XCD (private L2) and, for
 //     causal, issues the long rows first.
+#include <type_traits>
+
 #include "prefill_mfma.hpp"
 #include "rope.hpp"
 
@@ -45,10 +47,17 @@ namespace {
 // depend on the row: the workgroup computes its D/2 values once into `table` (LDS that nothing else uses before the
 // next barrier) and every lane multiplies them by its own position. Every thread of the workgroup must call this.
 template <typename MT, int D>
+__device__ inline void rotate_q_fragments_with_table(typename MT::vec8 (&qreg)[D / 16], const PrefillArgs &a, int b, int qi, int g, const float *table);
+template <typename MT, int D>
 __device__ inline void rotate_q_fragments(typename MT::vec8 (&qreg)[D / 16], const PrefillArgs &a, int b, int qi, int g, float *table) {
-  constexpr int KS = D / 16, HK = D / 32;
   if ((int)threadIdx.x < D / 2) table[threadIdx.x] = rope_inv_freq(threadIdx.x, D, a.q_log2_base);
   __syncthreads();
+  rotate_q_fragments_with_table<MT, D>(qreg, a, b, qi, g, table);
+}
+// the rotation itself, given the workgroup's table of D / 2 inverse frequencies
+template <typename MT, int D>
+__device__ inline void rotate_q_fragments_with_table(typename MT::vec8 (&qreg)[D / 16], const PrefillArgs &a, int b, int qi, int g, const float *table) {
+  constexpr int KS = D / 16, HK = D / 32;
   const float pos = (float)((a.q_pos0 ? a.q_pos0[b] : a.q_prev_seq) + qi);
   if (!a.q_interleaved) {
 #pragma unroll
@@ -707,6 +716,383 @@ __global__ __launch_bounds__(1024, 4) void prefill_mfma_wide_kernel(PrefillArgs 
   }
 }
 
+// ---------------------------------------------------------------------------------------------------------------
+// Causal launches whose query tiles are few enough to matter one by one: a workgroup of 8 waves owns TWO 256-row query
+// tiles of one (b, hq) — tile p and tile n - 1 - p — so that every workgroup of the launch walks the same number of keys
+// (the short rows of the early tile plus the long rows of the late one), one workgroup per CU, no second round and no
+// tail. Wave w carries rows 32 w .. of the early tile (row block 0) and rows 32 w .. of the late tile (row block 1).
+// While the keys are visible to both tiles, every K and V^T fragment the wave reads from LDS feeds two MFMAs, one per
+// row block (half the LDS reads per MFMA of the kernel above); past the early tile's diagonal the wave stores that
+// tile's rows and goes on with the late tile alone. K/V tiles are staged once for both query tiles.
+// ---------------------------------------------------------------------------------------------------------------
+template <typename MT, int D>
+__global__ __launch_bounds__(512, 2) void prefill_mfma_pair_kernel(PrefillArgs a, int n_q_tiles, int n_bh_groups) {
+  using vec8 = typename MT::vec8;
+  static_assert(!MT::kSplitP, "head + remainder weights do not fit the register budget of two row blocks");
+  constexpr int NW = 8, BM = 256;
+  constexpr int BT = 2 * BN;        // 128 keys per staged tile
+  constexpr int NKB = BT / 32;
+  constexpr int KS = D / 16, DB = D / 32;
+  const int cpr = a.D / 8;
+  constexpr int LDK = D + kPadK, LDV = D + pad_v<D>();
+
+  __shared__ __attribute__((aligned(16))) uint16_t Ks2[2][BT * LDK];
+  __shared__ __attribute__((aligned(16))) uint16_t Vs2[2][BT * LDV];
+
+  const int bid = blockIdx.x;
+  const int xcd = bid & 7, idx = bid >> 3;
+  const int pair = idx / n_bh_groups;
+  const int bh = (idx % n_bh_groups) * 8 + xcd;
+  if (bh >= a.B * a.Hq) return;
+  const int b = bh / a.Hq, hq = bh % a.Hq;
+  const int kvh = kv_head_of(hq, a.Hq, a.Hkv, a.head_map);
+  // tile p with tile n - 1 - p; with an odd number of tiles the middle one is alone (its workgroup has no early tile)
+  const int t_late = n_q_tiles - 1 - pair, t_early = pair;
+  const bool has_early = t_early < t_late;
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63, wave = tid >> 6;
+  const int n = lane & 31, g = lane >> 5;
+  // rows of this wave: qlo[rb] .. qlo[rb] + 31; without an early tile row block 0 lies past the last query
+  int qlo[2];
+  qlo[0] = has_early ? t_early * BM + 32 * wave : a.Sq + 64;
+  qlo[1] = t_late * BM + 32 * wave;
+
+  int n_keys = a.kv_len ? a.kv_len[b] : a.Sk;
+  n_keys = min(max(n_keys, 0), a.Sk);
+  const int k_end_early = has_early ? min(n_keys, (t_early + 1) * BM) : 0;   // keys the early tile can see
+  const int k_end_late = min(n_keys, (t_late + 1) * BM);
+  const int n_tiles_early = (k_end_early + BT - 1) / BT;
+  const int n_tiles_late = (k_end_late + BT - 1) / BT;
+
+  const uint16_t *qp = reinterpret_cast<const uint16_t *>(a.q) + b * a.qs[0] + hq * a.qs[1];
+  const uint16_t *kp = reinterpret_cast<const uint16_t *>(a.k) + b * a.ks[0] + kvh * a.ks[1];
+  const uint16_t *vp = reinterpret_cast<const uint16_t *>(a.v) + b * a.vs[0] + kvh * a.vs[1];
+
+  vec8 qreg[2][KS];
+#pragma unroll
+  for (int rb = 0; rb < 2; rb++) {
+    const int qi = qlo[rb] + n;
+#pragma unroll
+    for (int ks = 0; ks < KS; ks++) {
+      uint4 raw = make_uint4(0, 0, 0, 0);
+      if (qi < a.Sq && 16 * ks + 8 * g < a.D) raw = *reinterpret_cast<const uint4 *>(qp + (int64_t)qi * a.qs[2] + 16 * ks + 8 * g);
+      qreg[rb][ks] = __builtin_bit_cast(vec8, raw);
+    }
+  }
+
+  floatx16_t oacc[2][DB];
+#pragma unroll
+  for (int rb = 0; rb < 2; rb++)
+#pragma unroll
+    for (int db = 0; db < DB; db++)
+#pragma unroll
+      for (int i = 0; i < 16; i++) oacc[rb][db][i] = 0.f;
+  float m_i[2] = {-INFINITY, -INFINITY}, l_i[2] = {0.f, 0.f};
+  const float c = a.scale * kLog2e;
+
+  // ---- tile staging, as in prefill_mfma_kernel ----
+  typedef int32_t i32x4_t __attribute__((ext_vector_type(4)));
+  typedef __attribute__((address_space(3))) void lds_void_t;
+  constexpr int KC = LDK / 8, VC = LDV / 8;
+  constexpr int KI = KC * BT / 64, VI = VC * BT / 64;
+  constexpr int KJ = (KI + NW - 1) / NW, VJ = (VI + NW - 1) / NW;
+  const int wave_u = __builtin_amdgcn_readfirstlane(wave);
+  __builtin_assume(wave_u >= 0 && wave_u < NW);
+  auto make_desc = [](const uint16_t *base, int bytes) {
+    const uint64_t p = (uint64_t)base;
+    i32x4_t d;
+    d[0] = __builtin_amdgcn_readfirstlane((int)(uint32_t)p);
+    d[1] = __builtin_amdgcn_readfirstlane((int)((p >> 32) & 0xffff));
+    d[2] = __builtin_amdgcn_readfirstlane(bytes);
+    d[3] = 0x00020000;
+    return d;
+  };
+  const i32x4_t k_desc = make_desc(kp, (int)((int64_t)n_keys * a.ks[2] * 2));
+  const i32x4_t v_desc = make_desc(vp, (int)((int64_t)n_keys * a.vs[2] * 2));
+  int k_voff[KJ], v_voff[VJ];
+#pragma unroll
+  for (int j = 0; j < KJ; j++) {
+    const int ch = (wave + NW * j) * 64 + lane;
+    const int row = ch / KC, col = ch % KC;
+    k_voff[j] = col < cpr ? (int)((row * a.ks[2] + col * 8) * 2) : kOutOfRange;
+  }
+#pragma unroll
+  for (int j = 0; j < VJ; j++) {
+    const int ch = (wave + NW * j) * 64 + lane;
+    const int row = ch / VC, col = ch % VC;
+    v_voff[j] = col < cpr ? (int)((row * a.vs[2] + col * 8) * 2) : kOutOfRange;
+  }
+  const int k_tile_bytes = (int)(BT * a.ks[2] * 2), v_tile_bytes = (int)(BT * a.vs[2] * 2);
+  const uint32_t k_lds0 = (uint32_t)(uintptr_t)(lds_void_t *)&Ks2[0][0] + wave_u * 1024;
+  const uint32_t v_lds0 = (uint32_t)(uintptr_t)(lds_void_t *)&Vs2[0][0] + wave_u * 1024;
+#pragma clang diagnostic push
+#pragma clang diagnostic ignored "-Winline-asm"
+  auto load_block = [](i32x4_t desc, uint32_t lds_addr, int voff, int soff) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
+                 :: "s"(lds_addr), "v"(voff), "s"(desc), "s"(soff) : "memory", "m0");
+  };
+#pragma clang diagnostic pop
+  auto load_tile = [&](int kt, int buf) {
+#pragma unroll
+    for (int j = 0; j < KJ; j++)
+      if (wave_u + NW * j < KI)
+        load_block(k_desc, k_lds0 + buf * (BT * LDK * 2) + j * (NW * 1024), k_voff[j], kt * k_tile_bytes);
+#pragma unroll
+    for (int j = 0; j < VJ; j++)
+      if (wave_u + NW * j < VI)
+        load_block(v_desc, v_lds0 + buf * (BT * LDV * 2) + j * (NW * 1024), v_voff[j], kt * v_tile_bytes);
+  };
+
+  const int k_frag_off = n * LDK + 8 * g;
+  const int i16 = lane & 15;
+  const int v_frag_off = (4 * g + (i16 >> 2)) * LDV + 16 * ((lane >> 4) & 1) + 4 * (i16 & 3);
+
+  if (n_tiles_late > 0) load_tile(0, 0);
+  if (a.q_rope) {
+    float *table = reinterpret_cast<float *>(&Ks2[1][0]);
+    if ((int)threadIdx.x < D / 2) table[threadIdx.x] = rope_inv_freq(threadIdx.x, D, a.q_log2_base);
+    __syncthreads();
+#pragma unroll
+    for (int rb = 0; rb < 2; rb++) rotate_q_fragments_with_table<MT, D>(qreg[rb], a, b, qlo[rb] + n, g, table);
+  }
+#pragma unroll
+  for (int rb = 0; rb < 2; rb++)
+#pragma unroll
+    for (int ks = 0; ks < KS; ks++) asm volatile("" :: "v"(qreg[rb][ks]));
+
+  // One 32-key block at key k0 for row blocks RB0 .. 1 (RB0 = 0: both, every fragment read feeds two MFMAs; RB0 = 1: the
+  // late tile alone). Online softmax per row block as in prefill_mfma_kernel.
+  auto block = [&](auto rb0_c, auto nb_c, const uint16_t *Kb, const uint16_t *Vb, int k0) {
+    constexpr int RB0 = decltype(rb0_c)::value;
+    constexpr int NB = decltype(nb_c)::value;  // 32-key blocks taken together
+    floatx16_t sacc[2][NB];
+#pragma unroll
+    for (int rb = RB0; rb < 2; rb++)
+#pragma unroll
+      for (int kb = 0; kb < NB; kb++)
+#pragma unroll
+        for (int i = 0; i < 16; i++) sacc[rb][kb][i] = 0.f;
+#pragma unroll
+    for (int ks = 0; ks < KS; ks++)
+#pragma unroll
+      for (int kb = 0; kb < NB; kb++) {
+        const vec8 kf = *reinterpret_cast<const vec8 *>(&Kb[k_frag_off + kb * 32 * LDK + 16 * ks]);
+#pragma unroll
+        for (int rb = RB0; rb < 2; rb++) sacc[rb][kb] = MT::mfma(kf, qreg[rb][ks], sacc[rb][kb]);
+      }
+    vec8 pf[2][NB][2];
+#pragma unroll
+    for (int rb = RB0; rb < 2; rb++) {
+      if (k0 + 32 * NB > n_keys || k0 + 32 * NB - 1 > qlo[rb]) {  // the ragged last block, or a block on this row block's diagonal
+        const int qi = qlo[rb] + n;
+#pragma unroll
+        for (int kb = 0; kb < NB; kb++)
+#pragma unroll
+          for (int i = 0; i < 16; i++) {
+            const int key = k0 + 32 * kb + 8 * (i >> 2) + 4 * g + (i & 3);
+            if (key >= n_keys || key > qi) sacc[rb][kb][i] = -INFINITY;
+          }
+      }
+      float mx = sacc[rb][0][0];
+#pragma unroll
+      for (int kb = 0; kb < NB; kb++)
+#pragma unroll
+        for (int i = 0; i < 16; i++) mx = fmaxf(mx, sacc[rb][kb][i]);
+      mx = max_over_wave_halves(mx);
+      // (key 0 is visible to every query, so m is finite after the first block)
+      if (__builtin_amdgcn_ballot_w64((mx - m_i[rb]) * c > kLazyRescale) != 0) {
+        const float m_new = fmaxf(m_i[rb], mx);
+        const float alpha = __builtin_amdgcn_exp2f((m_i[rb] - m_new) * c);
+        m_i[rb] = m_new;
+        l_i[rb] *= alpha;
+#pragma unroll
+        for (int db = 0; db < DB; db++)
+#pragma unroll
+          for (int i = 0; i < 16; i++) oacc[rb][db][i] *= alpha;
+      }
+      const float mc = m_i[rb] * c;
+#pragma unroll
+      for (int kb = 0; kb < NB; kb++)
+#pragma unroll
+        for (int t = 0; t < 2; t++) {
+#pragma unroll
+          for (int e = 0; e < 8; e++) pf[rb][kb][t][e] = MT::cvt(__builtin_amdgcn_exp2f(sacc[rb][kb][8 * t + e] * c - mc));
+          l_i[rb] = MT::sum8(pf[rb][kb][t], l_i[rb]);
+        }
+    }
+#pragma unroll
+    for (int kb = 0; kb < NB; kb++)
+#pragma unroll
+      for (int t = 0; t < 2; t++)
+#pragma unroll
+        for (int db = 0; db < DB; db++) {
+          const uint16_t *vaddr = &Vb[v_frag_off + (32 * kb + 16 * t) * LDV + db * 32];
+          const shortx4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_shortx4_t *)(vaddr));
+          const shortx4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_shortx4_t *)(vaddr + 8 * LDV));
+          const vec8 v8 = __builtin_bit_cast(vec8, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+#pragma unroll
+          for (int rb = RB0; rb < 2; rb++) oacc[rb][db] = MT::mfma(v8, pf[rb][kb][t], oacc[rb][db]);
+        }
+  };
+  auto store_rows = [&](int rb) {
+    const int qi = qlo[rb] + n;
+    const float l_tot = sum_over_wave_halves(l_i[rb]);
+    const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
+    if (qi < a.Sq) {
+      const int64_t off = b * a.os[0] + hq * a.os[1] + (int64_t)qi * a.os[2];
+      uint16_t *op = reinterpret_cast<uint16_t *>(a.out) + off;
+      float *op32 = reinterpret_cast<float *>(a.out) + off;
+#pragma unroll
+      for (int db = 0; db < DB; db++)
+#pragma unroll
+        for (int i4 = 0; i4 < 4; i4++) {
+          const int d = db * 32 + 8 * i4 + 4 * g;
+          if (d >= a.D) continue;
+          if (a.out_f32) {
+            *reinterpret_cast<float4 *>(op32 + d) =
+                make_float4(oacc[rb][db][4 * i4 + 0] * inv, oacc[rb][db][4 * i4 + 1] * inv, oacc[rb][db][4 * i4 + 2] * inv,
+                            oacc[rb][db][4 * i4 + 3] * inv);
+            continue;
+          }
+          uint2 packed;
+          packed.x = (uint32_t)MT::cvt_bits(oacc[rb][db][4 * i4 + 0] * inv) |
+                     ((uint32_t)MT::cvt_bits(oacc[rb][db][4 * i4 + 1] * inv) << 16);
+          packed.y = (uint32_t)MT::cvt_bits(oacc[rb][db][4 * i4 + 2] * inv) |
+                     ((uint32_t)MT::cvt_bits(oacc[rb][db][4 * i4 + 3] * inv) << 16);
+          *reinterpret_cast<uint2 *>(op + d) = packed;
+        }
+    }
+  };
+  // A whole 128-key tile for the late row block alone: the loop body of prefill_mfma_kernel (four 32-key blocks at a
+  // time, their QK^T chains alternating two by two, one softmax pass over all 64 scores of a lane).
+  auto tile_late = [&](const uint16_t *Ks, const uint16_t *Vs, int k0) {
+    constexpr int rb = 1;
+    if (k0 > qlo[rb] + 31) return;  // the whole tile lies above this wave's rows
+    floatx16_t sacc[NKB];
+#pragma unroll
+    for (int kb = 0; kb < NKB; kb++)
+#pragma unroll
+      for (int i = 0; i < 16; i++) sacc[kb][i] = 0.f;
+#pragma unroll
+    for (int kb0 = 0; kb0 < NKB; kb0 += 2) {
+      vec8 kf[2][KS];
+#pragma unroll
+      for (int ks = 0; ks < KS; ks++)
+#pragma unroll
+        for (int kb = 0; kb < 2; kb++)
+          kf[kb][ks] = *reinterpret_cast<const vec8 *>(&Ks[k_frag_off + (kb0 + kb) * 32 * LDK + 16 * ks]);
+#pragma unroll
+      for (int ks = 0; ks < KS; ks++)
+#pragma unroll
+        for (int kb = 0; kb < 2; kb++) sacc[kb0 + kb] = MT::mfma(kf[kb][ks], qreg[rb][ks], sacc[kb0 + kb]);
+    }
+    if (k0 + BT > n_keys || k0 + BT - 1 > qlo[rb]) {
+      const int qi = qlo[rb] + n;
+#pragma unroll
+      for (int kb = 0; kb < NKB; kb++)
+#pragma unroll
+        for (int i = 0; i < 16; i++) {
+          const int key = k0 + kb * 32 + 8 * (i >> 2) + 4 * g + (i & 3);
+          if (key >= n_keys || key > qi) sacc[kb][i] = -INFINITY;
+        }
+    }
+    float mx = sacc[0][0];
+#pragma unroll
+    for (int kb = 0; kb < NKB; kb++)
+#pragma unroll
+      for (int i = 0; i < 16; i++) mx = fmaxf(mx, sacc[kb][i]);
+    mx = max_over_wave_halves(mx);
+    if (__builtin_amdgcn_ballot_w64((mx - m_i[rb]) * c > kLazyRescale) != 0) {
+      const float m_new = fmaxf(m_i[rb], mx);
+      const float alpha = __builtin_amdgcn_exp2f((m_i[rb] - m_new) * c);
+      m_i[rb] = m_new;
+      l_i[rb] *= alpha;
+#pragma unroll
+      for (int db = 0; db < DB; db++)
+#pragma unroll
+        for (int i = 0; i < 16; i++) oacc[rb][db][i] *= alpha;
+    }
+    const float mc = m_i[rb] * c;
+    vec8 pf[NKB][2];
+#pragma unroll
+    for (int kb = 0; kb < NKB; kb++)
+#pragma unroll
+      for (int t = 0; t < 2; t++) {
+#pragma unroll
+        for (int e = 0; e < 8; e++) pf[kb][t][e] = MT::cvt(__builtin_amdgcn_exp2f(sacc[kb][8 * t + e] * c - mc));
+        l_i[rb] = MT::sum8(pf[kb][t], l_i[rb]);
+      }
+#pragma unroll
+    for (int kb = 0; kb < NKB; kb++)
+#pragma unroll
+      for (int t = 0; t < 2; t++)
+#pragma unroll
+        for (int db = 0; db < DB; db++) {
+          const uint16_t *vaddr = &Vs[v_frag_off + (kb * 32 + 16 * t) * LDV + db * 32];
+          const shortx4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_shortx4_t *)(vaddr));
+          const shortx4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_shortx4_t *)(vaddr + 8 * LDV));
+          const vec8 v8 = __builtin_bit_cast(vec8, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+          oacc[rb][db] = MT::mfma(v8, pf[kb][t], oacc[rb][db]);
+        }
+  };
+  const std::integral_constant<int, 0> kBoth{};
+  const std::integral_constant<int, 1> kLate{};
+
+  // ---- keys the early tile sees: both row blocks ----
+  for (int kt = 0; kt < n_tiles_early; kt++) {
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    if (kt + 1 < n_tiles_late) load_tile(kt + 1, (kt + 1) & 1);
+    const uint16_t *Ks = Ks2[kt & 1];
+    const uint16_t *Vs = Vs2[kt & 1];
+    constexpr int NB = 2;  // two 32-key blocks of both row blocks at a time: four score blocks in flight, 244 registers
+    const std::integral_constant<int, NB> kNB{};
+    const std::integral_constant<int, 1> kOne{};
+#pragma unroll
+    for (int kb = 0; kb < NKB; kb += NB) {
+      const int k0 = kt * BT + kb * 32;
+      if (k0 >= k_end_late) break;
+      if (k0 + 32 * NB - 1 <= qlo[0] && k0 + 32 * NB <= k_end_early) {   // the whole group below the early rows' diagonal
+        block(kBoth, kNB, Ks + kb * 32 * LDK, Vs + kb * 32 * LDV, k0);
+      } else {
+#pragma unroll
+        for (int j = 0; j < NB; j++) {
+          const int kj = k0 + 32 * j;
+          if (kj >= k_end_late) break;
+          if (kj <= qlo[0] + 31 && kj < k_end_early)
+            block(kBoth, kOne, Ks + (kb + j) * 32 * LDK, Vs + (kb + j) * 32 * LDV, kj);
+          else
+            block(kLate, kOne, Ks + (kb + j) * 32 * LDK, Vs + (kb + j) * 32 * LDV, kj);
+        }
+      }
+    }
+  }
+  if (has_early) store_rows(0);
+  // ---- the rest: the late tile alone ----
+  for (int kt = n_tiles_early; kt < n_tiles_late; kt++) {
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    if (kt + 1 < n_tiles_late) load_tile(kt + 1, (kt + 1) & 1);
+    const uint16_t *Ks = Ks2[kt & 1];
+    const uint16_t *Vs = Vs2[kt & 1];
+    tile_late(Ks, Vs, kt * BT);
+  }
+  store_rows(1);
+}
+
+template <typename MT, int D>
+int launch_pair(const PrefillArgs &a, hipStream_t stream) {
+  const int n_q_tiles = (a.Sq + 255) / 256;
+  const int n_pairs = (n_q_tiles + 1) / 2;
+  const int n_bh_groups = (a.B * a.Hq + 7) / 8;
+  dim3 grid(8 * n_bh_groups * n_pairs), block(512);
+  if (plan_only("prefill_mfma_pair_kernel<%s, D=%d> query tiles=%d, workgroups=%u", MT::kName, D, n_q_tiles, grid.x)) return LMH_OK;
+  hipLaunchKernelGGL((prefill_mfma_pair_kernel<MT, D>), grid, block, 0, stream, a, n_q_tiles, n_bh_groups);
+  LMH_HIP_TRY(hipGetLastError());
+  return LMH_OK;
+}
+
 template <typename MT, int D, int KSPLIT, int NW, int WPS = default_wps<D, NW>()>
 int launch_split(const PrefillArgs &a, hipStream_t stream) {
   constexpr int BM = 32 * NW / KSPLIT;
@@ -773,6 +1159,15 @@ int launch_for_d(const PrefillArgs &a, hipStream_t stream) {
   // 46.7 us at B=1 H=32 S=2048 D=96) and loses for non-causal ones (79.8 vs 66.6 us); at three per
   // CU it loses for both.
   const int n_cus = device_cu_count();
+  // Causal launches that are exactly one round of paired 256-row tiles (tile p with tile n - 1 - p: equal work in every
+  // workgroup, one per CU): the Phi-3 prompt, 32 heads x 16 tiles = 256 pairs. Measured against the kernels below on
+  // 256 CUs, fp16: B=1 H=32 S=4096 D=96 -3.2 %, D=64 -6 %, D=80 -3 %; B=2 H=32 S=2048 -5 %; H=8 S=16384 -4.6 %;
+  // S=3900 -2 %. With the chip not exactly full it loses (1.25 rounds +23 %, 1.5 rounds +10 %, half a round +30 %),
+  // at exactly two rounds it ties (-1.4 ... +7 %).
+  if constexpr (D <= 96 && !MT::kSplitP) {
+    const int64_t wgs_pair = (int64_t)((a.B * a.Hq + 7) / 8) * 8 * (((a.Sq + 255) / 256 + 1) / 2);
+    if (a.causal && a.Sq > 256 && wgs_pair <= n_cus && 16 * wgs_pair >= 15 * n_cus) return launch_pair<MT, D>(a, stream);
+  }
   const int64_t wgs = (int64_t)((a.B * a.Hq + 7) / 8) * 8 * ((a.Sq + 127) / 128);
   const int64_t limit = a.causal ? 2 * n_cus : 2 * n_cus - 1;
   if (wgs <= limit && a.Sk >= 4 * BN) {

@@ -170,9 +170,15 @@ def test_kernel_plan_of_the_benchmark_configurations(lm):
     plan = lm.flash_attention_plan
     # C1: the reference's own fp32 example, far too small to fill the chip -> fp32 matrix cores, keys split four ways
     assert plan((1, 8, 128, 64), (1, 8, 128, 64), "f32", True).startswith("prefill_f32_kernel<D=64, causal, key groups=4>")
-    # C2: 512 workgroups of 256 rows, one per CU at a time, 128-key tiles
-    assert plan((1, 32, 4096, 96), (1, 32, 4096, 96), "f16", True).startswith(
-        "prefill_mfma_kernel<f16, D=96, causal, key groups=1, waves=8, waves per SIMD=2> workgroups=512")
+    # C2: 32 heads x 16 tiles of 256 rows = 256 pairs (tile p with tile 15 - p), one workgroup per CU, one round
+    assert plan((1, 32, 4096, 96), (1, 32, 4096, 96), "f16", True) == \
+        "prefill_mfma_pair_kernel<f16, D=96> query tiles=16, workgroups=256"
+    # the same in bf16 (head + remainder weights: no room for two row blocks), or with the chip not exactly full:
+    # 512 workgroups of 256 rows, one per CU at a time, 128-key tiles
+    assert plan((1, 32, 4096, 96), (1, 32, 4096, 96), "bf16", True).startswith(
+        "prefill_mfma_kernel<bf16, D=96, causal, key groups=1, waves=8, waves per SIMD=2> workgroups=512")
+    assert plan((1, 40, 4096, 96), (1, 40, 4096, 96), "f16", True).startswith(
+        "prefill_mfma_kernel<f16, D=96, causal, key groups=1, waves=8, waves per SIMD=2> workgroups=640")
     # C3: 80 heads x 14 row blocks on 256 CUs -> three workgroups per head of five row blocks x three key groups
     assert plan((4, 20, 448, 64), (4, 20, 1500, 64), "f16", False) == \
         "prefill_mfma_wide_kernel<f16, D=64> workgroups per head=3, waves=15, workgroups=240"
