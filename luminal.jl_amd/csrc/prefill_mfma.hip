@@ -1076,7 +1076,18 @@ __global__ __launch_bounds__(512, 2) void prefill_mfma_pair_kernel(PrefillArgs a
     if (kt + 1 < n_tiles_late) load_tile(kt + 1, (kt + 1) & 1);
     const uint16_t *Ks = Ks2[kt & 1];
     const uint16_t *Vs = Vs2[kt & 1];
-    tile_late(Ks, Vs, kt * BT);
+    if (kt * BT + BT - 1 > qlo[1]) {
+      // a tile on the late rows' diagonal: block by block, so that blocks above the wave's rows are skipped (four at a
+      // time they would be computed and masked: 109.9 -> 108.7 us on B=1 H=32 S=4096 D=96)
+#pragma unroll
+      for (int kb = 0; kb < NKB; kb++) {
+        const int k0 = kt * BT + kb * 32;
+        if (k0 > qlo[1] + 31 || k0 >= k_end_late) break;
+        block(kLate, std::integral_constant<int, 1>{}, Ks + kb * 32 * LDK, Vs + kb * 32 * LDV, k0);
+      }
+    } else {
+      tile_late(Ks, Vs, kt * BT);
+    }
   }
   store_rows(1);
 }
