@@ -724,8 +724,9 @@ __global__ __launch_bounds__(1024, 4) void prefill_mfma_wide_kernel(PrefillArgs 
 // While the keys are visible to both tiles, every K and V^T fragment the wave reads from LDS feeds two MFMAs, one per
 // row block (half the LDS reads per MFMA of the kernel above); past the early tile's diagonal the wave stores that
 // tile's rows and goes on with the late tile alone. K/V tiles are staged once for both query tiles.
+// Without a mask (CAUSAL = false) the two tiles are neighbours — a 512-row tile — and share every fragment to the end.
 // ---------------------------------------------------------------------------------------------------------------
-template <typename MT, int D>
+template <typename MT, int D, bool CAUSAL>
 __global__ __launch_bounds__(512, 2) void prefill_mfma_pair_kernel(PrefillArgs a, int n_q_tiles, int n_bh_groups) {
   using vec8 = typename MT::vec8;
   static_assert(!MT::kSplitP, "head + remainder weights do not fit the register budget of two row blocks");
@@ -747,8 +748,9 @@ __global__ __launch_bounds__(512, 2) void prefill_mfma_pair_kernel(PrefillArgs a
   const int b = bh / a.Hq, hq = bh % a.Hq;
   const int kvh = kv_head_of(hq, a.Hq, a.Hkv, a.head_map);
   // tile p with tile n - 1 - p; with an odd number of tiles the middle one is alone (its workgroup has no early tile)
-  const int t_late = n_q_tiles - 1 - pair, t_early = pair;
-  const bool has_early = t_early < t_late;
+  // (without a mask: two neighbouring tiles; the second one, row block 0 here, is missing at an odd end)
+  const int t_late = CAUSAL ? n_q_tiles - 1 - pair : 2 * pair, t_early = CAUSAL ? pair : 2 * pair + 1;
+  const bool has_early = CAUSAL ? t_early < t_late : t_early < n_q_tiles;
 
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = tid >> 6;
@@ -760,8 +762,8 @@ __global__ __launch_bounds__(512, 2) void prefill_mfma_pair_kernel(PrefillArgs a
 
   int n_keys = a.kv_len ? a.kv_len[b] : a.Sk;
   n_keys = min(max(n_keys, 0), a.Sk);
-  const int k_end_early = has_early ? min(n_keys, (t_early + 1) * BM) : 0;   // keys the early tile can see
-  const int k_end_late = min(n_keys, (t_late + 1) * BM);
+  const int k_end_early = !has_early ? 0 : CAUSAL ? min(n_keys, (t_early + 1) * BM) : n_keys;   // keys the early tile can see
+  const int k_end_late = CAUSAL ? min(n_keys, (t_late + 1) * BM) : n_keys;
   const int n_tiles_early = (k_end_early + BT - 1) / BT;
   const int n_tiles_late = (k_end_late + BT - 1) / BT;
 
@@ -884,14 +886,14 @@ __global__ __launch_bounds__(512, 2) void prefill_mfma_pair_kernel(PrefillArgs a
     vec8 pf[2][NB][2];
 #pragma unroll
     for (int rb = RB0; rb < 2; rb++) {
-      if (k0 + 32 * NB > n_keys || k0 + 32 * NB - 1 > qlo[rb]) {  // the ragged last block, or a block on this row block's diagonal
+      if (k0 + 32 * NB > n_keys || (CAUSAL && k0 + 32 * NB - 1 > qlo[rb])) {  // the ragged last block, or a block on this row block's diagonal
         const int qi = qlo[rb] + n;
 #pragma unroll
         for (int kb = 0; kb < NB; kb++)
 #pragma unroll
           for (int i = 0; i < 16; i++) {
             const int key = k0 + 32 * kb + 8 * (i >> 2) + 4 * g + (i & 3);
-            if (key >= n_keys || key > qi) sacc[rb][kb][i] = -INFINITY;
+            if (key >= n_keys || (CAUSAL && key > qi)) sacc[rb][kb][i] = -INFINITY;
           }
       }
       float mx = sacc[rb][0][0];
@@ -968,7 +970,7 @@ __global__ __launch_bounds__(512, 2) void prefill_mfma_pair_kernel(PrefillArgs a
   // time, their QK^T chains alternating two by two, one softmax pass over all 64 scores of a lane).
   auto tile_late = [&](const uint16_t *Ks, const uint16_t *Vs, int k0) {
     constexpr int rb = 1;
-    if (k0 > qlo[rb] + 31) return;  // the whole tile lies above this wave's rows
+    if (CAUSAL && k0 > qlo[rb] + 31) return;  // the whole tile lies above this wave's rows
     floatx16_t sacc[NKB];
 #pragma unroll
     for (int kb = 0; kb < NKB; kb++)
@@ -987,14 +989,14 @@ __global__ __launch_bounds__(512, 2) void prefill_mfma_pair_kernel(PrefillArgs a
 #pragma unroll
         for (int kb = 0; kb < 2; kb++) sacc[kb0 + kb] = MT::mfma(kf[kb][ks], qreg[rb][ks], sacc[kb0 + kb]);
     }
-    if (k0 + BT > n_keys || k0 + BT - 1 > qlo[rb]) {
+    if (k0 + BT > n_keys || (CAUSAL && k0 + BT - 1 > qlo[rb])) {
       const int qi = qlo[rb] + n;
 #pragma unroll
       for (int kb = 0; kb < NKB; kb++)
 #pragma unroll
         for (int i = 0; i < 16; i++) {
           const int key = k0 + kb * 32 + 8 * (i >> 2) + 4 * g + (i & 3);
-          if (key >= n_keys || key > qi) sacc[kb][i] = -INFINITY;
+          if (key >= n_keys || (CAUSAL && key > qi)) sacc[kb][i] = -INFINITY;
         }
     }
     float mx = sacc[0][0];
@@ -1053,7 +1055,7 @@ __global__ __launch_bounds__(512, 2) void prefill_mfma_pair_kernel(PrefillArgs a
     for (int kb = 0; kb < NKB; kb += NB) {
       const int k0 = kt * BT + kb * 32;
       if (k0 >= k_end_late) break;
-      if (k0 + 32 * NB - 1 <= qlo[0] && k0 + 32 * NB <= k_end_early) {   // the whole group below the early rows' diagonal
+      if (CAUSAL ? (k0 + 32 * NB - 1 <= qlo[0] && k0 + 32 * NB <= k_end_early) : true) {   // the whole group below the early rows' diagonal
         block(kBoth, kNB, Ks + kb * 32 * LDK, Vs + kb * 32 * LDV, k0);
       } else {
 #pragma unroll
@@ -1076,7 +1078,7 @@ __global__ __launch_bounds__(512, 2) void prefill_mfma_pair_kernel(PrefillArgs a
     if (kt + 1 < n_tiles_late) load_tile(kt + 1, (kt + 1) & 1);
     const uint16_t *Ks = Ks2[kt & 1];
     const uint16_t *Vs = Vs2[kt & 1];
-    if (kt * BT + BT - 1 > qlo[1]) {
+    if (CAUSAL && kt * BT + BT - 1 > qlo[1]) {
       // a tile on the late rows' diagonal: block by block, so that blocks above the wave's rows are skipped (four at a
       // time they would be computed and masked: 109.9 -> 108.7 us on B=1 H=32 S=4096 D=96)
 #pragma unroll
@@ -1098,8 +1100,11 @@ int launch_pair(const PrefillArgs &a, hipStream_t stream) {
   const int n_pairs = (n_q_tiles + 1) / 2;
   const int n_bh_groups = (a.B * a.Hq + 7) / 8;
   dim3 grid(8 * n_bh_groups * n_pairs), block(512);
-  if (plan_only("prefill_mfma_pair_kernel<%s, D=%d> query tiles=%d, workgroups=%u", MT::kName, D, n_q_tiles, grid.x)) return LMH_OK;
-  hipLaunchKernelGGL((prefill_mfma_pair_kernel<MT, D>), grid, block, 0, stream, a, n_q_tiles, n_bh_groups);
+  if (plan_only("prefill_mfma_pair_kernel<%s, D=%d, %s> query tiles=%d, workgroups=%u", MT::kName, D, a.causal ? "causal" : "full", n_q_tiles, grid.x)) return LMH_OK;
+  if (a.causal)
+    hipLaunchKernelGGL((prefill_mfma_pair_kernel<MT, D, true>), grid, block, 0, stream, a, n_q_tiles, n_bh_groups);
+  else
+    hipLaunchKernelGGL((prefill_mfma_pair_kernel<MT, D, false>), grid, block, 0, stream, a, n_q_tiles, n_bh_groups);
   LMH_HIP_TRY(hipGetLastError());
   return LMH_OK;
 }
@@ -1178,6 +1183,13 @@ int launch_for_d(const PrefillArgs &a, hipStream_t stream) {
   if constexpr (D <= 96 && !MT::kSplitP) {
     const int64_t wgs_pair = (int64_t)((a.B * a.Hq + 7) / 8) * 8 * (((a.Sq + 255) / 256 + 1) / 2);
     if (a.causal && a.Sq > 256 && wgs_pair <= n_cus && 16 * wgs_pair >= 15 * n_cus) return launch_pair<MT, D>(a, stream);
+    // Without a mask the same kernel takes two neighbouring tiles (512 rows, every fragment read shared all the way);
+    // its workgroups are equal, so it wants whole rounds: B=1 H=32 S=4096 D=96 (one round) -5.9 %, S=8192 (two) -3.5 %,
+    // B=4 (four) -1.1 %; D=64 one round -2.4 %, two rounds +2.5 %; 1.25 rounds +20 %.
+    if (!a.causal && a.Sq > 256 && wgs_pair >= n_cus) {
+      const int64_t rounds = (wgs_pair + n_cus - 1) / n_cus, last = wgs_pair - (rounds - 1) * n_cus;
+      if (16 * last >= 15 * n_cus && (rounds == 1 || (D > 64 && rounds <= 2))) return launch_pair<MT, D>(a, stream);
+    }
   }
   const int64_t wgs = (int64_t)((a.B * a.Hq + 7) / 8) * 8 * ((a.Sq + 127) / 128);
   const int64_t limit = a.causal ? 2 * n_cus : 2 * n_cus - 1;

@@ -172,7 +172,7 @@ def test_kernel_plan_of_the_benchmark_configurations(lm):
     assert plan((1, 8, 128, 64), (1, 8, 128, 64), "f32", True).startswith("prefill_f32_kernel<D=64, causal, key groups=4>")
     # C2: 32 heads x 16 tiles of 256 rows = 256 pairs (tile p with tile 15 - p), one workgroup per CU, one round
     assert plan((1, 32, 4096, 96), (1, 32, 4096, 96), "f16", True) == \
-        "prefill_mfma_pair_kernel<f16, D=96> query tiles=16, workgroups=256"
+        "prefill_mfma_pair_kernel<f16, D=96, causal> query tiles=16, workgroups=256"
     # the same in bf16 (head + remainder weights: no room for two row blocks), or with the chip not exactly full:
     # 512 workgroups of 256 rows, one per CU at a time, 128-key tiles
     assert plan((1, 32, 4096, 96), (1, 32, 4096, 96), "bf16", True).startswith(

@@ -129,44 +129,52 @@ def test_wide_workgroup_random_shapes(lm, hip, oracle):
     print("plans covered:", sorted(seen), flush=True)
 
 
-# (B, Hq, Hkv, Sq, Sk, D, kv_len or None, head_map, what is special)
+# (B, Hq, Hkv, Sq, Sk, D, kv_len or None, head_map, causal, what is special)
 PAIRED_TILE_CASES = [
-    (1, 64, 16, 2048, 2048, 64, None, 0, "GQA 4:1, 8 tiles"),
-    (1, 64, 16, 2048, 2048, 64, None, 1, "the same with the blocked head map"),
-    (2, 64, 64, 1024, 1024, 96, [700, 1024], 0, "ragged keys, 4 tiles"),
-    (2, 64, 64, 1024, 1024, 96, [0, 300], 0, "a sequence without keys, one with fewer keys than a tile"),
-    (1, 32, 8, 3700, 3700, 80, None, 0, "15 tiles (the middle one alone), a partial last tile, head dim padded to 96"),
-    (4, 64, 64, 512, 512, 64, None, 0, "two tiles: one pair per head"),
-    (1, 30, 30, 4000, 4000, 96, None, 0, "30 heads on 32 head slots"),
-    (1, 32, 32, 4096, 5000, 96, None, 0, "more keys than queries"),
-    (1, 32, 32, 4096, 3000, 96, None, 0, "fewer keys than queries"),
-    (1, 32, 32, 4096, 4096, 40, [2500], 0, "head dim 40 on the 64 tiling, keys end inside the late tiles"),
+    (1, 64, 16, 2048, 2048, 64, None, 0, True, "GQA 4:1, 8 tiles"),
+    (1, 64, 16, 2048, 2048, 64, None, 1, True, "the same with the blocked head map"),
+    (2, 64, 64, 1024, 1024, 96, [700, 1024], 0, True, "ragged keys, 4 tiles"),
+    (2, 64, 64, 1024, 1024, 96, [0, 300], 0, True, "a sequence without keys, one with fewer keys than a tile"),
+    (1, 32, 8, 3700, 3700, 80, None, 0, True, "15 tiles (the middle one alone), a partial last tile, head dim padded to 96"),
+    (4, 64, 64, 512, 512, 64, None, 0, True, "two tiles: one pair per head"),
+    (1, 30, 30, 4000, 4000, 96, None, 0, True, "30 heads on 32 head slots"),
+    (1, 32, 32, 4096, 5000, 96, None, 0, True, "more keys than queries"),
+    (1, 32, 32, 4096, 3000, 96, None, 0, True, "fewer keys than queries"),
+    (1, 32, 32, 4096, 4096, 40, [2500], 0, True, "head dim 40 on the 64 tiling, keys end inside the late tiles"),
+    # without a mask: two neighbouring tiles per workgroup, whole rounds only
+    (1, 32, 8, 4000, 1500, 64, None, 0, False, "no mask: GQA, a partial last tile, keys not a multiple of the tile"),
+    (2, 64, 64, 1000, 700, 80, [1, 699], 1, False, "no mask: one key; ragged; head dim padded to 96"),
+    (1, 32, 32, 3600, 2000, 96, None, 0, False, "no mask: 15 tiles, the last workgroup of a head has one tile"),
+    (1, 30, 10, 3900, 4500, 96, [0], 0, False, "no mask: a sequence without keys"),
+    (1, 32, 32, 8192, 1100, 96, None, 0, False, "no mask: two rounds"),
 ]
 
 
-@pytest.mark.parametrize("case", PAIRED_TILE_CASES, ids=lambda c: "B%d-H%d:%d-S%dx%d-D%d" % c[:6])
+@pytest.mark.parametrize("case", PAIRED_TILE_CASES, ids=lambda c: "B%d-H%d:%d-S%dx%d-D%d-%s" % (c[:6] + ("causal" if c[8] else "full",)))
 @pytest.mark.parametrize("out_f32", [False, True])
-def test_paired_tile_causal_kernel(lm, hip, oracle, case, out_f32):
-    """Causal fp16 launches that are one round of paired 256-row query tiles (tile p with tile n - 1 - p in one workgroup,
-    the early tile stored half way) against the oracle; the plan query confirms the kernel."""
-    B, Hq, Hkv, Sq, Sk, D, lens, head_map, what = case
-    plan = lm.flash_attention_plan((B, Hq, Sq, D), (B, Hkv, Sk, D), "f16", True)
+def test_paired_tile_kernel(lm, hip, oracle, case, out_f32):
+    """fp16 launches that are whole rounds of paired 256-row query tiles (causal: tile p with tile n - 1 - p in one
+    workgroup, the early tile stored half way; no mask: two neighbouring tiles) against the oracle; the plan query
+    confirms the kernel."""
+    B, Hq, Hkv, Sq, Sk, D, lens, head_map, causal, what = case
+    plan = lm.flash_attention_plan((B, Hq, Sq, D), (B, Hkv, Sk, D), "f16", causal)
     print(what, "->", plan, flush=True)
-    assert "prefill_mfma_pair_kernel" in plan, plan
+    assert "prefill_mfma_pair_kernel" in plan and ("causal" if causal else "full") in plan, plan
     lens = None if lens is None else np.asarray(lens, np.int32)
     q, k, v = inputs(oracle, (B, Hq, Sq, D), (B, Hkv, Sk, D), "f16", 97000 + Sq + D, 0.7)
     kp, vp = (k, v) if lens is None else poison_tail(k, v, lens)
-    got = run_flash(lm, hip, q, kp, vp, "f16", True, head_map=head_map, kv_len=lens, out_dtype="f32" if out_f32 else None)
+    got = run_flash(lm, hip, q, kp, vp, "f16", causal, head_map=head_map, kv_len=lens, out_dtype="f32" if out_f32 else None)
     rng = np.random.default_rng(97001)
     hq = np.unique(np.concatenate([[0, Hq - 1], rng.integers(0, Hq, size=4)]))
     G = Hq // Hkv
     kv_of = hq if Hq == Hkv else (hq // G if head_map == 1 else hq % Hkv)
     want_len = None if lens is None else np.maximum(lens, 1)
-    want = oracle.flash_attn(q[:, hq], k[:, kv_of], v[:, kv_of], causal=True, kv_len=want_len, nthreads=NT)
+    want = oracle.flash_attn(q[:, hq], k[:, kv_of], v[:, kv_of], causal=causal, kv_len=want_len, nthreads=NT)
     keep = np.arange(B) if lens is None else np.nonzero(lens > 0)[0]
     assert np.isfinite(got).all(), what
-    err = rel_err(got[keep][:, hq], want[keep])
-    assert err <= TOL["f16"], "%s: rel err %.3g" % (what, err)
+    if len(keep):
+        err = rel_err(got[keep][:, hq], want[keep])
+        assert err <= TOL["f16"], "%s: rel err %.3g" % (what, err)
     if lens is not None:
         for b in np.nonzero(lens == 0)[0]:
             assert np.all(got[b] == 0), what
