@@ -738,7 +738,8 @@ def main():
         line["other_configs"] = other_configs(lm, dev, check=args.cpu_seconds > 0, only="other" if args.only == "all" else args.only,
                                               zero_operands=not args.no_zero_operands)
     gate = [("C2", line.get("parity"))] + [("C5", line.get("decode", {}).get("parity"))] + \
-        [(k.split()[0], v.get("parity")) for k, v in line.get("other_configs", {}).items() if isinstance(v, dict) and "parity" in v]
+        [(k.split()[0] if k.split()[1] != "shape" else "C2 shape without the mask", v.get("parity"))
+         for k, v in line.get("other_configs", {}).items() if isinstance(v, dict) and "parity" in v]
     gate = [(n, p) for n, p in gate if p]
     if gate:
         line["parity_gate"] = {"configs": [n for n, _ in gate], "all_pass": all(p["max_rel_err"] <= p["tolerance"] for _, p in gate)}
