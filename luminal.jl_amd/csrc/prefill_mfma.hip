@@ -729,7 +729,6 @@ __global__ __launch_bounds__(1024, 4) void prefill_mfma_wide_kernel(PrefillArgs 
 template <typename MT, int D, bool CAUSAL>
 __global__ __launch_bounds__(512, 2) void prefill_mfma_pair_kernel(PrefillArgs a, int n_q_tiles, int n_bh_groups) {
   using vec8 = typename MT::vec8;
-  static_assert(!MT::kSplitP, "head + remainder weights do not fit the register budget of two row blocks");
   constexpr int NW = 8, BM = 256;
   constexpr int BT = 2 * BN;        // 128 keys per staged tile
   constexpr int NKB = BT / 32;
@@ -883,7 +882,7 @@ __global__ __launch_bounds__(512, 2) void prefill_mfma_pair_kernel(PrefillArgs a
 #pragma unroll
         for (int rb = RB0; rb < 2; rb++) sacc[rb][kb] = MT::mfma(kf, qreg[rb][ks], sacc[rb][kb]);
       }
-    vec8 pf[2][NB][2];
+    vec8 pf[2][NB][2], pf_lo[2][NB][2];
 #pragma unroll
     for (int rb = RB0; rb < 2; rb++) {
       if (k0 + 32 * NB > n_keys || (CAUSAL && k0 + 32 * NB - 1 > qlo[rb])) {  // the ragged last block, or a block on this row block's diagonal
@@ -919,8 +918,13 @@ __global__ __launch_bounds__(512, 2) void prefill_mfma_pair_kernel(PrefillArgs a
 #pragma unroll
         for (int t = 0; t < 2; t++) {
 #pragma unroll
-          for (int e = 0; e < 8; e++) pf[rb][kb][t][e] = MT::cvt(__builtin_amdgcn_exp2f(sacc[rb][kb][8 * t + e] * c - mc));
+          for (int e = 0; e < 8; e++) {
+            const float p = __builtin_amdgcn_exp2f(sacc[rb][kb][8 * t + e] * c - mc);
+            pf[rb][kb][t][e] = MT::cvt(p);
+            if (MT::kSplitP) pf_lo[rb][kb][t][e] = MT::cvt(p - (float)pf[rb][kb][t][e]);
+          }
           l_i[rb] = MT::sum8(pf[rb][kb][t], l_i[rb]);
+          if (MT::kSplitP) l_i[rb] = MT::sum8(pf_lo[rb][kb][t], l_i[rb]);
         }
     }
 #pragma unroll
@@ -934,7 +938,10 @@ __global__ __launch_bounds__(512, 2) void prefill_mfma_pair_kernel(PrefillArgs a
           const shortx4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_shortx4_t *)(vaddr + 8 * LDV));
           const vec8 v8 = __builtin_bit_cast(vec8, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
 #pragma unroll
-          for (int rb = RB0; rb < 2; rb++) oacc[rb][db] = MT::mfma(v8, pf[rb][kb][t], oacc[rb][db]);
+          for (int rb = RB0; rb < 2; rb++) {
+            oacc[rb][db] = MT::mfma(v8, pf[rb][kb][t], oacc[rb][db]);
+            if (MT::kSplitP) oacc[rb][db] = MT::mfma(v8, pf_lo[rb][kb][t], oacc[rb][db]);
+          }
         }
   };
   auto store_rows = [&](int rb) {
@@ -1016,14 +1023,19 @@ __global__ __launch_bounds__(512, 2) void prefill_mfma_pair_kernel(PrefillArgs a
         for (int i = 0; i < 16; i++) oacc[rb][db][i] *= alpha;
     }
     const float mc = m_i[rb] * c;
-    vec8 pf[NKB][2];
+    vec8 pf[NKB][2], pf_lo[NKB][2];
 #pragma unroll
     for (int kb = 0; kb < NKB; kb++)
 #pragma unroll
       for (int t = 0; t < 2; t++) {
 #pragma unroll
-        for (int e = 0; e < 8; e++) pf[kb][t][e] = MT::cvt(__builtin_amdgcn_exp2f(sacc[kb][8 * t + e] * c - mc));
+        for (int e = 0; e < 8; e++) {
+          const float p = __builtin_amdgcn_exp2f(sacc[kb][8 * t + e] * c - mc);
+          pf[kb][t][e] = MT::cvt(p);
+          if (MT::kSplitP) pf_lo[kb][t][e] = MT::cvt(p - (float)pf[kb][t][e]);
+        }
         l_i[rb] = MT::sum8(pf[kb][t], l_i[rb]);
+        if (MT::kSplitP) l_i[rb] = MT::sum8(pf_lo[kb][t], l_i[rb]);
       }
 #pragma unroll
     for (int kb = 0; kb < NKB; kb++)
@@ -1036,6 +1048,7 @@ __global__ __launch_bounds__(512, 2) void prefill_mfma_pair_kernel(PrefillArgs a
           const shortx4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_shortx4_t *)(vaddr + 8 * LDV));
           const vec8 v8 = __builtin_bit_cast(vec8, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
           oacc[rb][db] = MT::mfma(v8, pf[kb][t], oacc[rb][db]);
+          if (MT::kSplitP) oacc[rb][db] = MT::mfma(v8, pf_lo[kb][t], oacc[rb][db]);
         }
   };
   const std::integral_constant<int, 0> kBoth{};
@@ -1048,7 +1061,7 @@ __global__ __launch_bounds__(512, 2) void prefill_mfma_pair_kernel(PrefillArgs a
     if (kt + 1 < n_tiles_late) load_tile(kt + 1, (kt + 1) & 1);
     const uint16_t *Ks = Ks2[kt & 1];
     const uint16_t *Vs = Vs2[kt & 1];
-    constexpr int NB = 2;  // two 32-key blocks of both row blocks at a time: four score blocks in flight, 244 registers
+    constexpr int NB = 2;  // two 32-key blocks of both row blocks at a time: four score blocks in flight (fp16, D = 96: 244 registers)
     const std::integral_constant<int, NB> kNB{};
     const std::integral_constant<int, 1> kOne{};
 #pragma unroll
@@ -1180,13 +1193,15 @@ int launch_for_d(const PrefillArgs &a, hipStream_t stream) {
   // 256 CUs, fp16: B=1 H=32 S=4096 D=96 -3.2 %, D=64 -6 %, D=80 -3 %; B=2 H=32 S=2048 -5 %; H=8 S=16384 -4.6 %;
   // S=3900 -2 %. With the chip not exactly full it loses (1.25 rounds +23 %, 1.5 rounds +10 %, half a round +30 %),
   // at exactly two rounds it ties (-1.4 ... +7 %).
-  if constexpr (D <= 96 && !MT::kSplitP) {
+  // bf16 (weights as head + remainder: twice the weight registers) only at D <= 64 and only causal: B=1 H=32 S=4096
+  // D=64 -8 %, H=64 S=2048 -6 %; D=96 +1 % causal (and spills with two blocks at a time), -2.5 % without a mask.
+  if constexpr (D <= 96 && (!MT::kSplitP || D <= 64)) {
     const int64_t wgs_pair = (int64_t)((a.B * a.Hq + 7) / 8) * 8 * (((a.Sq + 255) / 256 + 1) / 2);
     if (a.causal && a.Sq > 256 && wgs_pair <= n_cus && 16 * wgs_pair >= 15 * n_cus) return launch_pair<MT, D>(a, stream);
     // Without a mask the same kernel takes two neighbouring tiles (512 rows, every fragment read shared all the way);
     // its workgroups are equal, so it wants whole rounds: B=1 H=32 S=4096 D=96 (one round) -5.9 %, S=8192 (two) -3.5 %,
     // B=4 (four) -1.1 %; D=64 one round -2.4 %, two rounds +2.5 %; 1.25 rounds +20 %.
-    if (!a.causal && a.Sq > 256 && wgs_pair >= n_cus) {
+    if (!a.causal && !MT::kSplitP && a.Sq > 256 && wgs_pair >= n_cus) {
       const int64_t rounds = (wgs_pair + n_cus - 1) / n_cus, last = wgs_pair - (rounds - 1) * n_cus;
       if (16 * last >= 15 * n_cus && (rounds == 1 || (D > 64 && rounds <= 2))) return launch_pair<MT, D>(a, stream);
     }

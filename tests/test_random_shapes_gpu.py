@@ -150,6 +150,38 @@ PAIRED_TILE_CASES = [
 ]
 
 
+PAIRED_TILE_CASES_BF16 = [
+    (1, 64, 16, 2048, 2048, 64, None, 0, True, "bf16: GQA 4:1, 8 tiles"),
+    (1, 32, 32, 3800, 3800, 40, [2500], 0, True, "bf16: head dim 40 on the 64 tiling, 15 tiles, keys end inside the late tiles"),
+    (4, 64, 64, 512, 512, 64, [512, 0, 77, 300], 1, True, "bf16: two tiles, ragged"),
+]
+
+
+@pytest.mark.parametrize("case", PAIRED_TILE_CASES_BF16, ids=lambda c: "B%d-H%d:%d-S%dx%d-D%d" % c[:6])
+def test_paired_tile_kernel_bf16(lm, hip, oracle, case):
+    """The same kernel with bf16 weights fed as head + remainder (causal, head dims up to 64 only), fp32 output."""
+    B, Hq, Hkv, Sq, Sk, D, lens, head_map, causal, what = case
+    plan = lm.flash_attention_plan((B, Hq, Sq, D), (B, Hkv, Sk, D), "bf16", causal)
+    print(what, "->", plan, flush=True)
+    assert "prefill_mfma_pair_kernel<bf16" in plan, plan
+    lens = None if lens is None else np.asarray(lens, np.int32)
+    q, k, v = inputs(oracle, (B, Hq, Sq, D), (B, Hkv, Sk, D), "bf16", 97500 + Sq + D, 0.7)
+    kp, vp = (k, v) if lens is None else poison_tail(k, v, lens)
+    got = run_flash(lm, hip, q, kp, vp, "bf16", causal, head_map=head_map, kv_len=lens)
+    hq = np.unique(np.concatenate([[0, Hq - 1], np.random.default_rng(97501).integers(0, Hq, size=4)]))
+    G = Hq // Hkv
+    kv_of = hq if Hq == Hkv else (hq // G if head_map == 1 else hq % Hkv)
+    want_len = None if lens is None else np.maximum(lens, 1)
+    want = oracle.flash_attn(q[:, hq], k[:, kv_of], v[:, kv_of], causal=causal, kv_len=want_len, nthreads=NT)
+    keep = np.arange(B) if lens is None else np.nonzero(lens > 0)[0]
+    assert np.isfinite(got).all(), what
+    err = rel_err(got[keep][:, hq], want[keep])
+    assert err <= TOL["bf16"], "%s: rel err %.3g" % (what, err)
+    if lens is not None:
+        for b in np.nonzero(lens == 0)[0]:
+            assert np.all(got[b] == 0), what
+
+
 @pytest.mark.parametrize("case", PAIRED_TILE_CASES, ids=lambda c: "B%d-H%d:%d-S%dx%d-D%d-%s" % (c[:6] + ("causal" if c[8] else "full",)))
 @pytest.mark.parametrize("out_f32", [False, True])
 def test_paired_tile_kernel(lm, hip, oracle, case, out_f32):
