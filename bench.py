@@ -535,37 +535,44 @@ def ops_leg(lm, dev, res, caches=None):
 
 
 def step_leg(lm, dev, res):
-    """One whole decode step of an attention layer (append with rotary q and K, split-KV attention, merge: 3
-    kernels), driven from the host step by step and as one recorded HIP graph; wall clock per step. On the C4
-    shape the GPU is the bottleneck either way; a single short sequence is bound by the host's launches."""
+    """One whole decode step of an attention layer, wall clock per step: as append (rotating q and K) + split-KV
+    attention + merge (3 kernels) driven from the host and as one recorded HIP graph, and as the fused step
+    (lmh_decode_step: the split kernel rotates q as it loads it, the merge launch adds and stores the new row; 2
+    kernels). The caches hold L - 1 rows and the step writes row L - 1, so every form reads the same bytes. On the C4
+    shape the GPU is the bottleneck either way; a single short sequence is bound by the launches."""
     for B, L in ((16, 4096), (1, 512)):
         Hq, Hkv, D = 32, 8, 128
-        g = lm.Graph()
-        tq, tkn, tvn = lm.tensor(g, (B, Hq, 1, D), "bf16"), lm.tensor(g, (B, Hkv, 1, D), "bf16"), lm.tensor(g, (B, Hkv, 1, D), "bf16")
-        tkc, tvc = lm.tensor(g, (B, Hkv, L, D), "bf16"), lm.tensor(g, (B, Hkv, L, D), "bf16")
-        tpos, tlen = lm.tensor(g, (B,), "i32"), lm.tensor(g, (B,), "i32")
-        lm.cached_self_attention_core(tq, tkn, tvn, tkc, tvc, tpos, tlen, rope_base=10000.0, out_dtype="f32")
-        cg = lm.compile(g, dev)
-        cg({tpos.id: np.full(B, L - 1, np.int32), tlen.id: np.full(B, L, np.int32)})
+        timings = {}
+        for fused in (False, True):
+            g = lm.Graph()
+            tq, tkn, tvn = lm.tensor(g, (B, Hq, 1, D), "bf16"), lm.tensor(g, (B, Hkv, 1, D), "bf16"), lm.tensor(g, (B, Hkv, 1, D), "bf16")
+            tkc, tvc = lm.tensor(g, (B, Hkv, L, D), "bf16"), lm.tensor(g, (B, Hkv, L, D), "bf16")
+            tpos, tlen = lm.tensor(g, (B,), "i32"), lm.tensor(g, (B,), "i32")
+            lm.cached_self_attention_core(tq, tkn, tvn, tkc, tvc, tpos, tlen, rope_base=10000.0, out_dtype="f32", fused=fused)
+            cg = lm.compile(g, dev)
+            assert len(cg.steps) == (1 if fused else 2)
+            cg({tpos.id: np.full(B, L - 1, np.int32), tlen.id: np.full(B, L, np.int32)})
 
-        def wall_us(n=200):
-            for _ in range(20):
-                cg({})
-            lm.binding.sync()
-            t0 = time.perf_counter()
-            for _ in range(n):
-                cg({})
-            lm.binding.sync(cg.cache.get("hip_stream"))
-            lm.binding.sync()
-            return (time.perf_counter() - t0) / n * 1e6
+            def wall_us(n=200):
+                for _ in range(20):
+                    cg({})
+                lm.binding.sync()
+                t0 = time.perf_counter()
+                for _ in range(n):
+                    cg({})
+                lm.binding.sync(cg.cache.get("hip_stream"))
+                lm.binding.sync()
+                return (time.perf_counter() - t0) / n * 1e6
 
-        eager = wall_us()
-        cg.capture()
-        replay = wall_us()
-        cg.release()
+            timings["fused" if fused else "eager"] = wall_us()
+            cg.capture()
+            timings["fused_graph" if fused else "graph"] = wall_us()
+            cg.release()
         res["decode step of a layer bf16 B=%d Hq=32 Hkv=8 L=%d D=128 (append with rotary q and K + attention), wall clock" % (B, L)] = {
-            "us_per_step_3_launches_from_the_host": eager, "us_per_step_one_hip_graph": replay}
-        log("[other] decode step B=%d L=%d, wall clock: %.1f us as 3 host launches, %.1f us as one HIP graph" % (B, L, eager, replay))
+            "us_per_step_3_launches_from_the_host": timings["eager"], "us_per_step_one_hip_graph": timings["graph"],
+            "us_per_step_fused_2_launches_from_the_host": timings["fused"], "us_per_step_fused_one_hip_graph": timings["fused_graph"]}
+        log("[other] decode step B=%d L=%d, wall clock: %.1f us as 3 host launches, %.1f us as one HIP graph; fused step: %.1f us as "
+            "2 host launches, %.1f us as one HIP graph" % (B, L, timings["eager"], timings["graph"], timings["fused"], timings["fused_graph"]))
 
 
 def ceiling_leg(lm, dev):

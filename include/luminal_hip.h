@@ -23,7 +23,7 @@
 extern "C" {
 #endif
 
-#define LMH_VERSION 104 /* major*10000 + minor*100 + patch */
+#define LMH_VERSION 105 /* major*10000 + minor*100 + patch */
 
 /* status codes */
 #define LMH_OK 0
@@ -190,6 +190,32 @@ size_t lmh_decode_workspace_bytes(int32_t B, int32_t Hq, int32_t Hkv, int32_t Lm
 /* the split count lmh_decode_attn uses when num_splits == 0 */
 int32_t lmh_decode_auto_splits(int32_t B, int32_t Hkv, int32_t Lmax);
 int lmh_decode_attn(const lmh_decode_params *p);
+
+/* ---- one decode step of a cached attention layer in two launches: append + attend.
+ * Replaces, for one layer, what decode_step! does with the self-attention caches (reference
+ * src/Whisper.jl:761-801: feed the caches in, run whisper_self_attn_cached :584-620, take the rebuilt caches
+ * out) and the rotary embedding of this step's q and k in front of it (src/NN.jl:356-358).
+ * `p` is the parameter block of lmh_decode_attn with these differences:
+ *   - kv_len is required: kv_len[b] = rows already in the caches = the row this step writes, 0 <= kv_len[b] < Lmax
+ *     (a sequence whose cache is full attends its old rows only and writes nothing);
+ *   - k_cache / v_cache are written: row kv_len[b] of every KV head receives x->k_new (rotated when x->rope)
+ *     and x->v_new; out = attention of q over rows 0 .. kv_len[b] inclusive. q itself is not modified.
+ *   - num_splits == 0 takes lmh_decode_step_splits(); an explicit count must be >= 2; the workspace is
+ *     lmh_decode_workspace_bytes(..., that count).
+ * The first launch is the split kernel of lmh_decode_attn over the old rows, rotating q as it loads it; the second
+ * merges the partials, adds the new row from k_new / v_new and stores it into the caches, so the separate append
+ * launch (lmh_kv_append) disappears. fp16 / bf16 on the matrix-core decode kernel only (head dims 64, 128, 256;
+ * 96 with the interleaved pairing); anything else returns LMH_E_UNSUPPORTED and the caller uses
+ * lmh_kv_append + lmh_decode_attn. The caller advances kv_len afterwards. */
+typedef struct lmh_decode_step_extra {
+  const void *k_new;  /* device [B, Hkv, D], contiguous, element type of the caches: this step's key rows */
+  const void *v_new;  /* device [B, Hkv, D]: this step's value rows */
+  int32_t rope;       /* 1: rotate q and k_new at position kv_len[b] */
+  int32_t pairing;    /* LMH_ROPE_HALF_SPLIT / LMH_ROPE_INTERLEAVED */
+  float rope_base;    /* e.g. 10000 */
+} lmh_decode_step_extra;
+int32_t lmh_decode_step_splits(int32_t B, int32_t Hkv, int32_t Lmax);
+int lmh_decode_step(const lmh_decode_params *p, const lmh_decode_step_extra *x);
 
 /* ---- decode attention that allocates nothing and takes no workspace. No counterpart in the reference: it
  * is lmh_decode_attn for callers that cannot call hipMalloc (code under HIP graph capture, tight serving

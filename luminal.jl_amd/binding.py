@@ -27,7 +27,7 @@ EXPORTS = [
     "lmh_decode_workspace_bytes", "lmh_decode_auto_splits", "lmh_decode_attn", "lmh_flash_attn_plan", "lmh_rope",
     "lmh_kv_append", "lmh_stream_create", "lmh_stream_destroy", "lmh_graph_capture_begin", "lmh_graph_capture_end",
     "lmh_graph_launch", "lmh_graph_destroy", "lmh_static_scratch_bytes", "lmh_decode_static_splits",
-    "lmh_decode_attn_static",
+    "lmh_decode_attn_static", "lmh_decode_step_splits", "lmh_decode_step",
 ]
 
 
@@ -63,6 +63,13 @@ class DecodeParams(ctypes.Structure):
         ("dtype", ctypes.c_int32), ("scale", ctypes.c_float), ("head_map", ctypes.c_int32),
         ("out_f32", ctypes.c_int32), ("num_splits", ctypes.c_int32), ("workspace", ctypes.c_void_p), ("workspace_bytes", ctypes.c_size_t),
         ("stream", ctypes.c_void_p),
+    ]
+
+
+class DecodeStepExtra(ctypes.Structure):
+    _fields_ = [
+        ("k_new", ctypes.c_void_p), ("v_new", ctypes.c_void_p), ("rope", ctypes.c_int32), ("pairing", ctypes.c_int32),
+        ("rope_base", ctypes.c_float),
     ]
 
 
@@ -137,6 +144,9 @@ def load():
     L.lmh_decode_workspace_bytes.argtypes = [ctypes.c_int32] * 6
     L.lmh_decode_auto_splits.restype = ctypes.c_int32
     L.lmh_decode_auto_splits.argtypes = [ctypes.c_int32] * 3
+    L.lmh_decode_step_splits.restype = ctypes.c_int32
+    L.lmh_decode_step_splits.argtypes = [ctypes.c_int32] * 3
+    L.lmh_decode_step.argtypes = [ctypes.POINTER(DecodeParams), ctypes.POINTER(DecodeStepExtra)]
     L.lmh_decode_attn_static.argtypes = [ctypes.POINTER(DecodeParams)]
     L.lmh_decode_attn_static.restype = ctypes.c_int
     L.lmh_static_scratch_bytes.restype = ctypes.c_size_t
@@ -264,6 +274,15 @@ def flash_attn_fwd(params):
 
 def decode_attn(params):
     check(load().lmh_decode_attn(ctypes.byref(params)))
+
+
+def decode_step(params, extra):
+    """lmh_decode_step: append this step's K / V rows and attend, in two launches."""
+    check(load().lmh_decode_step(ctypes.byref(params), ctypes.byref(extra)))
+
+
+def decode_step_splits(B, Hkv, Lmax):
+    return int(load().lmh_decode_step_splits(B, Hkv, Lmax))
 
 
 def decode_attn_static(params):

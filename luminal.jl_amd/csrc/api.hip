@@ -449,8 +449,15 @@ size_t lmh_decode_workspace_bytes(int32_t B, int32_t Hq, int32_t Hkv, int32_t Lm
 
 // Validation and launch shared by lmh_decode_attn (caller-owned workspace) and lmh_decode_attn_static (the
 // library's static scratch): `ws` / `ws_bytes` is the split-KV partial storage, `num_splits` already resolved.
-static int decode_launch(const lmh_decode_params *p, const char *fn, int32_t num_splits, void *ws, size_t ws_bytes) {
+static int decode_launch(const lmh_decode_params *p, const char *fn, int32_t num_splits, void *ws, size_t ws_bytes,
+                         const lmh_decode_step_extra *step = nullptr) {
   DecodeArgs a;
+  a.step = step ? 1 : 0;
+  a.q_rope = (step && step->rope) ? 1 : 0;
+  a.rope_interleaved = (step && step->pairing == LMH_ROPE_INTERLEAVED) ? 1 : 0;
+  a.rope_log2_base = step ? log2f(step->rope_base) : 0.f;
+  a.k_new = step ? step->k_new : nullptr;
+  a.v_new = step ? step->v_new : nullptr;
   a.out = p->out; a.q = p->q; a.k = p->k_cache; a.v = p->v_cache; a.kv_len = p->kv_len;
   a.B = p->B; a.Hq = p->Hq; a.Hkv = p->Hkv; a.Lmax = p->Lmax; a.D = p->D;
   a.scale = p->scale; a.head_map = p->head_map;
@@ -497,6 +504,15 @@ static int decode_launch(const lmh_decode_params *p, const char *fn, int32_t num
     a.ws_o = reinterpret_cast<float *>(ws);
     a.ws_ml = a.ws_o + (size_t)p->B * p->Hq * a.num_splits * p->D;
   }
+  if (step) {
+    // two launches only where the split kernel can rotate q in registers and the slice fits its addressing
+    if (!a.mfma_ok || !decode_mfma_supported(p->dtype, p->D, p->B))
+      return fail(LMH_E_UNSUPPORTED, "%s: needs the matrix-core decode kernel (fp16 / bf16, head dim 64, 96, 128 or 256, aligned q, "
+                  "batch <= 1024); use lmh_kv_append + lmh_decode_attn", fn);
+    if (a.q_rope && !decode_mfma_rope_ok(p->D, a.rope_interleaved))
+      return fail(LMH_E_UNSUPPORTED, "%s: head dim %d with the half-split pairing cannot be rotated in registers; use lmh_kv_append + "
+                  "lmh_decode_attn", fn, p->D);
+  }
   return launch_decode(a, p->dtype, (hipStream_t)p->stream);
 }
 
@@ -524,6 +540,26 @@ int lmh_decode_attn(const lmh_decode_params *p) {
   if (rc != LMH_OK) return rc;
   const int32_t splits = p->num_splits == 0 ? lmh_decode_auto_splits(p->B, p->Hkv, p->Lmax) : p->num_splits;
   return decode_launch(p, "lmh_decode_attn", splits, p->workspace, p->workspace_bytes);
+}
+
+int32_t lmh_decode_step_splits(int32_t B, int32_t Hkv, int32_t Lmax) {
+  const int32_t s = lmh_decode_auto_splits(B, Hkv, Lmax);
+  return s == 0 ? 0 : (s < 2 ? 2 : s);  // the merge launch always runs: it is what adds the new row
+}
+
+int lmh_decode_step(const lmh_decode_params *p, const lmh_decode_step_extra *x) {
+  const char *fn = "lmh_decode_step";
+  const int rc = decode_check(p, fn);
+  if (rc != LMH_OK) return rc;
+  if (!x || !x->k_new || !x->v_new) return fail(LMH_E_NULL, "%s: null k_new / v_new", fn);
+  if (!p->kv_len) return fail(LMH_E_NULL, "%s: kv_len (the rows already in the caches) is required", fn);
+  if (p->dtype == LMH_F32) return fail(LMH_E_UNSUPPORTED, "%s: fp16 / bf16 only; use lmh_kv_append + lmh_decode_attn", fn);
+  if (x->pairing != LMH_ROPE_HALF_SPLIT && x->pairing != LMH_ROPE_INTERLEAVED)
+    return fail(LMH_E_UNSUPPORTED, "%s: unknown rope pairing %d", fn, x->pairing);
+  if (x->rope && !(x->rope_base > 1.f)) return fail(LMH_E_SHAPE, "%s: rope base must be > 1", fn);
+  if (p->num_splits == 1) return fail(LMH_E_SHAPE, "%s: num_splits must be 0 or >= 2", fn);
+  const int32_t splits = p->num_splits == 0 ? lmh_decode_step_splits(p->B, p->Hkv, p->Lmax) : p->num_splits;
+  return decode_launch(p, fn, splits, p->workspace, p->workspace_bytes, x);
 }
 
 // --------------------------------------------------------------------------------------------

@@ -61,6 +61,13 @@ struct DecodeArgs {
   int32_t mfma_ok;  // q is 16-byte aligned with 8-element strides and scale > 0: the MFMA kernel may run
   float *ws_o;    // [B][Hq][num_splits][D] un-normalised partial outputs
   float *ws_ml;   // [B][Hq][num_splits][2] (running max in log2 units, partial sum)
+  // lmh_decode_step: the split kernel attends the kv_len[b] rows already in the cache with q rotated as it is loaded;
+  // the merge kernel adds row kv_len[b] from k_new / v_new (K rotated) and writes it into the caches.
+  int32_t step;             // 0: plain decode attention
+  int32_t q_rope;           // rotate q (and k_new) at position kv_len[b]
+  int32_t rope_interleaved;
+  float rope_log2_base;
+  const void *k_new, *v_new;  // [B][Hkv][D] contiguous
 };
 
 // Rotary embedding launch arguments.
@@ -120,6 +127,7 @@ int launch_decode(const DecodeArgs &a, int dtype, hipStream_t stream);
 int launch_rope(const RopeArgs &a, int dtype, hipStream_t stream);
 int launch_kv_append(const KvAppendArgs &a, int dtype, hipStream_t stream);
 bool decode_mfma_supported(int dtype, int D, int B);
+bool decode_mfma_rope_ok(int D, int interleaved);
 int launch_decode_mfma_split(const DecodeArgs &a, int dtype, hipStream_t stream);
 
 // Keys per split used for a given (Lmax, num_splits); always a multiple of 64.

@@ -18,6 +18,7 @@
 //     a second small kernel merges them with the log-sum-exp identity.
 #include "common.hpp"
 #include "dtypes.hpp"
+#include "rope.hpp"
 
 namespace lmh {
 namespace {
@@ -299,11 +300,15 @@ __global__ __launch_bounds__(kWaves * 64) void decode_split_kernel(DecodeArgs a,
 constexpr int kMergeThreads = 128;
 constexpr int kMergeMaxSlots = 1024;  // weights kept in LDS; more slots than this take the strided path below
 constexpr int kMergePrefetch = 16;     // partial rows fetched before the slot statistics are known
-template <typename E>
+// STEP (lmh_decode_step): the row this step appends, kv_len[b], never went through the split kernel. It joins here as
+// one more partial — score q . k_new (both rotated at position kv_len[b] when a.q_rope, and rounded to the element
+// type as the stored rows are), sum 1, output v_new — and the workgroup of the first query head of every KV head
+// writes the row into the caches (the reference rebuilds them with _kv_scatter, src/Whisper.jl:552-570).
+template <typename E, bool STEP>
 __global__ __launch_bounds__(kMergeThreads) void decode_merge_kernel(DecodeArgs a) {
   using raw = typename E::raw;
   __shared__ float w_s[kMergeMaxSlots];
-  __shared__ float red_m[kMergeThreads / 64], red_l[kMergeThreads / 64];
+  __shared__ float red_m[kMergeThreads / 64], red_l[kMergeThreads / 64], red_s[kMergeThreads / 64];
   const int hq = blockIdx.x, b = blockIdx.y;
   const int tid = threadIdx.x;
   const int64_t off = b * a.os[0] + hq * a.os[1];
@@ -324,9 +329,46 @@ __global__ __launch_bounds__(kMergeThreads) void decode_merge_kernel(DecodeArgs 
   L = min(max(L, 0), a.Lmax);
   const int n = (L + a.chunk - 1) / a.chunk;
 
+  // (this thread's first slot statistics are requested before the new row's arithmetic, not after its barrier)
+  const float2 ml_first = tid < n ? ml[tid] : make_float2(-INFINITY, 0.f);
+  // the new row: its score in log2 units, and (first query head of the KV head only) its place in the caches
+  float m_new = -INFINITY;
+  const raw *v_new_row = nullptr;
+  if (STEP && L < a.Lmax) {
+    const int kvh = kv_head_of(hq, a.Hq, a.Hkv, a.head_map);
+    const bool writer = q_head_of(kvh, 0, a.Hq, a.Hkv, a.head_map) == hq;
+    const raw *q_row = reinterpret_cast<const raw *>(a.q) + b * a.qs[0] + hq * a.qs[1];
+    const raw *k_new_row = reinterpret_cast<const raw *>(a.k_new) + ((int64_t)b * a.Hkv + kvh) * a.D;
+    v_new_row = reinterpret_cast<const raw *>(a.v_new) + ((int64_t)b * a.Hkv + kvh) * a.D;
+    raw *k_dst = const_cast<raw *>(reinterpret_cast<const raw *>(a.k)) + b * a.ks[0] + kvh * a.ks[1] + (int64_t)L * a.ks[2];
+    raw *v_dst = const_cast<raw *>(reinterpret_cast<const raw *>(a.v)) + b * a.vs[0] + kvh * a.vs[1] + (int64_t)L * a.vs[2];
+    auto ld = [](raw x) { return E::ld(x); };
+    float dot = 0.f;
+    for (int d = tid; d < a.D; d += kMergeThreads) {
+      raw qr = q_row[d], kr = k_new_row[d];
+      if (a.q_rope) {
+        qr = E::st(rope_element(q_row, d, a.D, (float)L, a.rope_log2_base, a.rope_interleaved != 0, ld));
+        kr = E::st(rope_element(k_new_row, d, a.D, (float)L, a.rope_log2_base, a.rope_interleaved != 0, ld));
+      }
+      dot += E::ld(qr) * E::ld(kr);
+      if (writer) {
+        k_dst[d] = kr;
+        v_dst[d] = v_new_row[d];
+      }
+    }
+#pragma unroll
+    for (int o = 32; o >= 1; o >>= 1) dot += __shfl_xor(dot, o);
+    if ((tid & 63) == 0) red_s[tid >> 6] = dot;
+    __syncthreads();
+    dot = 0.f;
+#pragma unroll
+    for (int w = 0; w < kMergeThreads / 64; w++) dot += red_s[w];
+    m_new = dot * a.scale * kLog2e;
+  }
+
   // running max over the slots
-  float M = -INFINITY;
-  for (int s = tid; s < n; s += kMergeThreads) M = fmaxf(M, ml[s].x);
+  float M = fmaxf(m_new, ml_first.x);
+  for (int s = tid + kMergeThreads; s < n; s += kMergeThreads) M = fmaxf(M, ml[s].x);
 #pragma unroll
   for (int o = 32; o >= 1; o >>= 1) M = fmaxf(M, __shfl_xor(M, o));
   if ((tid & 63) == 0) red_m[tid >> 6] = M;
@@ -339,7 +381,7 @@ __global__ __launch_bounds__(kMergeThreads) void decode_merge_kernel(DecodeArgs 
   // run and its output row is unset) and the normaliser
   float lsum = 0.f;
   for (int s = tid; s < n; s += kMergeThreads) {
-    const float2 v = ml[s];
+    const float2 v = s == tid ? ml_first : ml[s];
     const float w = v.x == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(v.x - M);
     if (s < kMergeMaxSlots) w_s[s] = w;
     lsum += v.y * w;
@@ -351,6 +393,8 @@ __global__ __launch_bounds__(kMergeThreads) void decode_merge_kernel(DecodeArgs 
   lsum = 0.f;
 #pragma unroll
   for (int w = 0; w < kMergeThreads / 64; w++) lsum += red_l[w];
+  const float w_new = (STEP && v_new_row) ? __builtin_amdgcn_exp2f(m_new - M) : 0.f;  // the new row's sum is 1
+  lsum += w_new;
   const float inv = lsum > 0.f ? 1.f / lsum : 0.f;
 
   for (int d = tid; d < a.D; d += kMergeThreads) {
@@ -382,7 +426,8 @@ __global__ __launch_bounds__(kMergeThreads) void decode_merge_kernel(DecodeArgs 
       const float x = po[(int64_t)s * a.D + d];
       acc[0] += w != 0.f ? x * w : 0.f;
     }
-    const float o = (acc[0] + acc[1]) + (acc[2] + acc[3]);
+    float o = (acc[0] + acc[1]) + (acc[2] + acc[3]);
+    if (STEP && v_new_row) o += w_new * E::ld(v_new_row[d]);
     if (a.out_f32) reinterpret_cast<float *>(a.out)[off + d] = o * inv;
     else reinterpret_cast<raw *>(a.out)[off + d] = E::st(o * inv);
   }
@@ -390,8 +435,11 @@ __global__ __launch_bounds__(kMergeThreads) void decode_merge_kernel(DecodeArgs 
 
 template <typename E>
 int launch_merge(const DecodeArgs &a, hipStream_t stream) {
-  if (a.num_splits > 1) {
-    hipLaunchKernelGGL((decode_merge_kernel<E>), dim3(a.Hq, a.B), dim3(kMergeThreads), 0, stream, a);
+  if (a.step) {  // (always with partials: lmh_decode_step asks for two splits or more)
+    hipLaunchKernelGGL((decode_merge_kernel<E, true>), dim3(a.Hq, a.B), dim3(kMergeThreads), 0, stream, a);
+    LMH_HIP_TRY(hipGetLastError());
+  } else if (a.num_splits > 1) {
+    hipLaunchKernelGGL((decode_merge_kernel<E, false>), dim3(a.Hq, a.B), dim3(kMergeThreads), 0, stream, a);
     LMH_HIP_TRY(hipGetLastError());
   }
   return LMH_OK;
@@ -444,6 +492,7 @@ int launch_decode(const DecodeArgs &a, int dtype, hipStream_t stream) {
     if (rc != LMH_OK) return rc;
     return dtype == LMH_F16 ? launch_merge<F16>(a, stream) : launch_merge<BF16>(a, stream);
   }
+  if (a.step) return fail(LMH_E_UNSUPPORTED, "decode step: only the matrix-core decode kernel rotates q as it loads it");
   switch (dtype) {
     case LMH_F32: return launch_for_dtype<F32>(a, stream);
     case LMH_F16: return launch_for_dtype<F16>(a, stream);

@@ -31,6 +31,7 @@
 // Split-KV partial layout and the merge kernel are shared with decode.hip.
 #include "common.hpp"
 #include "dtypes.hpp"
+#include "rope.hpp"
 
 namespace lmh {
 namespace {
@@ -213,8 +214,42 @@ __global__ __launch_bounds__(kWaves * 64) void decode_mfma_kernel(DecodeArgs a, 
     }
   };
 
+  auto rotate_q = [&]() {
+    // lmh_decode_step: this step's query is rotated at the position of the row the step appends, kv_len[b], as it is
+    // loaded (apply_rotary_embeddings on the queries, reference src/NN.jl:356). Lane (n, g) holds elements
+    // 32 ks + 8 g + e: the partner j + D/2 sits in fragment ks + KS/2 of the same lane when KS is even (the launcher
+    // sends other head dims elsewhere), interleaved partners are neighbours inside a fragment.
+    if (a.q_rope) {
+      const float pos = (float)L;
+      if (!a.rope_interleaved) {
+        if constexpr (KS % 2 == 0) {
+          constexpr int HK = KS / 2;
+#pragma unroll
+          for (int ks = 0; ks < HK; ks++)
+#pragma unroll
+            for (int e = 0; e < 8; e++) {
+              float o0, o1;
+              rope_pair((float)qreg[ks][e], (float)qreg[ks + HK][e], pos, 32 * ks + 8 * g + e, D, a.rope_log2_base, &o0, &o1);
+              qreg[ks][e] = MT::cvt(o0);
+              qreg[ks + HK][e] = MT::cvt(o1);
+            }
+        }
+      } else {
+#pragma unroll
+        for (int ks = 0; ks < KS; ks++)
+#pragma unroll
+          for (int e = 0; e < 8; e += 2) {
+            float o0, o1;
+            rope_pair((float)qreg[ks][e], (float)qreg[ks][e + 1], pos, (32 * ks + 8 * g + e) / 2, D, a.rope_log2_base, &o0, &o1);
+            qreg[ks][e] = MT::cvt(o0);
+            qreg[ks][e + 1] = MT::cvt(o1);
+          }
+      }
+    }
+  };
   const int n_blocks = (end - start + kBlk - 1) / kBlk;
   if (wave < n_blocks) load_tile(start + wave * kBlk);
+  rotate_q();  // (after the first loads are on their way: the rotation is a few hundred instructions per segment)
 
   for (int blk = wave; blk < n_blocks; blk += kWaves) {
     const int key0 = start + blk * kBlk;
@@ -388,6 +423,9 @@ int launch_for_type(const DecodeArgs &a, hipStream_t stream) {
 }
 
 }  // namespace
+
+// The query rotation of lmh_decode_step happens in registers: the partner of every element must be in the same lane.
+bool decode_mfma_rope_ok(int D, int interleaved) { return interleaved || (D / 32) % 2 == 0; }
 
 bool decode_mfma_supported(int dtype, int D, int B) {
   return (dtype == LMH_F16 || dtype == LMH_BF16) && (D == 64 || D == 96 || D == 128 || D == 256) &&

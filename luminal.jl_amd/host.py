@@ -254,6 +254,29 @@ class DecodeAttentionOp(Op):
         self.out_dtype = out_dtype
 
 
+class DecodeStepOp(Op):
+    """One decode step of a cached attention layer as ONE node and two launches (lmh_decode_step): inputs
+    (q (B,Hq,D), k_cache, v_cache, k_new (B,Hkv,1,D), v_new, pos int32[B]); output 0 is the attention result over rows
+    0 .. pos[b] inclusive, outputs 1 and 2 are the caches themselves with row pos[b] written (K rotated when rope_base
+    is set; q is rotated inside the kernel and left as it was). What decode_step! and whisper_self_attn_cached do for
+    one layer (reference src/Whisper.jl:761-801, :584-620) with the rotary embedding of src/NN.jl:356-358."""
+
+    def __init__(self, scale, head_map=HEADMAP_INTERLEAVED, num_splits=0, out_dtype=None, rope_base=None, interleaved=False):
+        self.scale = float(np.float32(scale))
+        self.head_map = head_map
+        self.num_splits = num_splits
+        self.out_dtype = out_dtype
+        self.rope_base = None if rope_base is None else float(rope_base)
+        self.interleaved = bool(interleaved)
+
+
+def decode_step_supported(dtype, head_dim, rope=True, interleaved=False):
+    """Whether lmh_decode_step takes this element type and head dim (otherwise: append + attend, three launches)."""
+    if dtype not in ("f16", "bf16") or head_dim not in (64, 96, 128, 256):
+        return False
+    return (not rope) or interleaved or (head_dim // 32) % 2 == 0
+
+
 class RotaryEmbeddingOp(Op):
     """apply_rotary_embeddings(input, prev_seq; base) (reference src/NN.jl:253-303) as one node; inputs (x,) or
     (x, pos0) with pos0 an int32[B] tensor of per-sequence start positions."""
@@ -487,6 +510,18 @@ def decode_attention(q, k_cache, v_cache, kv_len, scale=None, head_map=HEADMAP_I
                   out_dtype or q.graph_ref.dtypes[q.id])
 
 
+def decode_step(q, k_cache, v_cache, k_new, v_new, pos, scale=None, head_map=HEADMAP_INTERLEAVED, num_splits=0,
+                out_dtype=None, rope_base=None, interleaved=False):
+    """Graph form of lmh_decode_step: q (B,Hq,D); returns (out, k_cache, v_cache)."""
+    g = q.graph_ref
+    if scale is None:
+        scale = np.float32(1.0) / np.sqrt(np.float32(q.shape[-1]))
+    inputs = [(t.id, t.index, t.shape) for t in (q, k_cache, v_cache, k_new, v_new, pos)]
+    out = add_op(g, DecodeStepOp(np.float32(scale), head_map, num_splits, out_dtype, rope_base, interleaved), inputs, q.shape,
+                 out_dtype or g.dtypes[q.id])
+    return out, GraphTensor(out.id, k_cache.shape, g, index=1), GraphTensor(out.id, v_cache.shape, g, index=2)
+
+
 def rotary_embedding(x, prev_seq=0, base=10000.0, pos0=None, interleaved=False):
     """Graph form of apply_rotary_embeddings (reference src/NN.jl:253-303): x (B,H,S,D); row s of sequence b is
     rotated by position prev_seq + s, or pos0[b] + s when the int32[B] tensor pos0 is given."""
@@ -556,13 +591,19 @@ def prompt_self_attention_core(q, k_new, v_new, k_cache, v_cache, pos, kv_len, r
 
 
 def cached_self_attention_core(q, k_new, v_new, k_cache, v_cache, pos, kv_len, rope_base=None, scale=None,
-                               head_map=HEADMAP_INTERLEAVED, num_splits=0, out_dtype=None):
+                               head_map=HEADMAP_INTERLEAVED, num_splits=0, out_dtype=None, fused=False):
     """One decode step of a cached attention layer (reference src/Whisper.jl:584-620) as two fused nodes:
     q (B,Hq,1,D), k_new / v_new (B,Hkv,1,D) are this step's projections, pos int32[B] the row each sequence
     writes, kv_len = pos + 1 the rows it then attends over. Positions are tensors, so one compiled graph serves
     every step (the reference compiles one graph per position, src/Decoding.jl:98-106). Returns (out (B,Hq,D),
     k_cache, v_cache)."""
     g = q.graph_ref
+    if fused and len(q.shape) == 4 and q.shape[2] == 1 and decode_step_supported(g.dtypes[q.id], q.shape[-1], rope_base is not None):
+        # one node, two launches: the split kernel rotates q as it loads it, the merge launch adds and stores the new row
+        # (`kv_len` is not needed: the step attends rows 0 .. pos[b])
+        q3 = GraphTensor(q.id, (q.shape[0], q.shape[1], q.shape[3]), g, q.index)
+        return decode_step(q3, k_cache, v_cache, k_new, v_new, pos, scale=scale, head_map=head_map, num_splits=num_splits,
+                           out_dtype=out_dtype, rope_base=rope_base)
     if rope_base is not None:  # one launch: rotate q in place, write the new rows with K rotated on the way in
         k_cache, v_cache, q = kv_cache_append(k_cache, v_cache, k_new, v_new, pos, rope_k=True, base=rope_base, q=q)
     else:
@@ -625,6 +666,49 @@ def _host_fallback(op, inputs):
     result (the caller uploads it)."""
     host = [x.to_host() if isinstance(x, HipArray) else np.asarray(x, dtype=np.float32) for x in inputs]
     return np.ascontiguousarray(op.compute(*host), dtype=np.float32)
+
+
+def _prepare_decode_step(op, out, inputs, workspaces=None):
+    """Validates a DecodeStepOp call and fills its parameter blocks once; returns launch(stream). A compiled graph keeps
+    the launcher (its buffers never move), so a step costs one ctypes call on the host."""
+    if len(inputs) != 6:
+        raise ValueError("DecodeStepOp takes (q, k_cache, v_cache, k_new, v_new, pos)")
+    q, kc, vc, k_new, v_new, pos = inputs
+    res = out[0] if isinstance(out, tuple) else out
+    if isinstance(out, tuple) and not (out[1] is kc and out[2] is vc):
+        raise ValueError("DecodeStepOp updates the caches in place: outputs 1 and 2 are its cache inputs")
+    _require_hip(res, q, kc, vc, k_new, v_new, pos)
+    if len(q.shape) != 3 or len(kc.shape) != 4 or kc.shape != vc.shape or res.shape != q.shape:
+        raise ValueError("decode step expects q and out (B,H,D) and caches (B,Hkv,Lmax,D); got %s %s %s %s" %
+                         (q.shape, res.shape, kc.shape, vc.shape))
+    B, Hkv, Lmax, D = kc.shape
+    if k_new.shape != v_new.shape or k_new.shape not in ((B, Hkv, 1, D), (B, Hkv, D)) or pos.shape != (B,) or pos.dtype != "i32":
+        raise ValueError("decode step: new rows %s / %s for caches %s, pos %s" % (k_new.shape, v_new.shape, kc.shape, pos.shape))
+    if not (q.dtype == kc.dtype == vc.dtype == k_new.dtype == v_new.dtype) or res.dtype not in (q.dtype, "f32"):
+        raise ValueError("q, the caches and the new rows must share one element type; out has that type or f32")
+    p = binding.DecodeParams()
+    p.out, p.q, p.k_cache, p.v_cache, p.kv_len = res.ptr, q.ptr, kc.ptr, vc.ptr, pos.ptr
+    p.B, p.Hq, p.D = q.shape
+    p.Hkv, p.Lmax = Hkv, Lmax
+    p.dtype = binding.DTYPE_CODES[q.dtype]
+    p.scale, p.head_map = op.scale, op.head_map
+    p.out_f32 = int(res.dtype == "f32")
+    p.num_splits = op.num_splits or binding.decode_step_splits(p.B, p.Hkv, p.Lmax)
+    need = binding.decode_workspace_bytes(p.B, p.Hq, p.Hkv, p.Lmax, p.D, p.num_splits)
+    x = binding.DecodeStepExtra()
+    x.k_new, x.v_new = k_new.ptr, v_new.ptr
+    x.rope = int(op.rope_base is not None)
+    x.pairing = binding.ROPE_INTERLEAVED if op.interleaved else binding.ROPE_HALF_SPLIT
+    x.rope_base = op.rope_base if op.rope_base is not None else 10000.0
+    pool, result = (workspaces or _workspaces), (res, kc, vc)
+
+    def launch(stream=None):
+        p.workspace, p.workspace_bytes = pool.get(need, q.device)
+        p.stream = stream
+        binding.decode_step(p, x)
+        return result
+
+    return launch
 
 
 def execute_op_inplace(out, op, *inputs, stream=None, workspaces=None):
@@ -702,6 +786,8 @@ def execute_op_inplace(out, op, *inputs, stream=None, workspaces=None):
         p.stream = stream
         binding.decode_attn(p)
         return out
+    if isinstance(op, DecodeStepOp):
+        return _prepare_decode_step(op, out, inputs, workspaces)(stream)
     if isinstance(op, RotaryEmbeddingOp):
         x = inputs[0]
         pos0 = inputs[1] if len(inputs) > 1 else None
@@ -733,6 +819,9 @@ def execute_op(op, *inputs):
     _require_hip(q)
     if isinstance(op, KVAppendOp):
         return execute_op_inplace(None, op, *inputs)
+    if isinstance(op, DecodeStepOp):
+        res = HipArray(q.shape, op.out_dtype or q.dtype, q.device)
+        return execute_op_inplace((res, inputs[1], inputs[2]), op, *inputs)
     out = HipArray(q.shape, getattr(op, "out_dtype", None) or q.dtype, q.device)
     return execute_op_inplace(out, op, *inputs)
 
@@ -878,6 +967,10 @@ def compile(graph, device=None):
             refs = [node.inputs[0], node.inputs[1]] + ([node.inputs[5]] if node.op.rope_q else [])
             results.append(tuple(_pick(results, r) for r in refs))
             continue
+        if isinstance(node.op, DecodeStepOp):  # output 0 is a buffer of its own, outputs 1 and 2 are the cache inputs
+            results.append((HipArray(graph.shapes[node_id], graph.dtypes[node_id], device).fill_bytes(0),
+                            _pick(results, node.inputs[1]), _pick(results, node.inputs[2])))
+            continue
         results.append(HipArray(graph.shapes[node_id], graph.dtypes[node_id], device).fill_bytes(0))
     steps = []
     workspaces = _Workspaces()
@@ -885,6 +978,9 @@ def compile(graph, device=None):
         if isinstance(node.op, InputTensor):
             continue
         args = [_pick(results, ref) for ref in node.inputs]
+        if isinstance(node.op, DecodeStepOp):
+            steps.append(_prepare_decode_step(node.op, results[node_id], args, workspaces))
+            continue
         steps.append(lambda stream, out=results[node_id], op=node.op, args=args:
                      execute_op_inplace(out, op, *args, stream=stream, workspaces=workspaces))
     host_steps = sum(isinstance(node.op, HostOp) for node in graph.nodes)
@@ -988,7 +1084,7 @@ def default_scale(D):
 __all__ = [
     "AbstractDevice", "CPUDevice", "HIPDevice", "HipArray", "get_device", "to_device", "from_device", "Graph",
     "GraphTensor", "tensor", "add_op", "FlashAttentionOp", "DecodeAttentionOp", "flash_attention", "decode_attention",
-    "RotaryEmbeddingOp", "KVAppendOp", "rotary_embedding", "kv_cache_append", "self_attention_core",
+    "RotaryEmbeddingOp", "KVAppendOp", "DecodeStepOp", "decode_step", "decode_step_supported", "rotary_embedding", "kv_cache_append", "self_attention_core",
     "cached_self_attention_core", "prompt_self_attention_core", "FUSED_ROPE_HEAD_DIMS", "HostOp", "MatMulOp", "PermuteOp", "ReshapeOp", "AddOp", "ExpandOp", "matmul", "permute",
     "reshape", "add", "expand", "Linear", "SelfAttention", "execute_op", "execute_op_inplace", "execute", "compile", "CompiledGraph", "execute_with_capture", "release_capture", "HEADMAP_INTERLEAVED",
     "HEADMAP_BLOCKED", "LuminalHipError", "apply_rotary_embeddings", "kv_append", "KVCacheState", "encode", "decode", "f32_to_bf16_bits", "bf16_bits_to_f32", "default_scale",

@@ -321,6 +321,64 @@ execute_op(op::DecodeAttentionOp, q::HipArray, kc::HipArray, vc::HipArray, kv_le
     execute_op!(similar(q), op, q, kc, vc, kv_len)
 
 # ------------------------------------------------------------------------------------------
+# DecodeStepOp: one decode step of a cached attention layer as one node and two launches (lmh_decode_step): what
+# decode_step! and whisper_self_attn_cached do for one layer (src/Whisper.jl:761-801, :584-620) with the rotary embedding
+# of src/NN.jl:356-358. Inputs (q, k_cache, v_cache, k_new, v_new, pos); the value of the node is the attention result
+# over rows 0 .. pos[b] inclusive; the caches are updated in place (row pos[b]; K rotated when rope_base is set); q is
+# rotated inside the kernel and left as it was.
+# ------------------------------------------------------------------------------------------
+struct DecodeStepExtra
+    k_new::Ptr{Cvoid}; v_new::Ptr{Cvoid}; rope::Int32; pairing::Int32; rope_base::Float32
+end
+
+struct DecodeStepOp <: Op
+    scale::Float32
+    head_map::Int32
+    rope_base::Float32      # 0: no rotary embedding
+end
+
+"Whether lmh_decode_step takes this element type and head dim (otherwise: kv_append! + decode attention, three launches)."
+decode_step_supported(::Type{T}, head_dim::Integer; rope::Bool=true) where {T} =
+    (T === Float16 || T === BF16Bits) && head_dim in (64, 96, 128, 256) && (!rope || iseven(head_dim ÷ 32))
+
+function decode_step(q::GraphTensor, k_cache::GraphTensor, v_cache::GraphTensor, k_new::GraphTensor, v_new::GraphTensor,
+                     pos::GraphTensor; scale=nothing, head_map::Int32=HEADMAP_INTERLEAVED, rope_base=nothing)
+    q_dims = realized_dims(q.shape)
+    s = isnothing(scale) ? 1.0f0 / sqrt(Float32(q_dims[end])) : Float32(scale)
+    inputs = [(t.id, 0, t.shape) for t in (q, k_cache, v_cache, k_new, v_new, pos)]
+    return add_op!(q.graph_ref, DecodeStepOp(s, head_map, Float32(something(rope_base, 0.0f0))), inputs, q.shape)
+end
+
+function execute_op!(out::HipArray{TO,3}, op::DecodeStepOp, q::HipArray{T,3}, kc::HipArray{T,4}, vc::HipArray{T,4},
+                     k_new::HipArray{T,4}, v_new::HipArray{T,4}, pos::HipArray{Int32,1}) where {TO,T}
+    B, Hq, D = size(q)
+    _, Hkv, Lmax, _ = size(kc)
+    out_f32 = Int32(TO === Float32 && T !== Float32)
+    splits = ccall((:lmh_decode_step_splits, libluminal_hip), Int32, (Int32, Int32, Int32), B, Hkv, Lmax)
+    need = ccall((:lmh_decode_workspace_bytes, libluminal_hip), Csize_t, (Int32, Int32, Int32, Int32, Int32, Int32),
+                 B, Hq, Hkv, Lmax, D, splits)
+    ws = workspace(need)
+    p = Ref(DecodeParams(out.ptr, q.ptr, kc.ptr, vc.ptr, Ptr{Int32}(pos.ptr), B, Hq, Hkv, Lmax, D, Z2, Z2, Z3, Z3,
+                         dtype_code(T), op.scale, op.head_map, out_f32, splits,
+                         ws === nothing ? C_NULL : ws.ptr, need, current_stream()))
+    x = Ref(DecodeStepExtra(k_new.ptr, v_new.ptr, Int32(op.rope_base > 0), Int32(0), op.rope_base > 0 ? op.rope_base : 10000.0f0))
+    check(ccall((:lmh_decode_step, libluminal_hip), Cint, (Ref{DecodeParams}, Ref{DecodeStepExtra}), p, x))
+    return out
+end
+
+# q and out as (B,H,1,D): the same memory as (B,H,D)
+function execute_op!(out::HipArray{TO,4}, op::DecodeStepOp, q::HipArray{T,4}, kc::HipArray{T,4}, vc::HipArray{T,4},
+                     k_new::HipArray{T,4}, v_new::HipArray{T,4}, pos::HipArray{Int32,1}) where {TO,T}
+    size(q, 3) == 1 || error("DecodeStepOp takes one query token per sequence; got q of size $(size(q))")
+    dims3 = (size(q, 1), size(q, 2), size(q, 4))
+    execute_op!(Base.reshape(out, dims3), op, Base.reshape(q, dims3), kc, vc, k_new, v_new, pos)
+    return out
+end
+
+execute_op(op::DecodeStepOp, q::HipArray, kc::HipArray, vc::HipArray, k_new::HipArray, v_new::HipArray, pos::HipArray) =
+    execute_op!(similar(q), op, q, kc, vc, k_new, v_new, pos)
+
+# ------------------------------------------------------------------------------------------
 # the operators in front of decode attention
 # ------------------------------------------------------------------------------------------
 struct RopeParams
@@ -479,8 +537,14 @@ the rows it then attends over. Both are device arrays, so nothing is recompiled 
 function cached_self_attention_core!(out::HipArray{TO,3}, q::HipArray{T,4}, k_new::HipArray{T,4}, v_new::HipArray{T,4},
                                      kc::HipArray{T,4}, vc::HipArray{T,4}, pos::HipArray{Int32,1},
                                      kv_len::HipArray{Int32,1}; rope_base=nothing, scale=nothing,
-                                     head_map::Int32=HEADMAP_INTERLEAVED) where {TO,T}
+                                     head_map::Int32=HEADMAP_INTERLEAVED, fused::Bool=false) where {TO,T}
     size(q, 3) == 1 || error("cached attention takes one query token per sequence")
+    if fused && decode_step_supported(T, size(q, 4); rope=(rope_base !== nothing))
+        # two launches instead of three: the split kernel rotates q as it loads it, the merge launch adds and stores the new row
+        s = isnothing(scale) ? 1.0f0 / sqrt(Float32(size(q, 4))) : Float32(scale)
+        q3 = HipArray{T,3}(q.ptr, (size(q, 1), size(q, 2), size(q, 4)), q)
+        return execute_op!(out, DecodeStepOp(s, head_map, Float32(something(rope_base, 0.0f0))), q3, kc, vc, k_new, v_new, pos)
+    end
     # one launch: the new rows go into the caches (K rotated on the way in) and q is rotated in place
     kv_append!(kc, vc, k_new, v_new, pos; rope_k=(rope_base !== nothing), base=something(rope_base, 10000.0f0),
                q=(rope_base !== nothing ? q : nothing))
@@ -537,10 +601,11 @@ One layer of a decode step (whisper_self_attn_cached, src/Whisper.jl:584-620): t
 rotated at their positions (src/NN.jl:356-358). Returns out (B,Hq,D).
 """
 function decode_layer!(out::HipArray{TO,3}, c::HipKVCache{T}, layer::Integer, q::HipArray{T,4}, k_new::HipArray{T,4},
-                       v_new::HipArray{T,4}; rope_base=nothing, scale=nothing, head_map::Int32=HEADMAP_INTERLEAVED) where {TO,T}
+                       v_new::HipArray{T,4}; rope_base=nothing, scale=nothing, head_map::Int32=HEADMAP_INTERLEAVED,
+                       fused::Bool=true) where {TO,T}
     kc, vc = c.self_cache[layer]
     return cached_self_attention_core!(out, q, k_new, v_new, kc, vc, c.pos, c.kv_len; rope_base=rope_base, scale=scale,
-                                       head_map=head_map)
+                                       head_map=head_map, fused=fused)
 end
 
 "The prompt pass of layer `layer` (T tokens per sequence into empty caches), between begin_step!(cache, T) and advance!(cache, T)."
@@ -621,7 +686,7 @@ end
 cache_capturing() = _stream[] != C_NULL
 
 const FIXED_FALLBACK_ARITIES = 1:3
-const DeviceOp = Union{FlashAttentionOp,RopeFlashAttentionOp,DecodeAttentionOp,RotaryEmbeddingOp,KVAppendOp}
+const DeviceOp = Union{FlashAttentionOp,RopeFlashAttentionOp,DecodeAttentionOp,DecodeStepOp,RotaryEmbeddingOp,KVAppendOp}
 is_device_op_type(T) = T <: DeviceOp
 for T in subtypes(Op)
     (is_device_op_type(T) || parentmodule(T) === @__MODULE__) && continue
@@ -794,6 +859,6 @@ export HIPDevice, HipArray, BF16Bits, release_capture!, enable_capture!, compile
        RotaryEmbeddingOp, rotary_embedding, KVAppendOp, kv_cache_append, get_device, functional, rope!, kv_append!,
        self_attention_core!, cached_self_attention_core!, self_attention_core, cached_self_attention_core, flash_attention_plan,
        RopeFlashAttentionOp, rope_flash_attention, prompt_self_attention_core!, self_attention, host_fallback,
-       HipKVCache, step_pos, begin_step!, advance!, decode_layer!, prompt_layer!
+       HipKVCache, step_pos, begin_step!, advance!, decode_layer!, prompt_layer!, DecodeStepOp, decode_step, decode_step_supported
 
 end # module

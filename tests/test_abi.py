@@ -24,7 +24,7 @@ def test_library_exports_every_declared_symbol(lm):
     lib = lm.binding.load()
     for name in header_functions():
         assert hasattr(lib, name), name
-    assert lib.lmh_version() == 104
+    assert lib.lmh_version() == 105
     calib = lm.binding.load_calib()
     for name in header_functions("luminal_hip_calib.h"):
         assert hasattr(calib, name), name
@@ -63,6 +63,7 @@ def test_experiment_flags_need_the_measurement_marker(lm, monkeypatch):
 def test_struct_layout_matches_header(lm):
     # field order/size must match the C struct: compare against sizes computed by hand from the header
     assert ctypes.sizeof(lm.binding.AttnParams) == 5 * 8 + 6 * 4 + 4 * 24 + 5 * 4 + 4 + 8 + 2 * 4 + 8 + 2 * 4
+    assert ctypes.sizeof(lm.binding.DecodeStepExtra) == 2 * 8 + 3 * 4 + 4  # (4 bytes of tail padding)
     assert ctypes.sizeof(lm.binding.DecodeParams) == 5 * 8 + 5 * 4 + 4 + 2 * 16 + 2 * 24 + 5 * 4 + 4 + 8 + 8 + 8
 
 

@@ -11,6 +11,7 @@ STRUCTS = {  # header name -> (ctypes class, Julia struct)
     "lmh_decode_params": ("DecodeParams", "DecodeParams"),
     "lmh_rope_params": ("RopeParams", "RopeParams"),
     "lmh_kv_append_params": ("KvAppendParams", "KvAppendParams"),
+    "lmh_decode_step_extra": ("DecodeStepExtra", "DecodeStepExtra"),
 }
 
 
@@ -172,18 +173,19 @@ def test_glue_graph_nodes_have_builders_and_executors():
     # a builder that calls add_op!, an in-place executor and an allocating one; compile_hip knows all four ops
     text = glue_text()
     for op, builder in (("DecodeAttentionOp", "decode_attention"), ("RotaryEmbeddingOp", "rotary_embedding"),
-                        ("KVAppendOp", "kv_cache_append"), ("RopeFlashAttentionOp", "rope_flash_attention")):
+                        ("KVAppendOp", "kv_cache_append"), ("RopeFlashAttentionOp", "rope_flash_attention"),
+                        ("DecodeStepOp", "decode_step")):
         assert re.search(r"^struct %s <: Op$" % op, text, flags=re.M), op
         body = re.search(r"^function %s\(.*?^end$" % builder, text, flags=re.M | re.S)
         assert body and "add_op!(" in body.group(0) and op + "(" in body.group(0), builder
         assert re.search(r"^function execute_op!\(out::HipArray\{\w+,\d\}, op::%s," % op, text, flags=re.M), op
         assert re.search(r"^execute_op\(op::%s, " % op, text, flags=re.M), op
-    assert re.search(r"^const DeviceOp = Union\{FlashAttentionOp,RopeFlashAttentionOp,DecodeAttentionOp,RotaryEmbeddingOp,KVAppendOp\}$",
+    assert re.search(r"^const DeviceOp = Union\{FlashAttentionOp,RopeFlashAttentionOp,DecodeAttentionOp,DecodeStepOp,RotaryEmbeddingOp,KVAppendOp\}$",
                      text, flags=re.M)
     exported = re.search(r"^export (.*?)\n\n", text, flags=re.M | re.S).group(1)
     for name in ("compile_hip", "HipArray", "HIPDevice", "rotary_embedding", "kv_cache_append", "decode_attention",
                  "cached_self_attention_core", "self_attention_core", "enable_capture!", "rope_flash_attention",
-                 "prompt_self_attention_core!"):
+                 "prompt_self_attention_core!", "decode_step", "DecodeStepOp", "decode_step_supported"):
         assert name in re.split(r"[,\s]+", exported), name
 
 
@@ -291,7 +293,8 @@ def test_glue_ccalls_pass_as_many_arguments_as_the_header_declares():
         seen += 1
         names.add(name)
     assert seen >= 20
-    assert {"lmh_flash_attn_fwd", "lmh_flash_attn_plan", "lmh_decode_attn", "lmh_decode_attn_static", "lmh_rope", "lmh_kv_append"} <= names
+    assert {"lmh_flash_attn_fwd", "lmh_flash_attn_plan", "lmh_decode_attn", "lmh_decode_attn_static", "lmh_decode_step", "lmh_rope",
+            "lmh_kv_append"} <= names
 
 
 def _julia_spellings(c_decl):
@@ -301,7 +304,7 @@ def _julia_spellings(c_decl):
     assert m, c_decl
     base, stars = m.group(1), m.group(2).count("*")
     struct = {"lmh_attn_params": "AttnParams", "lmh_decode_params": "DecodeParams", "lmh_rope_params": "RopeParams",
-              "lmh_kv_append_params": "KvAppendParams"}
+              "lmh_kv_append_params": "KvAppendParams", "lmh_decode_step_extra": "DecodeStepExtra"}
     if base in struct:
         assert stars == 1
         return {"Ref{%s}" % struct[base]}
