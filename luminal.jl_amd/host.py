@@ -480,6 +480,38 @@ class SelfAttention:
         return self.o_proj(out)
 
 
+class WhisperAttention:
+    """WhisperSelfAttention and WhisperCrossAttention (reference src/Whisper.jl:238-272, :278-316) with the layer's own
+    nodes kept — projections (q, v and the output with a bias, k without: :247-251, :288-292), the column-major split of
+    hidden into heads, the permutes — and the matmul / mask / softmax / matmul between them replaced by one flash
+    attention node. The reference scales q and k by D^-0.25 each (:256, :305-307); here the product is scaled by
+    D^-0.5 inside the kernel. Self attention: layer(x, mask=True); cross attention: layer(x, mask=False, keys_from=enc,
+    values_from=enc) (queries from the decoder, keys and values from the encoder output)."""
+
+    def __init__(self, hidden, n_heads, graph, attn_dtype="f32"):
+        if hidden % n_heads:
+            raise ValueError("hidden must be a multiple of n_heads")
+        self.n_heads, self.head_dim, self.attn_dtype = n_heads, hidden // n_heads, attn_dtype
+        self.q_proj = Linear(hidden, hidden, graph, bias=True)
+        self.k_proj = Linear(hidden, hidden, graph, bias=False)
+        self.v_proj = Linear(hidden, hidden, graph, bias=True)
+        self.o_proj = Linear(hidden, hidden, graph, bias=True)
+
+    def __call__(self, x, mask=False, keys_from=None, values_from=None):
+        batch, seq, hidden = x.shape
+        k_in = x if keys_from is None else keys_from
+        v_in = x if values_from is None else values_from
+
+        def heads(proj, t):  # (B, S, H*D) -> (B, H, S, D), uploaded in the element type attention reads
+            return permute(reshape(proj(t), (t.shape[0], t.shape[1], self.n_heads, self.head_dim)), (0, 2, 1, 3),
+                           dtype=self.attn_dtype)
+
+        out = flash_attention(heads(self.q_proj, x), heads(self.k_proj, k_in), heads(self.v_proj, v_in), causal=bool(mask),
+                              out_dtype="f32")
+        out = reshape(permute(out, (0, 2, 1, 3)), (batch, seq, hidden))
+        return self.o_proj(out)
+
+
 def flash_attention(q, k, v, scale=None, causal=False, head_map=HEADMAP_INTERLEAVED, out_dtype=None, kv_len=None,
                     q_rope_base=None, q_prev_seq=0, q_pos0=None, q_rope_interleaved=False):
     """q, k, v: (Batch, Head, Seq, HeadDim). Output has q's shape; scale defaults to 1/sqrt(D)
@@ -1086,7 +1118,7 @@ __all__ = [
     "GraphTensor", "tensor", "add_op", "FlashAttentionOp", "DecodeAttentionOp", "flash_attention", "decode_attention",
     "RotaryEmbeddingOp", "KVAppendOp", "DecodeStepOp", "decode_step", "decode_step_supported", "rotary_embedding", "kv_cache_append", "self_attention_core",
     "cached_self_attention_core", "prompt_self_attention_core", "FUSED_ROPE_HEAD_DIMS", "HostOp", "MatMulOp", "PermuteOp", "ReshapeOp", "AddOp", "ExpandOp", "matmul", "permute",
-    "reshape", "add", "expand", "Linear", "SelfAttention", "execute_op", "execute_op_inplace", "execute", "compile", "CompiledGraph", "execute_with_capture", "release_capture", "HEADMAP_INTERLEAVED",
+    "reshape", "add", "expand", "Linear", "SelfAttention", "WhisperAttention", "execute_op", "execute_op_inplace", "execute", "compile", "CompiledGraph", "execute_with_capture", "release_capture", "HEADMAP_INTERLEAVED",
     "HEADMAP_BLOCKED", "LuminalHipError", "apply_rotary_embeddings", "kv_append", "KVCacheState", "encode", "decode", "f32_to_bf16_bits", "bf16_bits_to_f32", "default_scale",
     "flash_attention_plan",
 ]

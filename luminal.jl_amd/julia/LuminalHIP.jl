@@ -709,6 +709,28 @@ heads (a column-major Reshape: the head index is the fast one), the permutes —
 embedding of Q and K, repeat_kv, scaled causal softmax attention, src/NN.jl:356-382) replaced by
 self_attention_core: the fused op reads the Hkv key/value heads directly and rotates the queries inside the kernel.
 """
+"""
+WhisperSelfAttention / WhisperCrossAttention (src/Whisper.jl:253-272, :295-316) around one flash attention node: the
+layer's own projections (any struct with q_proj, k_proj, v_proj, o_proj, as both reference layers are), its
+column-major split into `n_heads` heads and its permutes are kept; matmul, mask, softmax and matmul between them
+become `flash_attention`. The reference scales q and k by D^-0.25 each (:256, :305-307): the kernel scales the product
+by D^-0.5. Self attention: `whisper_attention(sa, x; n_heads, mask=true)`; cross attention:
+`whisper_attention(ca, queries_t; n_heads, keys_from=enc, values_from=enc)`.
+"""
+function whisper_attention(layer, x::GraphTensor; n_heads::Int, mask::Bool=false, keys_from::GraphTensor=x,
+                           values_from::GraphTensor=x)
+    batch, seq, hidden = realized_dims(x.shape)
+    head_dim = hidden ÷ n_heads
+    function heads(proj, t)
+        b, s, _ = realized_dims(t.shape)
+        return Luminal.permute(Luminal.reshape(proj(t), [b, s, n_heads, head_dim]), [1, 3, 2, 4])
+    end
+    out = Luminal.flash_attention(heads(layer.q_proj, x), heads(layer.k_proj, keys_from), heads(layer.v_proj, values_from);
+                                  causal=mask)
+    out = Luminal.reshape(Luminal.permute(out, [1, 3, 2, 4]), [batch, seq, hidden])
+    return layer.o_proj(out)
+end
+
 function self_attention(sa::Luminal.NN.SelfAttention, x::GraphTensor, prev_seq::Int; rope_base=10000.0f0)
     batch, seq, hidden = realized_dims(x.shape)
     heads(proj, n) = Luminal.permute(Luminal.reshape(proj(x), [batch, seq, n, sa.head_dim]), [1, 3, 2, 4])
@@ -859,6 +881,7 @@ export HIPDevice, HipArray, BF16Bits, release_capture!, enable_capture!, compile
        RotaryEmbeddingOp, rotary_embedding, KVAppendOp, kv_cache_append, get_device, functional, rope!, kv_append!,
        self_attention_core!, cached_self_attention_core!, self_attention_core, cached_self_attention_core, flash_attention_plan,
        RopeFlashAttentionOp, rope_flash_attention, prompt_self_attention_core!, self_attention, host_fallback,
-       HipKVCache, step_pos, begin_step!, advance!, decode_layer!, prompt_layer!, DecodeStepOp, decode_step, decode_step_supported
+       HipKVCache, step_pos, begin_step!, advance!, decode_layer!, prompt_layer!, DecodeStepOp, decode_step, decode_step_supported,
+       whisper_attention
 
 end # module

@@ -39,3 +39,29 @@ def reference_layer_f64(x, wq, wk, wv, wo, n_heads, n_kv_heads, prev_seq, base=1
     p = w / w.sum(-1, keepdims=True)
     out = np.reshape(np.transpose(p @ v, (0, 2, 1, 3)), (B, S, hidden), order="F")
     return out @ wo.T
+
+
+def reference_whisper_attention_f64(x, wq, bq, wk, wv, bv, wo, bo, n_heads, mask, enc=None):
+    """WhisperSelfAttention (reference src/Whisper.jl:253-272) or, with `enc` (the encoder output the keys and values are
+    projected from), WhisperCrossAttention (:295-316), node by node in float64: q and k scaled by D^-0.25 each, additive
+    -1e9 strict upper mask for self attention with mask, column-major reshapes."""
+    x, wq, bq, wk, wv, bv, wo, bo = (np.asarray(a, np.float64) for a in (x, wq, bq, wk, wv, bv, wo, bo))
+    src = x if enc is None else np.asarray(enc, np.float64)
+    B, S, hidden = x.shape
+    Sk = src.shape[1]
+    D = hidden // n_heads
+    scale = float(D) ** -0.25
+
+    def heads(t, s_len):
+        return np.transpose(np.reshape(t, (B, s_len, n_heads, D), order="F"), (0, 2, 1, 3))
+
+    q = heads((x @ wq.T + bq) * scale, S)
+    k = heads((src @ wk.T) * scale, Sk)
+    v = heads(src @ wv.T + bv, Sk)
+    w = q @ np.transpose(k, (0, 1, 3, 2))
+    if mask:
+        w = w + np.triu(np.ones((S, Sk)), 1) * -1e9
+    w = np.exp(w - w.max(-1, keepdims=True))
+    p = w / w.sum(-1, keepdims=True)
+    out = np.reshape(np.transpose(p @ v, (0, 2, 1, 3)), (B, S, hidden), order="F")
+    return out @ wo.T + bo

@@ -341,6 +341,14 @@ def test_glue_host_fallback_and_layer_builder():
                   "[1, 3, 2, 4]", "self_attention_core(queries, keys, values; causal=true, prev_seq=prev_seq, rope_base=rope_base)",
                   "[batch, seq, hidden]"):
         assert piece in layer, piece
+    wh = re.search(r"^function whisper_attention\(layer, x::GraphTensor;.*?^end$", text, flags=re.M | re.S).group(0)
+    for piece in ("layer.q_proj, x", "layer.k_proj, keys_from", "layer.v_proj, values_from", "layer.o_proj(out)",
+                  "[b, s, n_heads, head_dim]", "[1, 3, 2, 4]", "Luminal.flash_attention(", "causal=mask", "[batch, seq, hidden]"):
+        assert piece in wh, piece
+    if os.path.isdir(REFERENCE):
+        w = open(os.path.join(REFERENCE, "src/Whisper.jl")).read()
+        assert "Luminal.permute(Luminal.reshape(sa.q_proj(x) * scale, [batch, seq, HEADS, HEAD_DIM]), [1, 3, 2, 4])" in w
+        assert "scale = (Float32(hidden) / Float32(HEADS)) ^ -0.25f0" in w
     if os.path.isdir(REFERENCE):  # the layer's own lines in the reference say the same
         nn = open(os.path.join(REFERENCE, "src/NN.jl")).read()
         assert "Luminal.reshape(sa.q_proj(x), [batch, seq, sa.n_heads, sa.head_dim])" in nn

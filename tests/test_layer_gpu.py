@@ -68,3 +68,33 @@ def test_attention_between_float64_projections_equals_the_oracle(lm, hip, oracle
     att = oracle.flash_attn(oracle.rope(q), oracle.rope(k), v, causal=True, head_map=0)
     want = np.reshape(np.transpose(att.astype(np.float64), (0, 2, 1, 3)), (B, S, hidden), order="F") @ ws[3].astype(np.float64).T
     assert rel_err(got, want) <= 3e-5
+
+
+@pytest.mark.parametrize("attn_dtype,cross", [("f32", False), ("f16", False), ("f16", True), ("bf16", True)])
+def test_whisper_attention_layers_run_with_attention_on_the_gpu(lm, hip, oracle, attn_dtype, cross):
+    """WhisperSelfAttention (masked) and WhisperCrossAttention (reference src/Whisper.jl:238-316) built by the mirror —
+    biased projections on the host, one flash attention node on the GPU — against a float64 replay of the reference
+    layers; Whisper-tiny's width (6 heads of 64)."""
+    from layer_reference import reference_whisper_attention_f64
+    B, S, Senc, hidden, n_heads = 2, 70, 150, 384, 6
+    x = oracle.gen_normal((B, S, hidden), 15200)
+    enc = oracle.gen_normal((B, Senc, hidden), 15201) if cross else None
+    ws = [oracle.gen_normal((hidden, hidden), 15210 + i, 1.0 / np.sqrt(hidden)) for i in range(4)]
+    bs = [oracle.gen_normal((hidden,), 15220 + i, 0.1) for i in range(3)]
+    g = lm.Graph()
+    tx = lm.tensor(g, x.shape)
+    tenc = lm.tensor(g, enc.shape) if cross else None
+    layer = lm.WhisperAttention(hidden, n_heads, g, attn_dtype=attn_dtype)
+    out = layer(tx, mask=not cross, keys_from=tenc, values_from=tenc)
+    assert sum(isinstance(n.op, lm.FlashAttentionOp) for n in g.nodes) == 1
+    feed = {tx.id: x, layer.q_proj.weight.id: ws[0], layer.q_proj.bias.id: bs[0], layer.k_proj.weight.id: ws[1],
+            layer.v_proj.weight.id: ws[2], layer.v_proj.bias.id: bs[1], layer.o_proj.weight.id: ws[3], layer.o_proj.bias.id: bs[2]}
+    if cross:
+        feed[tenc.id] = enc
+    got = lm.execute(g, out.id, feed, hip)
+    want = reference_whisper_attention_f64(x, ws[0], bs[0], ws[1], ws[2], bs[1], ws[3], bs[2], n_heads, mask=not cross, enc=enc)
+    tol = {"f32": 2e-5, "f16": 3e-3, "bf16": 1.5e-2}[attn_dtype]  # half precision: q, k, v are rounded before attention
+    assert rel_err(got, want) <= tol
+    cg = lm.compile(g, hip)
+    res = cg(feed)
+    assert rel_err(res[out.id].to_host(), want) <= tol
