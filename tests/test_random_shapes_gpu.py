@@ -210,3 +210,58 @@ def test_paired_tile_kernel(lm, hip, oracle, case, out_f32):
     if lens is not None:
         for b in np.nonzero(lens == 0)[0]:
             assert np.all(got[b] == 0), what
+
+
+def test_paired_tile_random_shapes(lm, hip, oracle):
+    """Shapes drawn so that the launch is exactly one round of paired tiles (heads x pairs = 256 on a 256-CU device):
+    tile counts from 2 to 32 (odd ones included), partial last tiles, head dims, GQA groups, head maps, ragged keys,
+    with and without the mask, fp16 and (causal, head dims up to 64) bf16."""
+    rng = np.random.default_rng(98000)
+    done, tried, reached = 0, 0, set()
+    while done < 16 and tried < 2000:
+        tried += 1
+        pairs = int(rng.choice([1, 2, 4, 8, 16, 32]))
+        heads = 256 // pairs
+        n_tiles = 2 * pairs - int(rng.integers(2))
+        if n_tiles < 2:
+            continue
+        Sq = int(rng.integers((n_tiles - 1) * 256 + 1, n_tiles * 256 + 1))
+        causal = bool(rng.integers(2))
+        dtype = "bf16" if (causal and rng.integers(3) == 0) else "f16"
+        D = int(rng.choice([16, 32, 40, 64] if dtype == "bf16" else [16, 32, 40, 64, 72, 88, 96]))
+        G = int(rng.choice([1, 1, 2, 4]))
+        B = int(rng.choice([b for b in (1, 2, 4) if heads % b == 0 and (heads // b) % G == 0]))
+        Hq = heads // B - int(rng.integers(0, 2)) * G  # (sometimes fewer heads than head slots)
+        if Hq < G or (B * Hq + 7) // 8 * 8 != heads:
+            continue
+        Hkv = Hq // G
+        Sk = int(rng.integers(max(1, Sq // 3), Sq + 600))
+        if B * Hq * Sq * Sk * D > 3e11:
+            continue
+        plan = lm.flash_attention_plan((B, Hq, Sq, D), (B, Hkv, Sk, D), dtype, causal)
+        if "prefill_mfma_pair_kernel" not in plan:
+            continue
+        head_map = int(rng.integers(2))
+        lens = None if rng.integers(2) == 0 else rng.integers(0, Sk + 1, size=B).astype(np.int32)
+        what = "case %d: %s B=%d Hq=%d Hkv=%d Sq=%d Sk=%d D=%d causal=%s head_map=%d kv_len=%s -> %s" % (
+            done, dtype, B, Hq, Hkv, Sq, Sk, D, causal, head_map, None if lens is None else lens.tolist(), plan)
+        print(what, flush=True)
+        q, k, v = inputs(oracle, (B, Hq, Sq, D), (B, Hkv, Sk, D), dtype, 98100 + 3 * done, float(rng.choice([0.5, 1.0, 1.5])))
+        kp, vp = (k, v) if lens is None else poison_tail(k, v, lens)
+        got = run_flash(lm, hip, q, kp, vp, dtype, causal, head_map=head_map, kv_len=lens)
+        hq = np.unique(rng.integers(0, Hq, size=min(Hq, 3)))
+        kv_of = hq if Hq == Hkv else (hq // G if head_map == 1 else hq % Hkv)
+        want_len = None if lens is None else np.maximum(lens, 1)
+        want = oracle.flash_attn(q[:, hq], k[:, kv_of], v[:, kv_of], causal=causal, kv_len=want_len, nthreads=NT)
+        keep = np.arange(B) if lens is None else np.nonzero(lens > 0)[0]
+        assert np.isfinite(got).all(), what
+        if len(keep):
+            err = rel_err(got[keep][:, hq], want[keep])
+            assert err <= TOL[dtype], "%s: rel err %.3g" % (what, err)
+        if lens is not None:
+            for b in np.nonzero(lens == 0)[0]:
+                assert np.all(got[b] == 0), what
+        reached.add((dtype, causal))
+        done += 1
+    assert done == 16, "only %d shapes reached the paired-tile kernel" % done
+    assert {("f16", True), ("f16", False)} <= reached
