@@ -29,8 +29,9 @@
 #include "prefill_mfma.hpp"
 #include "rope.hpp"
 
-#if (defined(LMH_FOLD_SCALE) || defined(LMH_ONLY_XCDS) || defined(LMH_WIDE_MARGIN) || defined(LMH_W64_KERNEL)) && !defined(LMH_MEASUREMENT_BUILD)
-#error "LMH_FOLD_SCALE / LMH_ONLY_XCDS / LMH_WIDE_MARGIN / LMH_W64_KERNEL are experiment switches: they need -DLMH_MEASUREMENT_BUILD, which marks the library"
+#if (defined(LMH_FOLD_SCALE) || defined(LMH_ONLY_XCDS) || defined(LMH_WIDE_MARGIN) || defined(LMH_W64_KERNEL) || defined(LMH_NO_PAIR_KERNEL)) && \
+    !defined(LMH_MEASUREMENT_BUILD)
+#error "LMH_FOLD_SCALE / LMH_ONLY_XCDS / LMH_WIDE_MARGIN / LMH_W64_KERNEL / LMH_NO_PAIR_KERNEL are experiment switches: they need -DLMH_MEASUREMENT_BUILD, which marks the library"
 #endif
 
 #ifndef LMH_WIDE_MARGIN
@@ -1195,6 +1196,7 @@ int launch_for_d(const PrefillArgs &a, hipStream_t stream) {
   // at exactly two rounds it ties (-1.4 ... +7 %).
   // bf16 (weights as head + remainder: twice the weight registers) only at D <= 64 and only causal: B=1 H=32 S=4096
   // D=64 -8 %, H=64 S=2048 -6 %; D=96 +1 % causal (and spills with two blocks at a time), -2.5 % without a mask.
+#ifndef LMH_NO_PAIR_KERNEL  // (measurement builds can keep these launches on the kernels below, for comparisons with them)
   if constexpr (D <= 96 && (!MT::kSplitP || D <= 64)) {
     const int64_t wgs_pair = (int64_t)((a.B * a.Hq + 7) / 8) * 8 * (((a.Sq + 255) / 256 + 1) / 2);
     if (a.causal && a.Sq > 256 && wgs_pair <= n_cus && 16 * wgs_pair >= 15 * n_cus) return launch_pair<MT, D>(a, stream);
@@ -1206,6 +1208,7 @@ int launch_for_d(const PrefillArgs &a, hipStream_t stream) {
       if (16 * last >= 15 * n_cus && (rounds == 1 || (D > 64 && rounds <= 2))) return launch_pair<MT, D>(a, stream);
     }
   }
+#endif
   const int64_t wgs = (int64_t)((a.B * a.Hq + 7) / 8) * 8 * ((a.Sq + 127) / 128);
   const int64_t limit = a.causal ? 2 * n_cus : 2 * n_cus - 1;
   if (wgs <= limit && a.Sk >= 4 * BN) {
