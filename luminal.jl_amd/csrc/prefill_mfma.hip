@@ -436,27 +436,7 @@ __global__ __launch_bounds__(64 * NW, WPS) void prefill_mfma_kernel(PrefillArgs 
   const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
   if (qi < a.Sq) {
     const int64_t off = b * a.os[0] + hq * a.os[1] + (int64_t)qi * a.os[2];
-    uint16_t *op = reinterpret_cast<uint16_t *>(a.out) + off;
-    float *op32 = reinterpret_cast<float *>(a.out) + off;
-#pragma unroll
-    for (int db = 0; db < DB; db++)
-#pragma unroll
-      for (int i4 = 0; i4 < 4; i4++) {
-        const int d = db * 32 + 8 * i4 + 4 * g;
-        if (d >= a.D) continue;
-        if (a.out_f32) {
-          *reinterpret_cast<float4 *>(op32 + d) =
-              make_float4(oacc[db][4 * i4 + 0] * inv, oacc[db][4 * i4 + 1] * inv, oacc[db][4 * i4 + 2] * inv,
-                          oacc[db][4 * i4 + 3] * inv);
-          continue;
-        }
-        uint2 packed;
-        packed.x = (uint32_t)MT::cvt_bits(oacc[db][4 * i4 + 0] * inv) |
-                   ((uint32_t)MT::cvt_bits(oacc[db][4 * i4 + 1] * inv) << 16);
-        packed.y = (uint32_t)MT::cvt_bits(oacc[db][4 * i4 + 2] * inv) |
-                   ((uint32_t)MT::cvt_bits(oacc[db][4 * i4 + 3] * inv) << 16);
-        *reinterpret_cast<uint2 *>(op + d) = packed;
-      }
+    store_out_rows<MT, DB, false>(oacc, inv, a.out, off, g, a.D, a.out_f32);
   }
 }
 
@@ -693,27 +673,7 @@ __global__ __launch_bounds__(1024, 4) void prefill_mfma_wide_kernel(PrefillArgs 
   const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
   if (qi < a.Sq) {
     const int64_t off = b * a.os[0] + hq * a.os[1] + (int64_t)qi * a.os[2];
-    uint16_t *op = reinterpret_cast<uint16_t *>(a.out) + off;
-    float *op32 = reinterpret_cast<float *>(a.out) + off;
-#pragma unroll
-    for (int db = 0; db < DB; db++)
-#pragma unroll
-      for (int i4 = 0; i4 < 4; i4++) {
-        const int d = db * 32 + 8 * i4 + 4 * g;
-        if (d >= a.D) continue;
-        if (a.out_f32) {
-          *reinterpret_cast<float4 *>(op32 + d) =
-              make_float4(oacc[db][4 * i4 + 0] * inv, oacc[db][4 * i4 + 1] * inv, oacc[db][4 * i4 + 2] * inv,
-                          oacc[db][4 * i4 + 3] * inv);
-          continue;
-        }
-        uint2 packed;
-        packed.x = (uint32_t)MT::cvt_bits(oacc[db][4 * i4 + 0] * inv) |
-                   ((uint32_t)MT::cvt_bits(oacc[db][4 * i4 + 1] * inv) << 16);
-        packed.y = (uint32_t)MT::cvt_bits(oacc[db][4 * i4 + 2] * inv) |
-                   ((uint32_t)MT::cvt_bits(oacc[db][4 * i4 + 3] * inv) << 16);
-        *reinterpret_cast<uint2 *>(op + d) = packed;
-      }
+    store_out_rows<MT, DB, true>(oacc, inv, a.out, off, g, a.D, a.out_f32);
   }
 }
 
@@ -949,30 +909,8 @@ __global__ __launch_bounds__(512, 2) void prefill_mfma_pair_kernel(PrefillArgs a
     const int qi = qlo[rb] + n;
     const float l_tot = sum_over_wave_halves(l_i[rb]);
     const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
-    if (qi < a.Sq) {
-      const int64_t off = b * a.os[0] + hq * a.os[1] + (int64_t)qi * a.os[2];
-      uint16_t *op = reinterpret_cast<uint16_t *>(a.out) + off;
-      float *op32 = reinterpret_cast<float *>(a.out) + off;
-#pragma unroll
-      for (int db = 0; db < DB; db++)
-#pragma unroll
-        for (int i4 = 0; i4 < 4; i4++) {
-          const int d = db * 32 + 8 * i4 + 4 * g;
-          if (d >= a.D) continue;
-          if (a.out_f32) {
-            *reinterpret_cast<float4 *>(op32 + d) =
-                make_float4(oacc[rb][db][4 * i4 + 0] * inv, oacc[rb][db][4 * i4 + 1] * inv, oacc[rb][db][4 * i4 + 2] * inv,
-                            oacc[rb][db][4 * i4 + 3] * inv);
-            continue;
-          }
-          uint2 packed;
-          packed.x = (uint32_t)MT::cvt_bits(oacc[rb][db][4 * i4 + 0] * inv) |
-                     ((uint32_t)MT::cvt_bits(oacc[rb][db][4 * i4 + 1] * inv) << 16);
-          packed.y = (uint32_t)MT::cvt_bits(oacc[rb][db][4 * i4 + 2] * inv) |
-                     ((uint32_t)MT::cvt_bits(oacc[rb][db][4 * i4 + 3] * inv) << 16);
-          *reinterpret_cast<uint2 *>(op + d) = packed;
-        }
-    }
+    if (qi < a.Sq)
+      store_out_rows<MT, DB, false>(oacc[rb], inv, a.out, b * a.os[0] + hq * a.os[1] + (int64_t)qi * a.os[2], g, a.D, a.out_f32);
   };
   // A whole 128-key tile for the late row block alone: the loop body of prefill_mfma_kernel (four 32-key blocks at a
   // time, their QK^T chains alternating two by two, one softmax pass over all 64 scores of a lane).

@@ -73,5 +73,65 @@ struct MfmaBF16 {
 };
 
 
+// Epilogue of the matrix-core flash attention kernels: out[qi][d] = O^T[d][qi] * inv for the wave's 32 query rows.
+// In the accumulator layout lane (n, g) holds, per 32-row block db of O^T, four groups of four consecutive head dims:
+// d = 32 db + 8 i4 + 4 g + (0..3). Written as they lie (WIDE16 = false), a 16-bit output takes one 8-byte store per
+// group, each a separate partial-line request. With WIDE16 one v_permlane32_swap per packed register hands the lower
+// half-wave both halves of the even groups and the upper half-wave both halves of the odd ones: 16 contiguous bytes
+// per lane and store, half the store instructions and requests. That pays where the epilogue is a visible share of
+// the launch (B=4 H=20 Sq=448 Sk=1500 D=64 fp16 through prefill_mfma_wide_kernel: 25.24 -> 24.75 us, and 7.3 -> 6.7 us
+// with no keys at all); in the long causal launches of prefill_mfma_kernel and prefill_mfma_pair_kernel it measured
+// no gain (B=1 H=32 S=4096 D=96: fp16 109.9 -> 110.3 us, bf16 153.2 -> 155.9 us), so those keep the plain form.
+template <typename MT, int DB, bool WIDE16>
+__device__ inline void store_out_rows(const floatx16_t (&oacc)[DB], float inv, void *out, int64_t row_off, int g, int d_valid,
+                                      bool out_f32) {
+  if (out_f32) {
+    float *op32 = reinterpret_cast<float *>(out) + row_off;
+#pragma unroll
+    for (int db = 0; db < DB; db++)
+#pragma unroll
+      for (int i4 = 0; i4 < 4; i4++) {
+        const int d = db * 32 + 8 * i4 + 4 * g;
+        if (d >= d_valid) continue;
+        *reinterpret_cast<float4 *>(op32 + d) = make_float4(oacc[db][4 * i4 + 0] * inv, oacc[db][4 * i4 + 1] * inv,
+                                                            oacc[db][4 * i4 + 2] * inv, oacc[db][4 * i4 + 3] * inv);
+      }
+    return;
+  }
+  uint16_t *op = reinterpret_cast<uint16_t *>(out) + row_off;
+  auto pack2 = [&](int db, int i) {
+    return (uint32_t)MT::cvt_bits(oacc[db][i] * inv) | ((uint32_t)MT::cvt_bits(oacc[db][i + 1] * inv) << 16);
+  };
+#pragma unroll
+  for (int db = 0; db < DB; db++) {
+    if constexpr (WIDE16) {
+#pragma unroll
+      for (int pr = 0; pr < 2; pr++) {
+        // w[0..1] = the even group (i4 = 2 pr), w[2..3] = the odd group (i4 = 2 pr + 1)
+        float w[4];
+#pragma unroll
+        for (int h = 0; h < 2; h++)
+#pragma unroll
+          for (int j = 0; j < 2; j++) w[2 * h + j] = __uint_as_float(pack2(db, 4 * (2 * pr + h) + 2 * j));
+        // afterwards the lower lanes hold (their even dims 0..3, the upper lanes' even dims 4..7) and the upper lanes
+        // (the lower lanes' odd dims 0..3, their own odd dims 4..7)
+        swap_wave_halves(w[0], w[2]);
+        swap_wave_halves(w[1], w[3]);
+        const int d = db * 32 + 8 * (2 * pr + g);
+        if (d >= d_valid) continue;
+        *reinterpret_cast<uint4 *>(op + d) =
+            make_uint4(__float_as_uint(w[0]), __float_as_uint(w[1]), __float_as_uint(w[2]), __float_as_uint(w[3]));
+      }
+    } else {
+#pragma unroll
+      for (int i4 = 0; i4 < 4; i4++) {
+        const int d = db * 32 + 8 * i4 + 4 * g;
+        if (d >= d_valid) continue;
+        *reinterpret_cast<uint2 *>(op + d) = make_uint2(pack2(db, 4 * i4), pack2(db, 4 * i4 + 2));
+      }
+    }
+  }
+}
+
 }  // namespace
 }  // namespace lmh
