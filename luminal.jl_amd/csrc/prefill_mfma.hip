@@ -29,9 +29,10 @@
 #include "prefill_mfma.hpp"
 #include "rope.hpp"
 
-#if (defined(LMH_FOLD_SCALE) || defined(LMH_ONLY_XCDS) || defined(LMH_WIDE_MARGIN) || defined(LMH_W64_KERNEL) || defined(LMH_NO_PAIR_KERNEL)) && \
+#if (defined(LMH_FOLD_SCALE) || defined(LMH_ONLY_XCDS) || defined(LMH_WIDE_MARGIN) || defined(LMH_W64_KERNEL) || defined(LMH_NO_PAIR_KERNEL) || \
+     defined(LMH_BF16_SPLIT_P)) && \
     !defined(LMH_MEASUREMENT_BUILD)
-#error "LMH_FOLD_SCALE / LMH_ONLY_XCDS / LMH_WIDE_MARGIN / LMH_W64_KERNEL / LMH_NO_PAIR_KERNEL are experiment switches: they need -DLMH_MEASUREMENT_BUILD, which marks the library"
+#error "LMH_FOLD_SCALE / LMH_ONLY_XCDS / LMH_WIDE_MARGIN / LMH_W64_KERNEL / LMH_NO_PAIR_KERNEL / LMH_BF16_SPLIT_P are experiment switches: they need -DLMH_MEASUREMENT_BUILD, which marks the library"
 #endif
 
 #ifndef LMH_WIDE_MARGIN
@@ -112,6 +113,8 @@ __global__ __launch_bounds__(64 * NW, WPS) void prefill_mfma_kernel(PrefillArgs 
   // D is the tiled head dim; the tensors' own head dim a.D may be smaller (any multiple of 8): the
   // missing columns are never fetched (zeros in Q, K and V) and never stored.
   const int cpr = a.D / 8;         // 16-byte chunks per K/V row in memory
+  constexpr bool CV = MT::kConvertV;  // V tiles rewritten as fp16 on their way into LDS
+  using pvec8 = typename MT::pvec8;
   constexpr int LDK = D + kPadK;   // LDS row strides in elements
   constexpr int LDV = D + pad_v<D>();
 
@@ -247,10 +250,83 @@ __global__ __launch_bounds__(64 * NW, WPS) void prefill_mfma_kernel(PrefillArgs 
     for (int j = 0; j < KJ; j++)
       if (wave_u + NW * j < KI)
         load_block(k_desc, k_lds0 + buf * (BT * LDK * 2) + j * (NW * 1024), k_voff[j], kt * k_tile_bytes);
+    if constexpr (!CV) {
 #pragma unroll
-    for (int j = 0; j < VJ; j++)
-      if (wave_u + NW * j < VI)
-        load_block(v_desc, v_lds0 + buf * (BT * LDV * 2) + j * (NW * 1024), v_voff[j], kt * v_tile_bytes);
+      for (int j = 0; j < VJ; j++)
+        if (wave_u + NW * j < VI)
+          load_block(v_desc, v_lds0 + buf * (BT * LDV * 2) + j * (NW * 1024), v_voff[j], kt * v_tile_bytes);
+    }
+  };
+
+  // ---- MT::kConvertV: V tiles pass through registers and are stored in LDS as fp16 relative to the largest finite |v|
+  // met so far. Tile kt + 1 is rewritten during iteration kt from registers loaded during iteration kt - 1; the
+  // workgroup agrees on the largest value through v_top[parity of the tile], posted before the tile's barrier (only by
+  // threads whose own largest exponent exceeds what they already know of) and read by everyone after it. A slot is
+  // posted to again two barriers later, after every thread has read it, and never shrinks. ----
+  constexpr int DC = D / 8;                                              // 16-byte chunks per tiled V row
+  constexpr int VR = CV ? (BT * DC + 64 * NW - 1) / (64 * NW) : 1;       // chunks per thread and tile
+  __shared__ uint32_t v_top[2];
+  uint4 vreg[VR];
+  int vr_voff[VR], vr_lds[VR];
+  uint32_t top_run = 0;    // largest finite |v| bits up to the tile last rewritten (the same in every thread)
+  int thr_next = 0, thr_cur = 0, thr_acc = 0;  // exponent base of the tile last rewritten / in use / of the accumulators
+  bool v_special = false;  // this thread's registers hold an infinity or a NaN
+  const __amdgpu_buffer_rsrc_t v_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<uint16_t *>(vp), 0, __builtin_amdgcn_readfirstlane((int)((int64_t)n_keys * a.vs[2] * 2)), 0x00020000);
+  if constexpr (CV) {
+#pragma unroll
+    for (int j = 0; j < VR; j++) {
+      const int ch = tid + j * (64 * NW);
+      const int row = ch / DC, col = ch % DC;
+      vr_voff[j] = (ch < BT * DC && col < cpr) ? (int)((row * a.vs[2] + col * 8) * 2) : kOutOfRange;
+      vr_lds[j] = (row * LDV + col * 8) * 2;
+    }
+  }
+  auto fetch_v = [&](int kt) {
+    const int soff = __builtin_amdgcn_readfirstlane(kt * v_tile_bytes);
+#pragma unroll
+    for (int j = 0; j < VR; j++) vreg[j] = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(v_rsrc, vr_voff[j], soff, 0));
+  };
+  auto post_top = [&](int slot) {
+    u16x2_t all = {0, 0};
+#pragma unroll
+    for (int j = 0; j < VR; j++) {
+      const uint32_t w[4] = {vreg[j].x, vreg[j].y, vreg[j].z, vreg[j].w};
+#pragma unroll
+      for (int e = 0; e < 4; e++) all = __builtin_elementwise_max(all, __builtin_bit_cast(u16x2_t, w[e] & 0x7fff7fffu));
+    }
+    uint32_t m = max((uint32_t)all[0], (uint32_t)all[1]);
+    v_special = m >= 0x7f80u;
+    if (v_special) {
+      m = 0;
+#pragma unroll
+      for (int j = 0; j < VR; j++) {
+        m = bf16x2_finite_top(vreg[j].x, m);
+        m = bf16x2_finite_top(vreg[j].y, m);
+        m = bf16x2_finite_top(vreg[j].z, m);
+        m = bf16x2_finite_top(vreg[j].w, m);
+      }
+    }
+    if ((m >> 7) > (top_run >> 7)) atomicMax(&v_top[slot], m);
+  };
+  auto rewrite_v = [&](int buf) {  // after the barrier that follows post_top(buf)
+    top_run = max(top_run, v_top[buf]);
+    thr_next = max((int)(top_run >> 7) - 29, 0);
+    const uint32_t tb2 = ((uint32_t)thr_next << 7) * 0x00010001u;
+    char *dst = reinterpret_cast<char *>(&Vs2[buf][0]);
+#pragma unroll
+    for (int j = 0; j < VR; j++) {
+      if ((BT * DC) % (64 * NW) != 0 && tid + j * (64 * NW) >= BT * DC) continue;
+      uint4 o;
+      if (!v_special) {
+        o = make_uint4(bf16x2_to_scaled_f16x2(vreg[j].x, tb2), bf16x2_to_scaled_f16x2(vreg[j].y, tb2),
+                       bf16x2_to_scaled_f16x2(vreg[j].z, tb2), bf16x2_to_scaled_f16x2(vreg[j].w, tb2));
+      } else {
+        o = make_uint4(bf16x2_to_scaled_f16x2_any(vreg[j].x, tb2), bf16x2_to_scaled_f16x2_any(vreg[j].y, tb2),
+                       bf16x2_to_scaled_f16x2_any(vreg[j].z, tb2), bf16x2_to_scaled_f16x2_any(vreg[j].w, tb2));
+      }
+      *reinterpret_cast<uint4 *>(dst + vr_lds[j]) = o;
+    }
   };
 
   // lane-constant pieces of the LDS addresses
@@ -262,6 +338,17 @@ __global__ __launch_bounds__(64 * NW, WPS) void prefill_mfma_kernel(PrefillArgs 
   // + (kb*32 + 16*t [+8]) * LDV + db*32
 
   if (n_kv_tiles > 0) load_tile(0, 0);
+  if constexpr (CV) {
+    if (tid < 2) v_top[tid] = 0;
+    if (n_kv_tiles > 0) fetch_v(0);
+    __syncthreads();
+    if (n_kv_tiles > 0) {
+      post_top(0);
+      __syncthreads();
+      rewrite_v(0);
+      if (n_kv_tiles > 1) fetch_v(1);
+    }
+  }
   // (the second K buffer is not written before the loop's first barrier: room for the inv_freq table)
   if (a.q_rope) rotate_q_fragments<MT, D>(qreg, a, b, qi, g, reinterpret_cast<float *>(&Ks2[1][0]));
   // The compiler does not model the asm loads or the asm wait below. Make it wait for Q here;
@@ -274,8 +361,17 @@ __global__ __launch_bounds__(64 * NW, WPS) void prefill_mfma_kernel(PrefillArgs 
     // One barrier per tile: tile kt (fetched during the previous iteration) becomes visible, and every
     // wave is done with tile kt-1, whose buffer the fetch of tile kt+1 now overwrites.
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wave's blocks of tile kt are in LDS
+    if constexpr (CV)
+      if (kt + 1 < n_kv_tiles) post_top((kt + 1) & 1);  // (its registers hold V of tile kt + 1)
     __syncthreads();  // ... and everyone's; tile kt-1 has been consumed, its buffer is free
     if (kt + 1 < n_kv_tiles) load_tile(kt + 1, (kt + 1) & 1);  // in flight while tile kt is computed
+    if constexpr (CV) {
+      thr_cur = thr_next;
+      if (kt + 1 < n_kv_tiles) {
+        rewrite_v((kt + 1) & 1);
+        if (kt + 2 < n_kv_tiles) fetch_v(kt + 2);
+      }
+    }
     const uint16_t *Ks = Ks2[kt & 1] + kg * (BW * LDK);
     const uint16_t *Vs = Vs2[kt & 1] + kg * (BW * LDV);
 
@@ -363,7 +459,7 @@ __global__ __launch_bounds__(64 * NW, WPS) void prefill_mfma_kernel(PrefillArgs 
     }
 #endif
     const float mc = m_i * c;
-    vec8 pf[NKB][2], pf_lo[NKB][2];
+    pvec8 pf[NKB][2], pf_lo[NKB][2];
 #pragma unroll
     for (int kb = 0; kb < NKB; kb++)
 #pragma unroll
@@ -375,14 +471,25 @@ __global__ __launch_bounds__(64 * NW, WPS) void prefill_mfma_kernel(PrefillArgs 
 #else
           const float p = __builtin_amdgcn_exp2f(sacc[kb][8 * t + e] * c - mc);
 #endif
-          pf[kb][t][e] = MT::cvt(p);
-          if (MT::kSplitP) pf_lo[kb][t][e] = MT::cvt(p - (float)pf[kb][t][e]);
+          pf[kb][t][e] = MT::cvt_p(p);
+          if (MT::kSplitP) pf_lo[kb][t][e] = MT::cvt_p(p - (float)pf[kb][t][e]);
         }
         l_i = MT::sum8(pf[kb][t], l_i);
         if (MT::kSplitP) l_i = MT::sum8(pf_lo[kb][t], l_i);
       }
 
     // ---- O^T += V^T P^T ----
+    if constexpr (CV) {
+      if (thr_cur != thr_acc) {  // this tile's V is stored against a larger value than the accumulated ones
+        const int d = thr_cur - thr_acc;
+        const float f = d < 127 ? __uint_as_float((uint32_t)(127 - d) << 23) : 0.f;
+        thr_acc = thr_cur;
+#pragma unroll
+        for (int db = 0; db < DB; db++)
+#pragma unroll
+          for (int i = 0; i < 16; i++) oacc[db][i] *= f;
+      }
+    }
 #pragma unroll
     for (int kb = 0; kb < NKB; kb++) {
 #pragma unroll
@@ -393,8 +500,8 @@ __global__ __launch_bounds__(64 * NW, WPS) void prefill_mfma_kernel(PrefillArgs 
           const shortx4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_shortx4_t *)(vaddr));
           const shortx4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_shortx4_t *)(vaddr + 8 * LDV));
           const shortx8_t v8 = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-          oacc[db] = MT::mfma(__builtin_bit_cast(vec8, v8), pf[kb][t], oacc[db]);
-          if (MT::kSplitP) oacc[db] = MT::mfma(__builtin_bit_cast(vec8, v8), pf_lo[kb][t], oacc[db]);
+          oacc[db] = MT::mfma_pv(__builtin_bit_cast(vec8, v8), pf[kb][t], oacc[db]);
+          if (MT::kSplitP) oacc[db] = MT::mfma_pv(__builtin_bit_cast(vec8, v8), pf_lo[kb][t], oacc[db]);
         }
       }
     }
@@ -403,6 +510,13 @@ __global__ __launch_bounds__(64 * NW, WPS) void prefill_mfma_kernel(PrefillArgs 
 #ifdef LMH_FOLD_SCALE
   m_i = have_m ? -neg_mc / c : -INFINITY;  // back to the units the merge below works in
 #endif
+  if constexpr (CV) {  // the accumulators hold O * 2^(112 - thr_acc)
+    const float f = __uint_as_float((uint32_t)(thr_acc + 15) << 23);
+#pragma unroll
+    for (int db = 0; db < DB; db++)
+#pragma unroll
+      for (int i = 0; i < 16; i++) oacc[db][i] *= f;
+  }
   // ---- key groups: fold group 1's (m, l, O) into group 0's; lane for lane the same layout ----
   if (KSPLIT > 1) {
     constexpr int NF = DB * 16 + 2;  // floats per lane
@@ -690,6 +804,7 @@ __global__ __launch_bounds__(1024, 4) void prefill_mfma_wide_kernel(PrefillArgs 
 template <typename MT, int D, bool CAUSAL>
 __global__ __launch_bounds__(512, 2) void prefill_mfma_pair_kernel(PrefillArgs a, int n_q_tiles, int n_bh_groups) {
   using vec8 = typename MT::vec8;
+  static_assert(!MT::kSplitP && !MT::kConvertV, "one weight fragment per V fragment, V tiles staged as they are: fp16");
   constexpr int NW = 8, BM = 256;
   constexpr int BT = 2 * BN;        // 128 keys per staged tile
   constexpr int NKB = BT / 32;
@@ -843,7 +958,7 @@ __global__ __launch_bounds__(512, 2) void prefill_mfma_pair_kernel(PrefillArgs a
 #pragma unroll
         for (int rb = RB0; rb < 2; rb++) sacc[rb][kb] = MT::mfma(kf, qreg[rb][ks], sacc[rb][kb]);
       }
-    vec8 pf[2][NB][2], pf_lo[2][NB][2];
+    vec8 pf[2][NB][2];
 #pragma unroll
     for (int rb = RB0; rb < 2; rb++) {
       if (k0 + 32 * NB > n_keys || (CAUSAL && k0 + 32 * NB - 1 > qlo[rb])) {  // the ragged last block, or a block on this row block's diagonal
@@ -882,10 +997,8 @@ __global__ __launch_bounds__(512, 2) void prefill_mfma_pair_kernel(PrefillArgs a
           for (int e = 0; e < 8; e++) {
             const float p = __builtin_amdgcn_exp2f(sacc[rb][kb][8 * t + e] * c - mc);
             pf[rb][kb][t][e] = MT::cvt(p);
-            if (MT::kSplitP) pf_lo[rb][kb][t][e] = MT::cvt(p - (float)pf[rb][kb][t][e]);
           }
           l_i[rb] = MT::sum8(pf[rb][kb][t], l_i[rb]);
-          if (MT::kSplitP) l_i[rb] = MT::sum8(pf_lo[rb][kb][t], l_i[rb]);
         }
     }
 #pragma unroll
@@ -901,7 +1014,6 @@ __global__ __launch_bounds__(512, 2) void prefill_mfma_pair_kernel(PrefillArgs a
 #pragma unroll
           for (int rb = RB0; rb < 2; rb++) {
             oacc[rb][db] = MT::mfma(v8, pf[rb][kb][t], oacc[rb][db]);
-            if (MT::kSplitP) oacc[rb][db] = MT::mfma(v8, pf_lo[rb][kb][t], oacc[rb][db]);
           }
         }
   };
@@ -962,7 +1074,7 @@ __global__ __launch_bounds__(512, 2) void prefill_mfma_pair_kernel(PrefillArgs a
         for (int i = 0; i < 16; i++) oacc[rb][db][i] *= alpha;
     }
     const float mc = m_i[rb] * c;
-    vec8 pf[NKB][2], pf_lo[NKB][2];
+    vec8 pf[NKB][2];
 #pragma unroll
     for (int kb = 0; kb < NKB; kb++)
 #pragma unroll
@@ -971,10 +1083,8 @@ __global__ __launch_bounds__(512, 2) void prefill_mfma_pair_kernel(PrefillArgs a
         for (int e = 0; e < 8; e++) {
           const float p = __builtin_amdgcn_exp2f(sacc[kb][8 * t + e] * c - mc);
           pf[kb][t][e] = MT::cvt(p);
-          if (MT::kSplitP) pf_lo[kb][t][e] = MT::cvt(p - (float)pf[kb][t][e]);
         }
         l_i[rb] = MT::sum8(pf[kb][t], l_i[rb]);
-        if (MT::kSplitP) l_i[rb] = MT::sum8(pf_lo[kb][t], l_i[rb]);
       }
 #pragma unroll
     for (int kb = 0; kb < NKB; kb++)
@@ -987,7 +1097,6 @@ __global__ __launch_bounds__(512, 2) void prefill_mfma_pair_kernel(PrefillArgs a
           const shortx4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_shortx4_t *)(vaddr + 8 * LDV));
           const vec8 v8 = __builtin_bit_cast(vec8, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
           oacc[rb][db] = MT::mfma(v8, pf[kb][t], oacc[rb][db]);
-          if (MT::kSplitP) oacc[rb][db] = MT::mfma(v8, pf_lo[kb][t], oacc[rb][db]);
         }
   };
   const std::integral_constant<int, 0> kBoth{};
@@ -1061,8 +1170,18 @@ int launch_pair(const PrefillArgs &a, hipStream_t stream) {
   return LMH_OK;
 }
 
-template <typename MT, int D, int KSPLIT, int NW, int WPS = default_wps<D, NW>()>
+// The policy prefill_mfma_kernel runs a tensor type with. bf16: V rewritten as fp16 in the workgroups that own their
+// query rows alone (B=1 H=32 S=4096 causal D=96 151 -> 122 us, D=128 202 -> 174, D=64 x 4 batches 443 -> 350; without a
+// mask -15 ... -24 %); the small launches whose wave pairs split the keys keep head + remainder weights and LDS-direct V
+// tiles (the rewrite sits on their critical path: 8 heads x 1024 rows 14.8 -> 20.6 us, 64 heads x 1024 rows 31.3 -> 35.6).
+template <typename MT, int KSPLIT> struct base_policy { using type = MT; };
+#ifndef LMH_BF16_SPLIT_P
+template <> struct base_policy<MfmaBF16, 1> { using type = MfmaBF16V16; };
+#endif
+
+template <typename MT0, int D, int KSPLIT, int NW, int WPS = default_wps<D, NW>()>
 int launch_split(const PrefillArgs &a, hipStream_t stream) {
+  using MT = typename base_policy<MT0, KSPLIT>::type;
   constexpr int BM = 32 * NW / KSPLIT;
   const int n_q_tiles = (a.Sq + BM - 1) / BM;
   const int n_bh_groups = (a.B * a.Hq + 7) / 8;
@@ -1132,16 +1251,16 @@ int launch_for_d(const PrefillArgs &a, hipStream_t stream) {
   // 256 CUs, fp16: B=1 H=32 S=4096 D=96 -3.2 %, D=64 -6 %, D=80 -3 %; B=2 H=32 S=2048 -5 %; H=8 S=16384 -4.6 %;
   // S=3900 -2 %. With the chip not exactly full it loses (1.25 rounds +23 %, 1.5 rounds +10 %, half a round +30 %),
   // at exactly two rounds it ties (-1.4 ... +7 %).
-  // bf16 (weights as head + remainder: twice the weight registers) only at D <= 64 and only causal: B=1 H=32 S=4096
-  // D=64 -8 %, H=64 S=2048 -6 %; D=96 +1 % causal (and spills with two blocks at a time), -2.5 % without a mask.
+  // bf16 stays on the kernels below: this one takes bf16 weights as head + remainder and V tiles as they are, and the
+  // fp16 rewrite of V that prefill_mfma_kernel does gains more (B=1 H=32 S=4096 D=64 causal: 117.7 us here, 99.8 us there).
 #ifndef LMH_NO_PAIR_KERNEL  // (measurement builds can keep these launches on the kernels below, for comparisons with them)
-  if constexpr (D <= 96 && (!MT::kSplitP || D <= 64)) {
+  if constexpr (D <= 96 && !MT::kSplitP) {
     const int64_t wgs_pair = (int64_t)((a.B * a.Hq + 7) / 8) * 8 * (((a.Sq + 255) / 256 + 1) / 2);
     if (a.causal && a.Sq > 256 && wgs_pair <= n_cus && 16 * wgs_pair >= 15 * n_cus) return launch_pair<MT, D>(a, stream);
     // Without a mask the same kernel takes two neighbouring tiles (512 rows, every fragment read shared all the way);
     // its workgroups are equal, so it wants whole rounds: B=1 H=32 S=4096 D=96 (one round) -5.9 %, S=8192 (two) -3.5 %,
     // B=4 (four) -1.1 %; D=64 one round -2.4 %, two rounds +2.5 %; 1.25 rounds +20 %.
-    if (!a.causal && !MT::kSplitP && a.Sq > 256 && wgs_pair >= n_cus) {
+    if (!a.causal && a.Sq > 256 && wgs_pair >= n_cus) {
       const int64_t rounds = (wgs_pair + n_cus - 1) / n_cus, last = wgs_pair - (rounds - 1) * n_cus;
       if (16 * last >= 15 * n_cus && (rounds == 1 || (D > 64 && rounds <= 2))) return launch_pair<MT, D>(a, stream);
     }
@@ -1161,8 +1280,8 @@ int launch_for_d(const PrefillArgs &a, hipStream_t stream) {
   // (too few to balance their unequal lengths), 1024 +3 %, 1536 +4..7 %, 2048 +5 %.
   // D = 128 does not fit the 128 registers that four waves per SIMD leave: one 256-row workgroup per CU there,
   // which turns over in rounds and balances earlier. fp16: non-causal 256 / 512 / 2048 workgroups +5 / +3 / +6 %,
-  // causal 256 / 384 -8 / -5 %, 512 / 1024 / 2048 +8 / +3 / +4 %; bf16 (more registers, more MFMAs per staged
-  // tile) 0 / -2 %: stays on 128 rows.
+  // causal 256 / 384 -8 / -5 %, 512 / 1024 / 2048 +8 / +3 / +4 %; bf16 (V rewritten as fp16) 512 workgroups causal
+  // +8 %, without a mask +5 %, 2048 causal +5 %.
   const int64_t wgs256 = (int64_t)((a.B * a.Hq + 7) / 8) * 8 * ((a.Sq + 255) / 256);
   if (a.Sq <= 128) return launch_split<MT, D, 1, 4>(a, stream);  // nothing for waves 4-7 to own
   if constexpr (D <= 96) {
@@ -1173,11 +1292,13 @@ int launch_for_d(const PrefillArgs &a, hipStream_t stream) {
     // bf16 164 -> 153 us), 2.25 / 2.5 rounds +1 %, 3 and 3.5 rounds +-0; one round -20 %; D = 64 (2 rounds) -5 %.
     // Non-causal workgroups are all equally long and a part-filled round is lost time: from two rounds on only
     // (2 rounds +1 %, bf16 +4 %; 2.5 rounds +3 %; 1.5 rounds -11 %).
+    // bf16 (V rewritten as fp16 through registers) spills at four waves per SIMD and stays on this form however many
+    // rounds there are: B=4 H=32 S=4096 causal 583 -> 507 us, without a mask 946 -> 892 us.
     if constexpr (D == 96)
-      if (wgs256 < 3 * n_cus && (a.causal ? 2 * wgs256 >= 3 * n_cus : wgs256 >= 2 * n_cus))
+      if ((MT::kSplitP || wgs256 < 3 * n_cus) && (a.causal ? 2 * wgs256 >= 3 * n_cus : wgs256 >= 2 * n_cus))
         return launch_split<MT, D, 1, 8, 2>(a, stream);
     if (wgs256 >= (a.causal ? 4 * n_cus : 2 * n_cus)) return launch_split<MT, D, 1, 8>(a, stream);
-  } else if constexpr (!MT::kSplitP) {
+  } else {
     if (wgs256 >= (a.causal ? 2 * n_cus : n_cus)) return launch_split<MT, D, 1, 8>(a, stream);
   }
   return launch_split<MT, D, 1, 4>(a, stream);

@@ -34,11 +34,15 @@ struct MfmaF16 {
   static constexpr const char *kName = "f16";
   using vec8 = half8_t;
   static constexpr bool kSplitP = false;  // 11 significant bits in P are within the 2e-3 budget
+  static constexpr bool kConvertV = false;
+  using pvec8 = vec8;  // the softmax weights, as the matrix cores take them
   __device__ static floatx16_t mfma(vec8 a, vec8 b, floatx16_t c) {
     return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
   }
   __device__ static uint16_t cvt_bits(float x) { return __builtin_bit_cast(uint16_t, (_Float16)x); }
   __device__ static _Float16 cvt(float x) { return (_Float16)x; }
+  __device__ static _Float16 cvt_p(float x) { return (_Float16)x; }
+  __device__ static floatx16_t mfma_pv(vec8 v, pvec8 p, floatx16_t c) { return mfma(v, p, c); }
   // acc + sum of the 8 (already rounded) elements: 4 x v_dot2_f32_f16 against (1, 1)
   __device__ static float sum8(vec8 p, float acc) {
     typedef _Float16 h2 __attribute__((ext_vector_type(2)));
@@ -56,11 +60,15 @@ struct MfmaBF16 {
   // A bf16 P has 8 significant bits; on short or peaked rows that alone is ~2.5e-3 of the output
   // range. P is therefore fed to the matrix cores as head + remainder (two MFMAs per V fragment).
   static constexpr bool kSplitP = true;
+  static constexpr bool kConvertV = false;
+  using pvec8 = vec8;
   __device__ static floatx16_t mfma(vec8 a, vec8 b, floatx16_t c) {
     return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
   }
   __device__ static uint16_t cvt_bits(float x) { return f32_to_bf16_bits(x); }
   __device__ static __bf16 cvt(float x) { return (__bf16)x; }
+  __device__ static __bf16 cvt_p(float x) { return (__bf16)x; }
+  __device__ static floatx16_t mfma_pv(vec8 v, pvec8 p, floatx16_t c) { return mfma(v, p, c); }
   __device__ static float sum8(vec8 p, float acc) {
     typedef __bf16 b2 __attribute__((ext_vector_type(2)));
     const b2 one = {(__bf16)1.f, (__bf16)1.f};
@@ -72,6 +80,48 @@ struct MfmaBF16 {
   }
 };
 
+
+// bf16 tensors with the second product in fp16: S^T = K Q^T runs on the bf16 MFMA (its operands are exact), the
+// softmax weights are rounded to fp16 (11 significant bits, one MFMA per V fragment instead of head + remainder) and
+// the V tiles are rewritten as fp16 on their way into LDS. A bf16 value has 8 significant bits, so the rewrite is exact
+// once the exponent fits: every tile is stored relative to the largest finite |v| the workgroup has met so far (that
+// value lands at 2^14), values more than 2^29 below it go to zero, and the accumulators carry the power of two.
+struct MfmaBF16V16 : MfmaBF16 {
+  static constexpr bool kSplitP = false;
+  static constexpr bool kConvertV = true;
+  using pvec8 = half8_t;
+  __device__ static _Float16 cvt_p(float x) { return (_Float16)x; }
+  __device__ static floatx16_t mfma_pv(vec8 v, pvec8 p, floatx16_t c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(half8_t, v), p, c, 0, 0, 0);
+  }
+  __device__ static float sum8(pvec8 p, float acc) { return MfmaF16::sum8(p, acc); }
+};
+
+// One 32-bit word = two bf16 values -> two fp16 values holding v * 2^(112 - thr) (thr = the biased bf16 exponent that
+// maps to the fp16 exponent field 0): exponent and mantissa bits shifted into place with 16-bit packed integer
+// instructions, no float arithmetic. Finite inputs whose exponent is at most thr come out as zero or as an fp16
+// subnormal (|result| < 2^-14); the caller guarantees exponent - thr <= 29 for every finite input.
+typedef uint16_t u16x2_t __attribute__((ext_vector_type(2)));
+__device__ inline uint32_t bf16x2_to_scaled_f16x2(uint32_t w, uint32_t thr_bits2) {
+  const u16x2_t t = __builtin_bit_cast(u16x2_t, w & 0x7fff7fffu);
+  const u16x2_t e = __builtin_elementwise_sub_sat(t, __builtin_bit_cast(u16x2_t, thr_bits2));
+  const u16x2_t three = {3, 3};
+  return (w & 0x80008000u) | __builtin_bit_cast(uint32_t, (u16x2_t)(e << three));
+}
+// the same for a word that may hold infinities or NaNs (kept as such)
+__device__ inline uint32_t bf16x2_to_scaled_f16x2_any(uint32_t w, uint32_t thr_bits2) {
+  uint32_t r = bf16x2_to_scaled_f16x2(w, thr_bits2);
+  if ((w & 0x7f80u) == 0x7f80u) r = (r & 0xffff0000u) | (w & 0x8000u) | 0x7c00u | ((w & 0x7fu) ? 0x200u : 0u);
+  if ((w & 0x7f800000u) == 0x7f800000u) r = (r & 0x0000ffffu) | (w & 0x80000000u) | 0x7c000000u | ((w & 0x7f0000u) ? 0x2000000u : 0u);
+  return r;
+}
+// largest |bits| (exponent and mantissa, 15 bits) over the finite halves of a word, folded into m
+__device__ inline uint32_t bf16x2_finite_top(uint32_t w, uint32_t m) {
+  const uint32_t lo = w & 0x7fffu, hi = (w >> 16) & 0x7fffu;
+  if (lo < 0x7f80u) m = max(m, lo);
+  if (hi < 0x7f80u) m = max(m, hi);
+  return m;
+}
 
 // Epilogue of the matrix-core flash attention kernels: out[qi][d] = O^T[d][qi] * inv for the wave's 32 query rows.
 // In the accumulator layout lane (n, g) holds, per 32-row block db of O^T, four groups of four consecutive head dims:

@@ -67,7 +67,8 @@ CASES = [
     (1, 32, 8, 4096, 4096, 96, True, "f16", "prefill_mfma_pair_kernel<f16, D=96, causal>"),
     (1, 64, 64, 2000, 2000, 64, True, "f16", "prefill_mfma_pair_kernel<f16, D=64, causal>"),
     (1, 32, 8, 4096, 1100, 96, False, "f16", "prefill_mfma_pair_kernel<f16, D=96, full>"),
-    (1, 64, 64, 2000, 2000, 64, True, "bf16", "prefill_mfma_pair_kernel<bf16, D=64, causal>"),
+    (1, 64, 64, 2000, 2000, 64, True, "bf16", "prefill_mfma_kernel<bf16, D=64, causal, key groups=1"),
+    (1, 32, 8, 4096, 4096, 96, True, "bf16", "prefill_mfma_kernel<bf16, D=96, causal, key groups=1, waves=8"),
     (4, 20, 20, 448, 704, 64, False, "f16", "prefill_mfma_wide_kernel<f16, D=64>"),
     (4, 20, 20, 448, 704, 96, False, "bf16", "prefill_mfma_wide_kernel<bf16, D=96>"),
     (1, 4, 2, 160, 160, 64, True, "f32", "prefill_f32_kernel<D=64, causal"),

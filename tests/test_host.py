@@ -173,10 +173,13 @@ def test_kernel_plan_of_the_benchmark_configurations(lm):
     # C2: 32 heads x 16 tiles of 256 rows = 256 pairs (tile p with tile 15 - p), one workgroup per CU, one round
     assert plan((1, 32, 4096, 96), (1, 32, 4096, 96), "f16", True) == \
         "prefill_mfma_pair_kernel<f16, D=96, causal> query tiles=16, workgroups=256"
-    # the same in bf16 (head + remainder weights: no room for two row blocks), or with the chip not exactly full:
-    # 512 workgroups of 256 rows, one per CU at a time, 128-key tiles
+    # the same in bf16 (V rewritten as fp16 through registers: no room for two row blocks), or with the chip not exactly
+    # full: 512 workgroups of 256 rows, one per CU at a time, 128-key tiles
     assert plan((1, 32, 4096, 96), (1, 32, 4096, 96), "bf16", True).startswith(
         "prefill_mfma_kernel<bf16, D=96, causal, key groups=1, waves=8, waves per SIMD=2> workgroups=512")
+    # ... in bf16 however many rounds there are (fp16 goes to two workgroups per CU from three rounds on)
+    assert "waves=8, waves per SIMD=2> workgroups=2048" in plan((4, 32, 4096, 96), (4, 32, 4096, 96), "bf16", True)
+    assert "waves=8, waves per SIMD=4> workgroups=2048" in plan((4, 32, 4096, 96), (4, 32, 4096, 96), "f16", True)
     assert plan((1, 40, 4096, 96), (1, 40, 4096, 96), "f16", True).startswith(
         "prefill_mfma_kernel<f16, D=96, causal, key groups=1, waves=8, waves per SIMD=2> workgroups=640")
     # C3: 80 heads x 14 row blocks on 256 CUs -> three workgroups per head of five row blocks x three key groups
