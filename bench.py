@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the attention hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--only all|prefill|decode|other|c1|nomask|c3|c4|ops|step|copy|ceiling|grid]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--only all|prefill|decode|other|c1|nomask|bf16|c3|c4|ops|step|copy|ceiling|grid]
 
 A step is one pass of the hot path over one batch of synthetic input, inputs resident in HBM:
   prefill leg (the headline `value`): causal flash attention, Phi-3-mini shape
@@ -378,6 +378,33 @@ def nomask_leg(lm, dev, res, check, zero_operands=True):
             raise SystemExit("parity check failed on %s: rel err %.3g > 2e-3" % (name, err))
 
 
+def bf16_leg(lm, dev, res, check):
+    """The C2 shape in bf16 (an extra line, not one of the five configurations): the element type of most models' prompts.
+    The kernel rewrites V as fp16 on its way into LDS and rounds the weights to fp16; parity against the oracle's bf16
+    inputs on four heads."""
+    name = "C2 shape in bf16 (causal B=1 H=32 S=4096 D=96)"
+    B, H, S, D = 1, 32, 4096, 96
+    hq, hk, hv = (lm.synth.normal((B, H, S, D), 2000 + i, 0.5) for i in range(3))
+    q, k, v = (lm.HipArray(x.shape, "bf16", dev).copy_from_host(x) for x in (hq, hk, hv))
+    o = lm.HipArray((B, H, S, D), "bf16", dev)
+    p = attn_params(lm, o, q, k, v, "bf16", True, lm.default_scale(D))
+    flops = 4.0 * B * H * D * S * (S + 1) / 2
+    _, ev = time_steps(lambda: lm.binding.flash_attn_fwd(p), 40, 5, lm.binding)
+    res[name] = {"launch_us": ev * 1e3, "TFLOP/s": flops / (ev * 1e-3) / 1e12, "frac_of_mfma_peak": flops / (ev * 1e-3) / 1e12 / PEAK_FP16_TFLOPS,
+                 "kernel": lm.binding.flash_attn_plan(p)}
+    log("[other] %s: %.1f us, %.1f TFLOP/s; %s" % (name, ev * 1e3, res[name]["TFLOP/s"], res[name]["kernel"]))
+    if check:
+        import oracle
+        heads = slice(0, 4)
+        qh, kh, vh = (np.asarray(x.to_host(), np.float32)[:, heads] for x in (q, k, v))
+        want = oracle.flash_attn(qh, kh, vh, scale=lm.default_scale(D), causal=True, nthreads=oracle.max_threads())
+        err = rel_err(np.asarray(o.to_host(), np.float32)[:, heads], want)
+        res[name]["parity"] = {"max_rel_err": err, "tolerance": 2e-3, "checked": "heads 0..3 vs CPU oracle"}
+        log("[other] %s: GPU vs oracle rel err %.2e" % (name, err))
+        if err > 2e-3:
+            raise SystemExit("parity check failed on %s: rel err %.3g > 2e-3" % (name, err))
+
+
 def c3_leg(lm, dev, res, check):
     flash_config(lm, dev, res, "C3 cross fp16 B=4 H=20 Sq=448 Sk=1500 D=64", 4, 20, 20, 448, 1500, 64, "f16", False,
                  4.0 * 4 * 20 * 448 * 1500 * 64, 3000, tol=2e-3 if check else None, steps=40, peak=PEAK_FP16_TFLOPS)
@@ -633,13 +660,15 @@ def ceiling_leg(lm, dev):
 def other_configs(lm, dev, check=False, only="other", zero_operands=True):
     """Short timings of the remaining contract configurations. With `check`, C1, C3 and C4 are also compared with the
     CPU oracle on the whole output (the parity gate of the five configurations: C2 and C5 are checked in their own
-    legs). `only` = "other" runs everything, or one of c1 / nomask / c3 / c4 / ops / step (a profile of one kernel)."""
+    legs). `only` = "other" runs everything, or one of c1 / nomask / bf16 / c3 / c4 / ops / step (a profile of one kernel)."""
     res = {}
     caches = None
     if only in ("other", "c1"):
         c1_leg(lm, dev, res, check)
     if only in ("other", "nomask"):
         nomask_leg(lm, dev, res, check, zero_operands)
+    if only in ("other", "bf16"):
+        bf16_leg(lm, dev, res, check)
     if only in ("other", "c3"):
         c3_leg(lm, dev, res, check)
     if only in ("other", "c4"):
@@ -694,7 +723,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--only", choices=["all", "prefill", "decode", "other", "c1", "nomask", "c3", "c4", "ops", "step", "copy", "ceiling", "grid"], default="all")
+    ap.add_argument("--only", choices=["all", "prefill", "decode", "other", "c1", "nomask", "bf16", "c3", "c4", "ops", "step", "copy", "ceiling", "grid"], default="all")
     ap.add_argument("--decode-splits", type=int, default=0, help="KV splits for the decode leg (0 = library heuristic)")
     ap.add_argument("--cpu-seconds", type=float, default=15.0, help="CPU-baseline budget per leg; 0 disables it")
     ap.add_argument("--no-zero-operands", action="store_true",
@@ -741,11 +770,11 @@ def main():
             line["cpu_baseline_single_thread"] = r["cpu_baseline_single_thread"]
     if args.only in ("all", "decode"):
         line["decode"] = decode_leg(lm, dev, args.steps, args.warmup, args.cpu_seconds, args.decode_splits)
-    if args.only in ("all", "other", "c1", "nomask", "c3", "c4", "ops", "step"):
+    if args.only in ("all", "other", "c1", "nomask", "bf16", "c3", "c4", "ops", "step"):
         line["other_configs"] = other_configs(lm, dev, check=args.cpu_seconds > 0, only="other" if args.only == "all" else args.only,
                                               zero_operands=not args.no_zero_operands)
     gate = [("C2", line.get("parity"))] + [("C5", line.get("decode", {}).get("parity"))] + \
-        [(k.split()[0] if k.split()[1] != "shape" else "C2 shape without the mask", v.get("parity"))
+        [(k.split()[0] if k.split()[1] != "shape" else k.split(" (")[0], v.get("parity"))
          for k, v in line.get("other_configs", {}).items() if isinstance(v, dict) and "parity" in v]
     gate = [(n, p) for n, p in gate if p]
     if gate:
