@@ -314,18 +314,21 @@ __global__ __launch_bounds__(64 * NW, WPS) void prefill_mfma_kernel(PrefillArgs 
     thr_next = max((int)(top_run >> 7) - 29, 0);
     const uint32_t tb2 = ((uint32_t)thr_next << 7) * 0x00010001u;
     char *dst = reinterpret_cast<char *>(&Vs2[buf][0]);
+    uint4 o[VR];
+#pragma unroll
+    for (int j = 0; j < VR; j++)
+      o[j] = make_uint4(bf16x2_to_scaled_f16x2(vreg[j].x, tb2), bf16x2_to_scaled_f16x2(vreg[j].y, tb2),
+                        bf16x2_to_scaled_f16x2(vreg[j].z, tb2), bf16x2_to_scaled_f16x2(vreg[j].w, tb2));
+    if (v_special) {
+#pragma unroll
+      for (int j = 0; j < VR; j++)
+        o[j] = make_uint4(bf16x2_to_scaled_f16x2_any(vreg[j].x, tb2), bf16x2_to_scaled_f16x2_any(vreg[j].y, tb2),
+                          bf16x2_to_scaled_f16x2_any(vreg[j].z, tb2), bf16x2_to_scaled_f16x2_any(vreg[j].w, tb2));
+    }
 #pragma unroll
     for (int j = 0; j < VR; j++) {
       if ((BT * DC) % (64 * NW) != 0 && tid + j * (64 * NW) >= BT * DC) continue;
-      uint4 o;
-      if (!v_special) {
-        o = make_uint4(bf16x2_to_scaled_f16x2(vreg[j].x, tb2), bf16x2_to_scaled_f16x2(vreg[j].y, tb2),
-                       bf16x2_to_scaled_f16x2(vreg[j].z, tb2), bf16x2_to_scaled_f16x2(vreg[j].w, tb2));
-      } else {
-        o = make_uint4(bf16x2_to_scaled_f16x2_any(vreg[j].x, tb2), bf16x2_to_scaled_f16x2_any(vreg[j].y, tb2),
-                       bf16x2_to_scaled_f16x2_any(vreg[j].z, tb2), bf16x2_to_scaled_f16x2_any(vreg[j].w, tb2));
-      }
-      *reinterpret_cast<uint4 *>(dst + vr_lds[j]) = o;
+      *reinterpret_cast<uint4 *>(dst + vr_lds[j]) = o[j];
     }
   };
 
@@ -365,19 +368,19 @@ __global__ __launch_bounds__(64 * NW, WPS) void prefill_mfma_kernel(PrefillArgs 
       if (kt + 1 < n_kv_tiles) post_top((kt + 1) & 1);  // (its registers hold V of tile kt + 1)
     __syncthreads();  // ... and everyone's; tile kt-1 has been consumed, its buffer is free
     if (kt + 1 < n_kv_tiles) load_tile(kt + 1, (kt + 1) & 1);  // in flight while tile kt is computed
-    if constexpr (CV) {
-      thr_cur = thr_next;
-      if (kt + 1 < n_kv_tiles) {
-        rewrite_v((kt + 1) & 1);
-        if (kt + 2 < n_kv_tiles) fetch_v(kt + 2);
-      }
-    }
+    if constexpr (CV) thr_cur = thr_next;
     const uint16_t *Ks = Ks2[kt & 1] + kg * (BW * LDK);
     const uint16_t *Vs = Vs2[kt & 1] + kg * (BW * LDV);
 
     const int k0 = kt * BT + kg * BW;         // first key of this wave's share of the tile
-    if (CAUSAL && k0 > wave_q_hi) continue;   // all of it above this wave's diagonal
-    if (KSPLIT > 1 && k0 >= k_end) continue;  // ... or past the last key (second half of the last tile)
+    // all of it above this wave's diagonal, or past the last key (second half of the last tile)
+    if ((CAUSAL && k0 > wave_q_hi) || (KSPLIT > 1 && k0 >= k_end)) {
+      if constexpr (CV) {
+        rewrite_v((kt + 1) & 1);
+        if (kt + 2 < n_kv_tiles) fetch_v(kt + 2);
+      }
+      continue;
+    }
 
     // ---- S^T = K Q^T for the wave's 32-key blocks, two at a time: their fragments are fetched first, then
     // the two accumulator chains alternate so that neither waits on LDS or on its own previous MFMA ----
@@ -405,6 +408,13 @@ __global__ __launch_bounds__(64 * NW, WPS) void prefill_mfma_kernel(PrefillArgs 
           sacc[kb0 + kb] = MT::mfma(kf[kb][ks], qreg[ks], sacc[kb0 + kb]);
 #endif
         }
+    }
+
+    // The next V tile is rewritten here, in the shadow of the MFMAs just issued. (After the last tile this rewrites
+    // stale registers into the buffer of tile kt - 1, which nobody reads any more.)
+    if constexpr (CV) {
+      rewrite_v((kt + 1) & 1);
+      if (kt + 2 < n_kv_tiles) fetch_v(kt + 2);
     }
 
     // ---- masking (diagonal tiles and the ragged last tile only) ----
