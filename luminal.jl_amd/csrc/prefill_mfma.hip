@@ -1303,9 +1303,12 @@ int launch_for_d(const PrefillArgs &a, hipStream_t stream) {
     // Non-causal workgroups are all equally long and a part-filled round is lost time: from two rounds on only
     // (2 rounds +1 %, bf16 +4 %; 2.5 rounds +3 %; 1.5 rounds -11 %).
     // bf16 (V rewritten as fp16 through registers) spills at four waves per SIMD and stays on this form however many
-    // rounds there are: B=4 H=32 S=4096 causal 583 -> 507 us, without a mask 946 -> 892 us.
-    if constexpr (D == 96)
-      if ((MT::kSplitP || wgs256 < 3 * n_cus) && (a.causal ? 2 * wgs256 >= 3 * n_cus : wgs256 >= 2 * n_cus))
+    // rounds there are: B=4 H=32 S=4096 causal 583 -> 507 us, without a mask 946 -> 892 us. At D = 64 it takes this form for
+    // causal launches of 1.5 to 3 rounds (the rewrite is shared by eight waves instead of four: B=1 H=32 S=4096 100.1 -> 96.5
+    // us, H=64 S=2048 60.3 -> 58.6); from three rounds on and without a mask two workgroups per CU are 6-10 % ahead there.
+    if constexpr (D == 96 || MT::kSplitP)
+      if ((D == 96 || a.causal) && ((D == 96 && MT::kSplitP) || wgs256 < 3 * n_cus) &&
+          (a.causal ? 2 * wgs256 >= 3 * n_cus : wgs256 >= 2 * n_cus))
         return launch_split<MT, D, 1, 8, 2>(a, stream);
     if (wgs256 >= (a.causal ? 4 * n_cus : 2 * n_cus)) return launch_split<MT, D, 1, 8>(a, stream);
   } else {
