@@ -1261,8 +1261,9 @@ int launch_for_d(const PrefillArgs &a, hipStream_t stream) {
   // 256 CUs, fp16: B=1 H=32 S=4096 D=96 -3.2 %, D=64 -6 %, D=80 -3 %; B=2 H=32 S=2048 -5 %; H=8 S=16384 -4.6 %;
   // S=3900 -2 %. With the chip not exactly full it loses (1.25 rounds +23 %, 1.5 rounds +10 %, half a round +30 %),
   // at exactly two rounds it ties (-1.4 ... +7 %).
-  // bf16 stays on the kernels below: this one takes bf16 weights as head + remainder and V tiles as they are, and the
-  // fp16 rewrite of V that prefill_mfma_kernel does gains more (B=1 H=32 S=4096 D=64 causal: 117.7 us here, 99.8 us there).
+  // bf16 stays on the kernels below: the fp16 rewrite of V that prefill_mfma_kernel does gains more than the pairing did
+  // with bf16 weights as head + remainder (B=1 H=32 S=4096 D=64 causal: 117.7 us here, 99.8 us there), and two row blocks
+  // plus the rewrite's registers do not fit; this kernel is built for fp16 only.
 #ifndef LMH_NO_PAIR_KERNEL  // (measurement builds can keep these launches on the kernels below, for comparisons with them)
   if constexpr (D <= 96 && !MT::kSplitP) {
     const int64_t wgs_pair = (int64_t)((a.B * a.Hq + 7) / 8) * 8 * (((a.Sq + 255) / 256 + 1) / 2);
