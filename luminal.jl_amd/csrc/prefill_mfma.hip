@@ -1180,24 +1180,22 @@ int launch_pair(const PrefillArgs &a, hipStream_t stream) {
   return LMH_OK;
 }
 
-// The policy prefill_mfma_kernel runs a tensor type with. bf16: V rewritten as fp16 in the workgroups that own their
-// query rows alone (B=1 H=32 S=4096 causal D=96 151 -> 122 us, D=128 202 -> 174, D=64 x 4 batches 443 -> 350; without a
-// mask -15 ... -24 %); the small launches whose wave pairs split the keys keep head + remainder weights and LDS-direct V
+// The policy prefill_mfma_kernel runs a tensor type with. bf16 with V16: V rewritten as fp16 in the workgroups that own
+// their query rows alone (B=1 H=32 S=4096 causal D=96 151 -> 122 us, D=128 202 -> 174, D=64 x 4 batches 443 -> 350; without
+// a mask -15 ... -24 %); the small launches whose wave pairs split the keys keep head + remainder weights and LDS-direct V
 // tiles (the rewrite sits on their critical path: 8 heads x 1024 rows 14.8 -> 20.6 us, 64 heads x 1024 rows 31.3 -> 35.6).
-template <typename MT, int KSPLIT> struct base_policy { using type = MT; };
-#ifndef LMH_BF16_SPLIT_P
-template <> struct base_policy<MfmaBF16, 1> { using type = MfmaBF16V16; };
-#endif
+template <typename MT, bool V16, int KSPLIT> struct base_policy { using type = MT; };
+template <> struct base_policy<MfmaBF16, true, 1> { using type = MfmaBF16V16; };
 
-template <typename MT0, int D, int KSPLIT, int NW, int WPS = default_wps<D, NW>()>
+template <typename MT0, bool V16, int D, int KSPLIT, int NW, int WPS = default_wps<D, NW>()>
 int launch_split(const PrefillArgs &a, hipStream_t stream) {
-  using MT = typename base_policy<MT0, KSPLIT>::type;
+  using MT = typename base_policy<MT0, V16, KSPLIT>::type;
   constexpr int BM = 32 * NW / KSPLIT;
   const int n_q_tiles = (a.Sq + BM - 1) / BM;
   const int n_bh_groups = (a.B * a.Hq + 7) / 8;
   dim3 grid(8 * n_bh_groups * n_q_tiles), block(64 * NW);
-  if (plan_only("prefill_mfma_kernel<%s, D=%d, %s, key groups=%d, waves=%d, waves per SIMD=%d> workgroups=%u", MT::kName, D,
-                a.causal ? "causal" : "full", KSPLIT, NW, WPS, grid.x))
+  if (plan_only("prefill_mfma_kernel<%s, D=%d, %s, key groups=%d, waves=%d, waves per SIMD=%d> workgroups=%u%s", MT::kName, D,
+                a.causal ? "causal" : "full", KSPLIT, NW, WPS, grid.x, MT::kConvertV ? ", V as fp16" : ""))
     return LMH_OK;
   if (a.causal)
     hipLaunchKernelGGL((prefill_mfma_kernel<MT, D, true, KSPLIT, NW, WPS>), grid, block, 0, stream, a, n_q_tiles, n_bh_groups);
@@ -1248,8 +1246,10 @@ int launch_wide(const PrefillArgs &a, int wgs_per_head, int n_waves, hipStream_t
   return LMH_OK;
 }
 
-template <typename MT, int D>
+// V16 (bf16 only): the launches of one key group hand V to the matrix cores as fp16 (base_policy above).
+template <typename MT, int D, bool V16>
 int launch_for_d(const PrefillArgs &a, hipStream_t stream) {
+  static_assert(!V16 || MT::kSplitP, "V16 is a form of the bf16 kernels");
   // With fewer than two 128-row workgroups per CU the launch is bound by how long one workgroup
   // takes to walk its keys, not by the matrix pipes: split the keys of a tile between wave pairs.
   // Measured on 256 CUs: at exactly two per CU the split still wins for causal launches (41.8 vs
@@ -1284,7 +1284,7 @@ int launch_for_d(const PrefillArgs &a, hipStream_t stream) {
       int wgs_per_head, n_waves;
       if (wide_plan(a, n_cus, &wgs_per_head, &n_waves)) return launch_wide<MT, D>(a, wgs_per_head, n_waves, stream);
     }
-    return launch_split<MT, D, 2, 4>(a, stream);
+    return launch_split<MT, V16, D, 2, 4>(a, stream);
   }
   // Large launches: 256-row workgroups of eight waves. Measured against the 128-row ones at D = 96, fp16:
   // non-causal 512 / 768 / 1024 / 1536 / 2048 workgroups +3 / +2 / +2 / +6 / +5 %, causal 512 -7 %
@@ -1294,7 +1294,7 @@ int launch_for_d(const PrefillArgs &a, hipStream_t stream) {
   // causal 256 / 384 -8 / -5 %, 512 / 1024 / 2048 +8 / +3 / +4 %; bf16 (V rewritten as fp16) 512 workgroups causal
   // +8 %, without a mask +5 %, 2048 causal +5 %.
   const int64_t wgs256 = (int64_t)((a.B * a.Hq + 7) / 8) * 8 * ((a.Sq + 255) / 256);
-  if (a.Sq <= 128) return launch_split<MT, D, 1, 4>(a, stream);  // nothing for waves 4-7 to own
+  if (a.Sq <= 128) return launch_split<MT, V16, D, 1, 4>(a, stream);  // nothing for waves 4-7 to own
   if constexpr (D <= 96) {
     // Causal launches of 1.5 to 3 rounds of one 256-row workgroup per CU (the Phi-3 prompt, 32 heads x 4096 rows,
     // is exactly two): the workgroups turn over heaviest first, so every CU ends up with about the same number
@@ -1307,24 +1307,40 @@ int launch_for_d(const PrefillArgs &a, hipStream_t stream) {
     // rounds there are: B=4 H=32 S=4096 causal 583 -> 507 us, without a mask 946 -> 892 us. At D = 64 it takes this form for
     // causal launches of 1.5 to 3 rounds (the rewrite is shared by eight waves instead of four: B=1 H=32 S=4096 100.1 -> 96.5
     // us, H=64 S=2048 60.3 -> 58.6); from three rounds on and without a mask two workgroups per CU are 6-10 % ahead there.
-    if constexpr (D == 96 || MT::kSplitP)
-      if ((D == 96 || a.causal) && ((D == 96 && MT::kSplitP) || wgs256 < 3 * n_cus) &&
+    if constexpr (D == 96 || V16)
+      if ((D == 96 || a.causal) && ((D == 96 && V16) || wgs256 < 3 * n_cus) &&
           (a.causal ? 2 * wgs256 >= 3 * n_cus : wgs256 >= 2 * n_cus))
-        return launch_split<MT, D, 1, 8, 2>(a, stream);
-    if (wgs256 >= (a.causal ? 4 * n_cus : 2 * n_cus)) return launch_split<MT, D, 1, 8>(a, stream);
-  } else {
-    if (wgs256 >= (a.causal ? 2 * n_cus : n_cus)) return launch_split<MT, D, 1, 8>(a, stream);
+        return launch_split<MT, V16, D, 1, 8, 2>(a, stream);
+    if constexpr (!(D == 96 && V16))  // (with V16, D = 96 never gets here with that many workgroups)
+      if (wgs256 >= (a.causal ? 4 * n_cus : 2 * n_cus)) return launch_split<MT, V16, D, 1, 8>(a, stream);
+  } else if constexpr (!MT::kSplitP || V16) {  // (bf16 with head + remainder weights: 0 / -2 %, stays on 128 rows)
+    if (wgs256 >= (a.causal ? 2 * n_cus : n_cus)) return launch_split<MT, V16, D, 1, 8>(a, stream);
   }
-  return launch_split<MT, D, 1, 4>(a, stream);
+  return launch_split<MT, V16, D, 1, 4>(a, stream);
 }
 
 template <typename MT>
 int launch_for_type(const PrefillArgs &a, hipStream_t stream) {
+  if (a.D > 128) return fail(LMH_E_UNSUPPORTED, "MFMA flash attention: head dim %d not tiled", a.D);
+#ifndef LMH_BF16_SPLIT_P
+  if constexpr (MT::kSplitP) {
+    // bf16: V as fp16 pays from about 512 keys per query row on. Its prologue (the first V tile through registers before
+    // the first barrier) and one workgroup per CU cost short rows more than the second MFMA per fragment does: 512 heads,
+    // fp16 rewrite against head + remainder, causal S=128 +15 ... +35 %, S=256 +7 ... +44 %, S=512 -3 ... +18 %, S=1024
+    // -13 ... 0 %; without a mask S=128 0 ... +30 %, S=256 -7 ... -1 %, S=512 -13 ... +5 %, S=1024 -5 ... -19 %. (The
+    // D = 96 tiling, one workgroup per CU in this form, is the one that ties or loses at 512 keys per row: 1024 there.)
+    const int64_t keys_per_row = a.causal ? (a.Sq < a.Sk ? a.Sq : a.Sk) / 2 : a.Sk;
+    if (keys_per_row >= (a.D > 64 && a.D <= 96 ? 1024 : 512)) {
+      if (a.D <= 64) return launch_for_d<MT, 64, true>(a, stream);
+      if (a.D <= 96) return launch_for_d<MT, 96, true>(a, stream);
+      return launch_for_d<MT, 128, true>(a, stream);
+    }
+  }
+#endif
   // the smallest tiling that holds the head dim; the padding costs its share of the MFMAs
-  if (a.D <= 64) return launch_for_d<MT, 64>(a, stream);
-  if (a.D <= 96) return launch_for_d<MT, 96>(a, stream);
-  if (a.D <= 128) return launch_for_d<MT, 128>(a, stream);
-  return fail(LMH_E_UNSUPPORTED, "MFMA flash attention: head dim %d not tiled", a.D);
+  if (a.D <= 64) return launch_for_d<MT, 64, false>(a, stream);
+  if (a.D <= 96) return launch_for_d<MT, 96, false>(a, stream);
+  return launch_for_d<MT, 128, false>(a, stream);
 }
 
 }  // namespace

@@ -36,7 +36,7 @@ def setup(lm, oracle, shape, seed):
     B, H, S, D, causal = shape
     plan = lm.flash_attention_plan((B, H, S, D), (B, H, S, D), "bf16", causal)
     print(plan, flush=True)
-    assert "prefill_mfma_kernel<bf16" in plan and "key groups=1" in plan, plan
+    assert "prefill_mfma_kernel<bf16" in plan and "key groups=1" in plan and plan.endswith("V as fp16"), plan
     q, k, v = inputs(oracle, (B, H, S, D), (B, H, S, D), "bf16", seed, 0.8)
     heads = np.array([0, H // 2, H - 1])
     return q, k, v, heads

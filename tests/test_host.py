@@ -178,7 +178,16 @@ def test_kernel_plan_of_the_benchmark_configurations(lm):
     assert plan((1, 32, 4096, 96), (1, 32, 4096, 96), "bf16", True).startswith(
         "prefill_mfma_kernel<bf16, D=96, causal, key groups=1, waves=8, waves per SIMD=2> workgroups=512")
     # ... in bf16 however many rounds there are (fp16 goes to two workgroups per CU from three rounds on)
-    assert "waves=8, waves per SIMD=2> workgroups=2048" in plan((4, 32, 4096, 96), (4, 32, 4096, 96), "bf16", True)
+    assert "waves=8, waves per SIMD=2> workgroups=2048, V as fp16" in plan((4, 32, 4096, 96), (4, 32, 4096, 96), "bf16", True)
+    # bf16 hands V to the matrix cores as fp16 from about 512 keys per query row on (1024 at the D = 96 tiling), and only in
+    # the launches of one key group
+    assert plan((1, 32, 4096, 96), (1, 32, 4096, 96), "bf16", True).endswith("V as fp16")
+    assert plan((16, 32, 1024, 128), (16, 32, 1024, 128), "bf16", True).endswith("V as fp16")
+    assert not plan((16, 32, 1024, 96), (16, 32, 1024, 96), "bf16", True).endswith("V as fp16")
+    assert not plan((16, 32, 512, 128), (16, 32, 512, 128), "bf16", True).endswith("V as fp16")
+    assert plan((16, 32, 512, 128), (16, 32, 512, 128), "bf16", False).endswith("V as fp16")
+    assert "key groups=2" in plan((1, 8, 1024, 64), (1, 8, 1024, 64), "bf16", True)
+    assert not plan((1, 8, 1024, 64), (1, 8, 1024, 64), "bf16", True).endswith("V as fp16")
     assert "waves=8, waves per SIMD=4> workgroups=2048" in plan((4, 32, 4096, 96), (4, 32, 4096, 96), "f16", True)
     assert plan((1, 40, 4096, 96), (1, 40, 4096, 96), "f16", True).startswith(
         "prefill_mfma_kernel<f16, D=96, causal, key groups=1, waves=8, waves per SIMD=2> workgroups=640")
