@@ -42,7 +42,12 @@ extern "C" {
 /* out_f32 (a field of both parameter blocks): 0 writes the result in the input element type,
  * 1 writes fp32. A bf16 result carries a rounding error of up to 2^-8 of its magnitude on its
  * own, more than the 2e-3 parity budget of the half-precision configurations, so bf16 callers
- * that need that budget ask for fp32. */
+ * that need that budget ask for fp32.
+ * The softmax weights reach the matrix cores with 11 (fp16) or 16 (bf16, head + remainder) significant bits.
+ * bf16 flash attention with long rows (from about 512 keys per query row on; lmh_flash_attn_plan ends in
+ * "V as fp16") rounds the weights to 11 bits and hands V over as fp16, rewritten exactly tile by tile relative to
+ * the largest finite |v| staged so far for the row's 256-row tile (causally hidden keys of that tile included):
+ * values more than 2^29 below it count as zero; infinities and NaNs stay what they are. */
 
 /* which KV head a query head reads.
  * INTERLEAVED: hq % Hkv — what the reference's repeat_kv produces, because its
