@@ -46,7 +46,8 @@ extern "C" {
  * The softmax weights reach the matrix cores with 11 (fp16) or 16 (bf16, head + remainder) significant bits.
  * bf16 flash attention with long rows (from about 512 keys per query row on; lmh_flash_attn_plan ends in
  * "V as fp16") rounds the weights to 11 bits and hands V over as fp16, rewritten exactly tile by tile relative to
- * the largest finite |v| staged so far for the row's 256-row tile (causally hidden keys of that tile included):
+ * the largest finite |v| staged so far by the row's workgroup (128 or 256 query rows; the keys the causal mask hides from
+ * the row but not from the workgroup's last row included):
  * values more than 2^29 below it count as zero; infinities and NaNs stay what they are. */
 
 /* which KV head a query head reads.
