@@ -9,6 +9,7 @@ import pytest
 
 from conftest import TOL, rel_err
 from test_parity_gpu import inputs, run_flash
+from test_random_shapes_gpu import poison_tail
 
 pytestmark = pytest.mark.gpu
 
@@ -135,3 +136,56 @@ def test_zero_values_give_zeros(lm, hip, oracle, shape):
     assert np.all(got[:, 1:] == 0.0)
     want = oracle.flash_attn(q[:, :1], k[:, :1], v[:, :1], causal=causal, nthreads=NT)
     assert rel_err(got[:, :1], want) <= TOL["bf16"]
+
+
+def test_long_row_random_shapes(lm, hip, oracle):
+    """Shapes drawn until at least 16 of them reach the fp16-V form (the plan query says which do) and all three tilings
+    have been seen with and without the mask: head dims on all three tilings,
+    GQA groups and head maps, ragged key counts with a NaN tail, with and without the mask, V scaled by a random power of
+    two per (batch, KV head), bf16 and fp32 outputs."""
+    rng = np.random.default_rng(99500)
+    done, tried, reached = 0, 0, set()
+    while (done < 16 or len(reached) < 6) and done < 40 and tried < 4000:
+        tried += 1
+        D = int(rng.choice([16, 40, 64, 72, 80, 96, 96, 104, 128]))
+        G = int(rng.choice([1, 1, 2, 4]))
+        Hkv = int(rng.integers(1, 17))
+        Hq = Hkv * G
+        B = int(rng.integers(1, 5))
+        causal = bool(rng.integers(2))
+        Sq = int(rng.integers(129, 3001))
+        Sk = Sq if causal and rng.integers(2) else int(rng.integers(600, 3001))
+        if B * Hq * Sq * Sk * D > 4e11:
+            continue
+        plan = lm.flash_attention_plan((B, Hq, Sq, D), (B, Hkv, Sk, D), "bf16", causal)
+        if not plan.endswith("V as fp16"):
+            continue
+        head_map = int(rng.integers(2))
+        lens = None if rng.integers(2) == 0 else rng.integers(0, Sk + 1, size=B).astype(np.int32)
+        out_f32 = bool(rng.integers(2))
+        what = "case %d: B=%d Hq=%d Hkv=%d Sq=%d Sk=%d D=%d causal=%s head_map=%d kv_len=%s out_f32=%s -> %s" % (
+            done, B, Hq, Hkv, Sq, Sk, D, causal, head_map, None if lens is None else lens.tolist(), out_f32, plan)
+        print(what, flush=True)
+        q, k, v = inputs(oracle, (B, Hq, Sq, D), (B, Hkv, Sk, D), "bf16", 99600 + 3 * done, float(rng.choice([0.5, 1.0, 1.5])))
+        v = v * power_of_two(rng.integers(-60, 61, size=(B, Hkv)))[:, :, None, None]
+        kp, vp = (k, v) if lens is None else poison_tail(k, v, lens)
+        got = run_flash(lm, hip, q, kp, vp, "bf16", causal, head_map=head_map, kv_len=lens, out_dtype="f32" if out_f32 else None)
+        hq = np.unique(rng.integers(0, Hq, size=min(Hq, 3)))
+        kv_of = hq if Hq == Hkv else (hq // G if head_map == 1 else hq % Hkv)
+        want_len = None if lens is None else np.maximum(lens, 1)
+        want = oracle.flash_attn(q[:, hq], k[:, kv_of], v[:, kv_of], causal=causal, kv_len=want_len, nthreads=NT)
+        keep = np.arange(B) if lens is None else np.nonzero(lens > 0)[0]
+        assert np.isfinite(got).all(), what
+        # every (batch, head) against its own scale: the heads' values differ by up to 2^120
+        tol = TOL["bf16"] if out_f32 else 2.0 ** -8 + TOL["bf16"]  # (a bf16 result is rounded once more)
+        for b in keep:
+            for i, h in enumerate(hq):
+                err = rel_err(got[b, h], want[b, i])
+                assert err <= tol, "%s: batch %d head %d rel err %.3g" % (what, b, h, err)
+        if lens is not None:
+            for b in np.nonzero(lens == 0)[0]:
+                assert np.all(got[b] == 0), what
+        reached.add((plan.split("<")[1].split(",")[1].strip(), causal))
+        done += 1
+    print("cases:", done, "tilings and masks covered:", sorted(reached), flush=True)
+    assert len(reached) == 6, reached
