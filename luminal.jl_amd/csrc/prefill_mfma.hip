@@ -573,9 +573,14 @@ __global__ __launch_bounds__(64 * NW, WPS) void prefill_mfma_kernel(PrefillArgs 
 // Measured against those workgroups (B=4 H=20 Sq=448 D=64 fp16, five row blocks x three key groups): 1500 keys 28.7 ->
 // 25.3 us, 3000 keys 51.4 -> 43.7, 750 keys 17.0 -> 16.4, 256 keys 9.2 -> 10.5 (one prologue per CU instead of three
 // that overlap). Taller tiles (two blocks per wave and tile) and a third tile buffer were 1 % and 7 % slower.
+// `mixed`: with five or seven row blocks no equal number of key groups fills four SIMDs evenly (5 x 3 = 15 waves: 4, 4, 4, 3).
+// Then the workgroup runs 16 waves on tiles of 128 keys, some row blocks split between two waves (two 32-key blocks of a
+// tile each) and the others between four, so that every SIMD walks R / 4 of a block's keys: 1.25 against 1.33 at R = 5
+// (B=4 H=20 Sq=448 Sk=1500 D=64: 23.85 -> 23.55 us; D=96 with 3000 keys 54.9 -> 53.5), 1.75 against 2 at R = 7 (Sq=672:
+// 37.4 us on the 64-row workgroups -> 32.7 us here).
 constexpr int kWideMaxKeyGroups = 6;  // tiles of up to 192 keys: two buffers of them fit the LDS at D = 96
 template <typename MT, int D>
-__global__ __launch_bounds__(1024, 4) void prefill_mfma_wide_kernel(PrefillArgs a, int wgs_per_head, int n_bh_groups) {
+__global__ __launch_bounds__(1024, 4) void prefill_mfma_wide_kernel(PrefillArgs a, int wgs_per_head, int n_bh_groups, int mixed) {
   using vec8 = typename MT::vec8;
   constexpr int KS = D / 16, DB = D / 32;
   constexpr int LDK = D + kPadK, LDV = D + pad_v<D>();
@@ -606,15 +611,35 @@ __global__ __launch_bounds__(1024, 4) void prefill_mfma_wide_kernel(PrefillArgs 
   if (R == 0) return;
   const int block0 = j_wg * base + min(j_wg, extra);
   const int NW = blockDim.x >> 6;
-  // the host launches R_max x KG waves; a workgroup with fewer row blocks may use more key groups or leave waves idle
-  const int KG = min(min(NW / R, KG_MAX), kWideMaxSlots / R + 1);
-  const int BT = 32 * KG;
-
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = tid >> 6;
   const int n = lane & 31, g = lane >> 5;
-  const int r = wave % R, kg = wave / R;
-  const bool active = kg < KG;  // waves beyond R x KG only help to stage
+  // Which row block r of the workgroup the wave takes, as key group kg of that block's n_groups, and which 32-key blocks of
+  // every staged tile: blocks kb0 .. kb0 + nkb - 1. The partial results of groups 1 .. n_groups - 1 go to LDS slots
+  // slot0 + (kg - 1) * slot_step; group 0 folds them.
+  int BT, r, kg, n_groups, kb0, nkb, slot0, slot_step;
+  if (!mixed) {
+    // the host launches R_max x KG waves; a workgroup with fewer row blocks may use more key groups or leave waves idle
+    const int KG = min(min(NW / R, KG_MAX), kWideMaxSlots / R + 1);
+    BT = 32 * KG;
+    r = wave % R, kg = wave / R, n_groups = KG;
+    kb0 = kg, nkb = 1, slot0 = r, slot_step = R;
+  } else {
+    // 16 waves on tiles of 128 keys: `heavy` row blocks are split between two waves (two 32-key blocks of a tile each), the
+    // others between four (one block each). The heavy waves come first, so that dealt round-robin every SIMD gets the same
+    // number of 32-key blocks per tile: R of them (R = 5: 2 + 1 + 1 + 1 against 4 x 1 per 96 keys with three key groups).
+    BT = 128;
+    const int heavy = max(2 * R - 8, 0), light = R - heavy;
+    if (wave < 2 * heavy) {
+      r = wave % heavy, kg = wave / heavy, n_groups = 2;
+      kb0 = 2 * kg, nkb = 2, slot0 = r, slot_step = 0;
+    } else {
+      const int l = wave - 2 * heavy;
+      r = heavy + l % light, kg = l / light, n_groups = 4;
+      kb0 = kg, nkb = 1, slot0 = heavy + 3 * (l % light), slot_step = 1;
+    }
+  }
+  const bool active = kg < n_groups;  // waves beyond the groups only help to stage
   const int qi = (block0 + r) * 32 + n;
 
   int n_keys = a.kv_len ? a.kv_len[b] : a.Sk;
@@ -692,9 +717,9 @@ __global__ __launch_bounds__(1024, 4) void prefill_mfma_wide_kernel(PrefillArgs 
         load_block(v_desc, v_lds0 + buf * (V_BUF * 2) + j * (nw_u * 1024), v_voff[j], kt * v_tile_bytes);
   };
 
-  const int k_frag_off = (kg * 32 + n) * LDK + 8 * g;
+  const int k_frag_off = (kb0 * 32 + n) * LDK + 8 * g;  // + 32 LDK per further block
   const int i16 = lane & 15;
-  const int v_frag_off = (kg * 32 + 4 * g + (i16 >> 2)) * LDV + 16 * ((lane >> 4) & 1) + 4 * (i16 & 3);
+  const int v_frag_off = (kb0 * 32 + 4 * g + (i16 >> 2)) * LDV + 16 * ((lane >> 4) & 1) + 4 * (i16 & 3);
 
   if (n_kv_tiles > 0) load_tile(0, 0);
   if (a.q_rope) rotate_q_fragments<MT, D>(qreg, a, b, qi, g, reinterpret_cast<float *>(&lds[K_BUF]));
@@ -705,10 +730,11 @@ __global__ __launch_bounds__(1024, 4) void prefill_mfma_wide_kernel(PrefillArgs 
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wave's blocks of tile kt are in LDS
     __syncthreads();  // ... and everyone's; tile kt-1 has been consumed, its buffer is free
     if (kt + 1 < n_kv_tiles) load_tile(kt + 1, (kt + 1) & 1);
-    const int k0 = kt * BT + kg * 32;  // this wave's 32 keys of the tile
-    if (!active || k0 >= n_keys) continue;
-    const uint16_t *Ks = &lds[(kt & 1) * K_BUF];
-    const uint16_t *Vs = &lds[NBUF * K_BUF + (kt & 1) * V_BUF];
+    for (int j = 0; j < nkb; j++) {
+    const int k0 = kt * BT + (kb0 + j) * 32;  // this wave's 32 keys of the tile (nkb = 2: the second 32 follow)
+    if (!active || k0 >= n_keys) break;
+    const uint16_t *Ks = &lds[(kt & 1) * K_BUF + j * 32 * LDK];
+    const uint16_t *Vs = &lds[NBUF * K_BUF + (kt & 1) * V_BUF + j * 32 * LDV];
 
     floatx16_t sacc;
 #pragma unroll
@@ -762,13 +788,14 @@ __global__ __launch_bounds__(1024, 4) void prefill_mfma_wide_kernel(PrefillArgs 
         if (MT::kSplitP) oacc[db] = MT::mfma(__builtin_bit_cast(vec8, v8), pf_lo[t], oacc[db]);
       }
     }
+    }
   }
 
   // ---- fold the key groups of a row block: groups 1 .. KG-1 leave (m, l, O) in LDS, group 0 takes them in order ----
   float *xch = reinterpret_cast<float *>(&lds[0]) + lane;  // slot s at xch + s * NF * 64, [NF][64 lanes]
   __syncthreads();  // every wave has read its last tile
   if (active && kg > 0) {
-    float *slot = xch + ((kg - 1) * R + r) * (NF * 64);
+    float *slot = xch + (slot0 + (kg - 1) * slot_step) * (NF * 64);
     slot[0] = m_i;
     slot[64] = l_i;
 #pragma unroll
@@ -778,8 +805,8 @@ __global__ __launch_bounds__(1024, 4) void prefill_mfma_wide_kernel(PrefillArgs 
   }
   __syncthreads();
   if (!active || kg > 0) return;
-  for (int k2 = 1; k2 < KG; k2++) {
-    const float *slot = xch + ((k2 - 1) * R + r) * (NF * 64);
+  for (int k2 = 1; k2 < n_groups; k2++) {
+    const float *slot = xch + (slot0 + (k2 - 1) * slot_step) * (NF * 64);
     const float m1 = slot[0], l1 = slot[64];
     const float m_new = fmaxf(m_i, m1);
     // a group that saw no key has m = -inf, l = 0, O = 0
@@ -1210,7 +1237,7 @@ int launch_split(const PrefillArgs &a, hipStream_t stream) {
 // of the busiest CU walks, the quantity the launch time follows when the chip is not full. Measured (fp16, 1500 keys,
 // wide against 64-row workgroups): load 1.33 vs 1.5 -12 % (D = 64), -14 % (D = 96); 0.75 vs 1.0 -7 ... -12 %; equal loads
 // +-2 %, and +7 % at 1024 keys; under about 500 keys the single prologue per CU costs more than the balance wins.
-inline bool wide_plan(const PrefillArgs &a, int n_cus, int *wgs_per_head, int *n_waves) {
+inline bool wide_plan(const PrefillArgs &a, int n_cus, int *wgs_per_head, int *n_waves, int *mixed) {
   const int heads = a.B * a.Hq, heads8 = (heads + 7) / 8 * 8;
   const int n_blocks = (a.Sq + 31) / 32;
   if (a.causal || heads8 > n_cus || n_blocks < 2 || a.Sk < 640) return false;
@@ -1224,24 +1251,28 @@ inline bool wide_plan(const PrefillArgs &a, int n_cus, int *wgs_per_head, int *n
     const double load = (double)((r_max * kg + 3) / 4) / kg;
     if (load <= best) best = load, best_kg = kg;  // on a tie, more waves
   }
-  if (!best_kg) return false;
+  // two waves for some row blocks and four for the others (16 waves, tiles of 128 keys): every SIMD walks r_max / 4 of a
+  // block's keys. Ahead of the equal key groups at five and seven row blocks (1.25 against 1.33, 1.75 against 2).
+  *mixed = 0;
+  if (r_max >= 5 && r_max <= 8 && r_max / 4.0 < best - 1e-9) best = r_max / 4.0, *mixed = 1;
+  if (!best_kg && !*mixed) return false;
   // the equal 64-row workgroups, wave pairs splitting the keys: up to three resident on a CU, half a block's keys a wave
   const int64_t n64 = (int64_t)heads8 * ((a.Sq + 63) / 64);
   const double load_now = 0.5 * (double)((n64 + n_cus - 1) / n_cus);
   if (best > LMH_WIDE_MARGIN * load_now) return false;
   *wgs_per_head = w;
-  *n_waves = r_max * best_kg;
+  *n_waves = *mixed ? 16 : r_max * best_kg;
   return true;
 }
 
 template <typename MT, int D>
-int launch_wide(const PrefillArgs &a, int wgs_per_head, int n_waves, hipStream_t stream) {
+int launch_wide(const PrefillArgs &a, int wgs_per_head, int n_waves, int mixed, hipStream_t stream) {
   const int n_bh_groups = (a.B * a.Hq + 7) / 8;
   dim3 grid(8 * n_bh_groups * wgs_per_head), block(64 * n_waves);
-  if (plan_only("prefill_mfma_wide_kernel<%s, D=%d> workgroups per head=%d, waves=%d, workgroups=%u", MT::kName, D, wgs_per_head,
-                n_waves, grid.x))
+  if (plan_only("prefill_mfma_wide_kernel<%s, D=%d> workgroups per head=%d, waves=%d, workgroups=%u%s", MT::kName, D, wgs_per_head,
+                n_waves, grid.x, mixed ? ", two and four key groups" : ""))
     return LMH_OK;
-  hipLaunchKernelGGL((prefill_mfma_wide_kernel<MT, D>), grid, block, 0, stream, a, wgs_per_head, n_bh_groups);
+  hipLaunchKernelGGL((prefill_mfma_wide_kernel<MT, D>), grid, block, 0, stream, a, wgs_per_head, n_bh_groups, mixed);
   LMH_HIP_TRY(hipGetLastError());
   return LMH_OK;
 }
@@ -1281,8 +1312,8 @@ int launch_for_d(const PrefillArgs &a, hipStream_t stream) {
   const int64_t limit = a.causal ? 2 * n_cus : 2 * n_cus - 1;
   if (wgs <= limit && a.Sk >= 4 * BN) {
     if constexpr (D <= 96) {
-      int wgs_per_head, n_waves;
-      if (wide_plan(a, n_cus, &wgs_per_head, &n_waves)) return launch_wide<MT, D>(a, wgs_per_head, n_waves, stream);
+      int wgs_per_head, n_waves, mixed;
+      if (wide_plan(a, n_cus, &wgs_per_head, &n_waves, &mixed)) return launch_wide<MT, D>(a, wgs_per_head, n_waves, mixed, stream);
     }
     return launch_split<MT, V16, D, 2, 4>(a, stream);
   }

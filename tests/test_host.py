@@ -191,9 +191,13 @@ def test_kernel_plan_of_the_benchmark_configurations(lm):
     assert "waves=8, waves per SIMD=4> workgroups=2048" in plan((4, 32, 4096, 96), (4, 32, 4096, 96), "f16", True)
     assert plan((1, 40, 4096, 96), (1, 40, 4096, 96), "f16", True).startswith(
         "prefill_mfma_kernel<f16, D=96, causal, key groups=1, waves=8, waves per SIMD=2> workgroups=640")
-    # C3: 80 heads x 14 row blocks on 256 CUs -> three workgroups per head of five row blocks x three key groups
+    # C3: 80 heads x 14 row blocks on 256 CUs -> three workgroups per head of five row blocks; two of the five are split
+    # between two waves and three between four (16 waves, every SIMD walks 5/4 of a block's keys)
     assert plan((4, 20, 448, 64), (4, 20, 1500, 64), "f16", False) == \
-        "prefill_mfma_wide_kernel<f16, D=64> workgroups per head=3, waves=15, workgroups=240"
+        "prefill_mfma_wide_kernel<f16, D=64> workgroups per head=3, waves=16, workgroups=240, two and four key groups"
+    # seven row blocks per workgroup likewise (7/4 against 2 with two key groups each); two or three row blocks: equal groups
+    assert plan((4, 20, 672, 64), (4, 20, 1500, 64), "f16", False).endswith("waves=16, workgroups=240, two and four key groups")
+    assert plan((2, 20, 448, 64), (2, 20, 1500, 64), "f16", False).endswith("workgroups per head=6, waves=12, workgroups=240")
     # the same heads against few keys, or causal: 64-row workgroups whose wave pairs split the keys
     assert "key groups=2, waves=4" in plan((4, 20, 448, 64), (4, 20, 512, 64), "f16", False)
     assert "key groups=2, waves=4" in plan((4, 20, 448, 64), (4, 20, 1500, 64), "f16", True)
