@@ -281,11 +281,13 @@ WIDE_CASES = [
     ("bf16", "f32", 2, 20, 10, 430, 777, 64, 0, None),       # 6 workgroups per head: 3, 3, 2, 2, 2, 2 row blocks, the last one ragged
     ("f16", "f32", 16, 8, 8, 190, 1000, 96, 0, [1000, 0, 1, 31, 32, 33, 95, 96, 97, 640, 999, 128, 129, 500, 767, 768]),
     ("bf16", "bf16", 1, 256, 256, 96, 700, 80, 0, None),     # one workgroup per head, head dim padded to 96
-    ("f16", "f16", 4, 20, 20, 448, 1500, 64, 0, [1500, 1499, 97, 0]),  # 5 row blocks x 3 key groups = 15 waves, one SIMD a wave short
+    ("f16", "f16", 4, 20, 20, 448, 1500, 64, 0, [1500, 1499, 97, 0]),  # 5 row blocks on 16 waves: two split two ways, three split four ways
     ("f16", "f32", 2, 24, 6, 448, 900, 64, 1, [900, 650]),   # blocked GQA map; 3, 3, 3, 3, 2 row blocks
     ("bf16", "f32", 4, 20, 4, 448, 1500, 96, 0, None),
-    ("f16", "f32", 2, 32, 32, 576, 1200, 64, 0, None),       # 5, 5, 4, 4 row blocks on 15 waves: three waves idle where there are 4
+    ("f16", "f32", 2, 32, 32, 576, 1200, 64, 0, None),       # 5, 5, 4, 4 row blocks: four key groups each where there are 4
     ("f16", "f16", 1, 40, 8, 440, 800, 40, 0, [799]),        # head dim 40 on the D = 64 tiling
+    ("f16", "f32", 4, 20, 20, 672, 1500, 64, 0, [1500, 1499, 97, 0]),  # 7 row blocks: six split two ways, one four ways
+    ("bf16", "f32", 2, 40, 10, 650, 900, 96, 1, [900, 129]),  # 7, 7, 7 row blocks, the last ragged; 128-key tiles end inside the keys
 ]
 
 
