@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the attention hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--only all|prefill|decode|other|c1|nomask|bf16|c3|c4|ops|step|copy|ceiling|grid]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--only all|prefill|decode|other|c1|nomask|bf16|c3|c4|ops|step|copy|ceiling|grid|shapes]
 
 A step is one pass of the hot path over one batch of synthetic input, inputs resident in HBM:
   prefill leg (the headline `value`): causal flash attention, Phi-3-mini shape
@@ -405,6 +405,22 @@ def bf16_leg(lm, dev, res, check):
             raise SystemExit("parity check failed on %s: rel err %.3g > 2e-3" % (name, err))
 
 
+def shapes_leg(lm, dev, spec):
+    """Any flash-attention launches by shape (--only shapes --shapes B,Hq,Hkv,Sq,Sk,D,dtype,causal|full[;...]): µs per
+    launch, TFLOP/s and the kernel reached, for comparing two builds of the library (the measurement switches of the
+    kernels) on shapes that are not contract configurations."""
+    res = {}
+    for item in spec.split(";"):
+        f = item.split(",")
+        B, Hq, Hkv, Sq, Sk, D = (int(x) for x in f[:6])
+        dtype, causal = f[6], f[7] == "causal"
+        flops = 4.0 * B * Hq * D * (Sq * (Sq + 1) / 2 if causal and Sq == Sk else Sq * Sk)
+        steps = 40 if flops < 4e11 else 12
+        flash_config(lm, dev, res, item, B, Hq, Hkv, Sq, Sk, D, dtype, causal, flops, 7000, mul=0.5, steps=steps, peak=PEAK_FP16_TFLOPS)
+        res[item].pop("launch_us_one_by_one", None)
+    return res
+
+
 def c3_leg(lm, dev, res, check):
     flash_config(lm, dev, res, "C3 cross fp16 B=4 H=20 Sq=448 Sk=1500 D=64", 4, 20, 20, 448, 1500, 64, "f16", False,
                  4.0 * 4 * 20 * 448 * 1500 * 64, 3000, tol=2e-3 if check else None, steps=40, peak=PEAK_FP16_TFLOPS)
@@ -723,9 +739,11 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--only", choices=["all", "prefill", "decode", "other", "c1", "nomask", "bf16", "c3", "c4", "ops", "step", "copy", "ceiling", "grid"], default="all")
+    ap.add_argument("--only", choices=["all", "prefill", "decode", "other", "c1", "nomask", "bf16", "c3", "c4", "ops", "step", "copy", "ceiling", "grid", "shapes"], default="all")
     ap.add_argument("--decode-splits", type=int, default=0, help="KV splits for the decode leg (0 = library heuristic)")
     ap.add_argument("--cpu-seconds", type=float, default=15.0, help="CPU-baseline budget per leg; 0 disables it")
+    ap.add_argument("--shapes", default="1,32,32,4096,4096,96,bf16,causal",
+                    help="for --only shapes: B,Hq,Hkv,Sq,Sk,D,dtype,causal|full, several separated by ';'")
     ap.add_argument("--no-zero-operands", action="store_true",
                     help="leave out the second timing of the prefill / nomask launch on all-zero tensors (for counter and "
                          "kernel-trace runs, whose per-kernel averages should cover the workload's launches only)")
@@ -755,6 +773,10 @@ def main():
         return
     if args.only == "ceiling":
         line["ceiling"] = ceiling_leg(lm, dev)
+        print(json.dumps(line))
+        return
+    if args.only == "shapes":
+        line["shapes"] = shapes_leg(lm, dev, args.shapes)
         print(json.dumps(line))
         return
     if args.only == "grid":

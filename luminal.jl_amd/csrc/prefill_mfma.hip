@@ -30,9 +30,9 @@
 #include "rope.hpp"
 
 #if (defined(LMH_FOLD_SCALE) || defined(LMH_ONLY_XCDS) || defined(LMH_WIDE_MARGIN) || defined(LMH_W64_KERNEL) || defined(LMH_NO_PAIR_KERNEL) || \
-     defined(LMH_BF16_SPLIT_P)) && \
+     defined(LMH_BF16_SPLIT_P) || defined(LMH_NO_MIXED_KEY_GROUPS)) && \
     !defined(LMH_MEASUREMENT_BUILD)
-#error "LMH_FOLD_SCALE / LMH_ONLY_XCDS / LMH_WIDE_MARGIN / LMH_W64_KERNEL / LMH_NO_PAIR_KERNEL / LMH_BF16_SPLIT_P are experiment switches: they need -DLMH_MEASUREMENT_BUILD, which marks the library"
+#error "LMH_FOLD_SCALE / LMH_ONLY_XCDS / LMH_WIDE_MARGIN / LMH_W64_KERNEL / LMH_NO_PAIR_KERNEL / LMH_BF16_SPLIT_P / LMH_NO_MIXED_KEY_GROUPS are experiment switches: they need -DLMH_MEASUREMENT_BUILD, which marks the library"
 #endif
 
 #ifndef LMH_WIDE_MARGIN
@@ -1254,7 +1254,9 @@ inline bool wide_plan(const PrefillArgs &a, int n_cus, int *wgs_per_head, int *n
   // two waves for some row blocks and four for the others (16 waves, tiles of 128 keys): every SIMD walks r_max / 4 of a
   // block's keys. Ahead of the equal key groups at five and seven row blocks (1.25 against 1.33, 1.75 against 2).
   *mixed = 0;
+#ifndef LMH_NO_MIXED_KEY_GROUPS  // (a measurement build can keep equal key groups everywhere, for comparisons)
   if (r_max >= 5 && r_max <= 8 && r_max / 4.0 < best - 1e-9) best = r_max / 4.0, *mixed = 1;
+#endif
   if (!best_kg && !*mixed) return false;
   // the equal 64-row workgroups, wave pairs splitting the keys: up to three resident on a CU, half a block's keys a wave
   const int64_t n64 = (int64_t)heads8 * ((a.Sq + 63) / 64);
