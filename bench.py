@@ -645,7 +645,9 @@ def ceiling_leg(lm, dev):
     mixes = ["MFMA only", "MFMA + 6 vector instr (1 exp)", "MFMA + 6 vector instr (1 exp) + 1 LDS fragment read",
              "MFMA + 6 vector instr (1 exp) + 1 LDS fragment read per 2 MFMAs", "MFMA + 4 vector instr (1 exp) + 1 LDS fragment read",
              "MFMA + 4 vector instr (1 exp) + 1 LDS fragment read per 2 MFMAs",
-             "MFMA + 11 vector instr (the exp as a 6-instruction polynomial) + 1 LDS fragment read"]
+             "MFMA + 11 vector instr (the exp as a 6-instruction polynomial) + 1 LDS fragment read",
+             "MFMA + 6 vector instr (1 exp) + 1 LDS fragment read, accumulators in AGPRs",
+             "MFMA + 4 vector instr (1 exp) + 1 LDS fragment read per 2 MFMAs, accumulators in AGPRs"]
     res["instruction_mix_streams"] = {}
     mix_sink = lm.HipArray((512 * 512,), "f32", dev)
     for mix, label in enumerate(mixes):

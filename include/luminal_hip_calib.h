@@ -48,6 +48,7 @@ int lmh_calib_mfma_xcds(void *sink_dev, const void *operands_dev, size_t operand
  *   mix 2: mix 1 + one 16-byte-per-lane LDS fragment read      mix 3: mix 1 + one such read per two MFMAs
  *   mix 4: 4 vector instructions (1 exp) + one read            mix 5: 4 vector instructions (1 exp) + one read per two
  *   mix 6: 11 vector instructions, none of them exp (the exp of mix 2 as a six-instruction polynomial) + one read
+ *   mix 7: mix 2, mix 8: mix 5, with the MFMA accumulators in accumulation registers (AGPRs) instead of vector registers
  * `sink_dev` receives 512*512 floats, operands as for lmh_calib_mfma; `*flops` (host, optional) the flops of the launch. */
 int lmh_calib_mix(void *sink_dev, const void *operands_dev, size_t operand_bytes, int iters, int mix, int waves_per_simd,
                   double *flops, void *stream);

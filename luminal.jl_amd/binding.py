@@ -357,7 +357,7 @@ def flash_attn_plan(params):
 
 
 def calib_mix(sink, operands, operand_bytes, iters, mix, waves_per_simd=2, stream=None):
-    """Launch the synthetic instruction-mix stream `mix` (0..5) at 2 or 4 waves per SIMD; returns the flops of the launch."""
+    """Launch the synthetic instruction-mix stream `mix` (0..8) at 2 or 4 waves per SIMD; returns the flops of the launch."""
     flops = ctypes.c_double(0.0)
     check_calib(load_calib().lmh_calib_mix(sink, operands, operand_bytes, iters, mix, waves_per_simd, ctypes.byref(flops), stream))
     return flops.value

@@ -84,7 +84,14 @@ __global__ __launch_bounds__(256) void calib_copy_kernel(uint4 *__restrict__ dst
 // feeds the A operand of the next LDS_EVERY MFMAs). Two or four waves per SIMD, operands from caller-supplied values. This
 // is the best case of a kernel with that mix — no barriers, no staging, no dependencies between the MFMA and the
 // vector work — so its rate on the whole chip is the ceiling for an attention kernel of the same mix.
-template <int NV, int NE, int LDS_EVERY>
+// AGPR_ACC = true keeps the MFMA accumulators in accumulation registers (AGPRs) instead of the vector registers the
+// compiler picks for a kernel of this size: does it matter to the vector work beside the MFMAs which file they are in?
+template <bool AGPR_ACC>
+__device__ inline void calib_mfma(calib_floatx16_t &acc, calib_half8_t a, calib_half8_t b) {
+  if constexpr (AGPR_ACC) asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+a"(acc) : "v"(a), "v"(b));
+  else acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, acc, 0, 0, 0);
+}
+template <int NV, int NE, int LDS_EVERY, bool AGPR_ACC = false>
 __global__ __launch_bounds__(512) void calib_mix_kernel(float *__restrict__ sink, const calib_half8_t *__restrict__ operands,
                                                         int n_operands, int iters) {
   __shared__ calib_half8_t lds[4096];
@@ -108,7 +115,7 @@ __global__ __launch_bounds__(512) void calib_mix_kernel(float *__restrict__ sink
 #pragma unroll
     for (int m = 0; m < 8; m++) {
       const int frag = LDS_EVERY > 1 ? (m / LDS_EVERY) * LDS_EVERY : m;
-      acc[m & 3] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[frag & 7], b[m & 3], acc[m & 3], 0, 0, 0);
+      calib_mfma<AGPR_ACC>(acc[m & 3], a[frag & 7], b[m & 3]);
 #pragma unroll
       for (int j = 0; j < NV; j++) {
         if (j < NE) v[j & 7] = __builtin_amdgcn_exp2f(v[j & 7] * 0.001f);
@@ -215,7 +222,9 @@ extern "C" int lmh_calib_mix(void *sink, const void *operands, size_t operand_by
     case 4: hipLaunchKernelGGL((calib_mix_kernel<4, 1, 1>), grid, block, 0, st, snk, ops, n_ops, iters); break;
     case 5: hipLaunchKernelGGL((calib_mix_kernel<4, 1, 2>), grid, block, 0, st, snk, ops, n_ops, iters); break;
     case 6: hipLaunchKernelGGL((calib_mix_kernel<11, 0, 1>), grid, block, 0, st, snk, ops, n_ops, iters); break;
-    default: return fail(LMH_E_UNSUPPORTED, "lmh_calib_mix: mix %d is not one of 0..6", mix);
+    case 7: hipLaunchKernelGGL((calib_mix_kernel<6, 1, 1, true>), grid, block, 0, st, snk, ops, n_ops, iters); break;
+    case 8: hipLaunchKernelGGL((calib_mix_kernel<4, 1, 2, true>), grid, block, 0, st, snk, ops, n_ops, iters); break;
+    default: return fail(LMH_E_UNSUPPORTED, "lmh_calib_mix: mix %d is not one of 0..8", mix);
   }
   LMH_HIP_TRY(hipGetLastError());
   if (flops) *flops = (double)grid.x * 8.0 * iters * 8.0 * (2.0 * 32 * 32 * 16);
