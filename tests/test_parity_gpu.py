@@ -794,13 +794,13 @@ def test_calibration_kernels(lm, hip):
     big = lm.HipArray((512 * 512,), "f32", hip).fill_bytes(0xFF)
     assert lm.binding.calib_mix(big.ptr, ones.ptr, 1 << 13, 3, 0, 4) == 2 * flops  # two workgroups per CU
     assert np.all(big.to_host() == 64 * 16 * 2 * 3 + 8)
-    for mix in (2, 5):  # LDS fragments are ones too, so the matrix part is unchanged; the vector part is bounded
+    for mix in (2, 5, 7, 8):  # LDS fragments are ones too, so the matrix part is unchanged; the vector part is bounded (7, 8: accumulators in AGPRs)
         sink.fill_bytes(0xFF)
         lm.binding.calib_mix(sink.ptr, ones.ptr, 1 << 13, 3, mix)
         got = sink.to_host()
         assert np.all(np.isfinite(got)) and np.all(np.abs(got - 64 * 16 * 2 * 3) < 4096)
     with pytest.raises(lm.LuminalHipError):
-        lm.binding.calib_mix(sink.ptr, ones.ptr, 1 << 13, 3, 7)
+        lm.binding.calib_mix(sink.ptr, ones.ptr, 1 << 13, 3, 9)
     with pytest.raises(lm.LuminalHipError):
         lm.binding.calib_mix(sink.ptr, ones.ptr, 1 << 13, 3, 0, 3)
 
