@@ -63,8 +63,13 @@ __global__ __launch_bounds__(256, 2) void calib_mfma_kernel(float *__restrict__ 
     for (int i = 0; i < 16; i++) acc[c][i] = 0.f;
   for (int it = 0; it < iters; it++) {
 #pragma unroll
-    for (int m = 0; m < kCalibMfmaPerIter; m++)
+    for (int m = 0; m < kCalibMfmaPerIter; m++) {
       acc[m & 3] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[m & 3], b[(m >> 1) & 3], acc[m & 3], 0, 0, 0);
+      // Several waves of a SIMD running MFMAs with nothing in between settle into one of two rates, the full one or two
+      // thirds of it, depending on how far apart they started; one scalar instruction between the MFMAs keeps the full rate.
+      asm volatile("s_nop 0");
+      __builtin_amdgcn_sched_barrier(0);
+    }
   }
   float s = 0.f;
 #pragma unroll
@@ -116,6 +121,10 @@ __global__ __launch_bounds__(512) void calib_mix_kernel(float *__restrict__ sink
     for (int m = 0; m < 8; m++) {
       const int frag = LDS_EVERY > 1 ? (m / LDS_EVERY) * LDS_EVERY : m;
       calib_mfma<AGPR_ACC>(acc[m & 3], a[frag & 7], b[m & 3]);
+      if (NV == 0 && LDS_EVERY == 0) {  // nothing between the MFMAs otherwise: see calib_mfma_kernel
+        asm volatile("s_nop 0");
+        __builtin_amdgcn_sched_barrier(0);
+      }
 #pragma unroll
       for (int j = 0; j < NV; j++) {
         if (j < NE) v[j & 7] = __builtin_amdgcn_exp2f(v[j & 7] * 0.001f);
