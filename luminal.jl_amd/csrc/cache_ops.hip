@@ -24,6 +24,7 @@ namespace {
 
 template <typename E>
 __global__ __launch_bounds__(256) void rope_kernel(RopeArgs a) {
+  request_args(a);
   using raw = typename E::raw;
   const int half = a.D / 2;
   const int64_t total = (int64_t)a.B * a.H * a.S * half;
@@ -46,6 +47,7 @@ __global__ __launch_bounds__(256) void rope_kernel(RopeArgs a) {
 
 template <typename E>
 __global__ __launch_bounds__(256) void kv_append_kernel(KvAppendArgs a) {
+  request_args(a);
   using raw = typename E::raw;
   const int64_t total = (int64_t)a.B * a.Hkv * a.T * a.D;
   const int half = a.D / 2;
@@ -134,6 +136,8 @@ __device__ inline void sincos_pairs(float pos, int j0, int n, int D, float log2_
 // IL = true : thread owns pairs j = c V/2 .. , i.e. chunk c of the row.
 template <typename E, bool IL>
 __global__ __launch_bounds__(256) void rope_vec_kernel(RopeArgs a, int heads_per_block) {
+  request_args(a);
+  request_arg(heads_per_block);
   using raw = typename E::raw;
   constexpr int V = E::kVec;
   const int half = a.D / 2;
@@ -185,6 +189,8 @@ __global__ __launch_bounds__(256) void rope_vec_kernel(RopeArgs a, int heads_per
 // blocks of heads.
 template <typename E>
 __global__ __launch_bounds__(256) void kv_append_vec_kernel(KvAppendArgs a, int heads_per_block) {
+  request_args(a);
+  request_arg(heads_per_block);
   using raw = typename E::raw;
   constexpr int V = E::kVec;
   const int half = a.D / 2;

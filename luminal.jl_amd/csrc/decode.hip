@@ -121,6 +121,8 @@ struct QFrag<BF16> {
 // for LPK <= 16, none through LDS at all. Slots, then waves, are merged once after the loop.
 template <typename E, int LPK, int G>
 __global__ __launch_bounds__(kWaves * 64) void decode_split_kernel(DecodeArgs a, int g_chunks) {
+  request_args(a);
+  request_arg(g_chunks);
   using raw = typename E::raw;
   constexpr int VEC = E::kVec;
   constexpr int KPW = 64 / LPK;                          // keys per wave per load step
@@ -306,6 +308,7 @@ constexpr int kMergePrefetch = 16;     // partial rows fetched before the slot s
 // writes the row into the caches (the reference rebuilds them with _kv_scatter, src/Whisper.jl:552-570).
 template <typename E, bool STEP>
 __global__ __launch_bounds__(kMergeThreads) void decode_merge_kernel(DecodeArgs a) {
+  request_args(a);
   using raw = typename E::raw;
   __shared__ float w_s[kMergeMaxSlots];
   __shared__ float red_m[kMergeThreads / 64], red_l[kMergeThreads / 64], red_s[kMergeThreads / 64];

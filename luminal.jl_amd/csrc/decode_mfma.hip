@@ -72,6 +72,8 @@ constexpr int kMaxBatchPersistent = 1024;  // prefix sums live in LDS
 
 template <typename MT, int D>
 __global__ __launch_bounds__(kWaves * 64) void decode_mfma_kernel(DecodeArgs a, int g_chunks) {
+  request_args(a);
+  request_arg(g_chunks);
   using vec8 = typename MT::vec8;
   constexpr int KS = D / 32;             // k-steps of S^T = K Q^T
   constexpr int DB = D / 16;             // 16-row blocks of O^T

@@ -41,6 +41,9 @@ typedef float floatx4_t __attribute__((ext_vector_type(4)));
 // own running max / sum / output, and the groups are merged through LDS at the end.
 template <int D, bool CAUSAL, int KSPLIT>
 __global__ __launch_bounds__(256, (KSPLIT > 1 ? 1 : D <= 96 ? 3 : 2)) void prefill_f32_kernel(PrefillArgs a, int n_q_tiles, int n_bh_groups) {
+  request_args(a);
+  request_arg(n_q_tiles);
+  request_arg(n_bh_groups);
   constexpr int BM = 128 / KSPLIT;  // query rows per workgroup
   constexpr int BT = BN * KSPLIT;   // keys per staged tile
   constexpr int RG = 4 / KSPLIT;    // waves (32-row groups) per key group

@@ -100,6 +100,9 @@ __device__ inline void rotate_q_fragments_with_table(typename MT::vec8 (&qreg)[D
 template <int D, int NW> constexpr int default_wps() { return D > 96 ? 2 : NW == 8 ? 4 : 3; }
 template <typename MT, int D, bool CAUSAL, int KSPLIT, int NW, int WPS>
 __global__ __launch_bounds__(64 * NW, WPS) void prefill_mfma_kernel(PrefillArgs a, int n_q_tiles, int n_bh_groups) {
+  request_args(a);
+  request_arg(n_q_tiles);
+  request_arg(n_bh_groups);
   using vec8 = typename MT::vec8;
   constexpr int BM = 32 * NW / KSPLIT;  // query rows per workgroup
   // keys per staged tile: 64; 128 where one workgroup has the CU to itself and LDS and registers allow (half the
@@ -581,6 +584,10 @@ __global__ __launch_bounds__(64 * NW, WPS) void prefill_mfma_kernel(PrefillArgs 
 constexpr int kWideMaxKeyGroups = 6;  // tiles of up to 192 keys: two buffers of them fit the LDS at D = 96
 template <typename MT, int D>
 __global__ __launch_bounds__(1024, 4) void prefill_mfma_wide_kernel(PrefillArgs a, int wgs_per_head, int n_bh_groups, int mixed) {
+  request_args(a);
+  request_arg(wgs_per_head);
+  request_arg(n_bh_groups);
+  request_arg(mixed);
   using vec8 = typename MT::vec8;
   constexpr int KS = D / 16, DB = D / 32;
   constexpr int LDK = D + kPadK, LDV = D + pad_v<D>();
@@ -840,6 +847,9 @@ __global__ __launch_bounds__(1024, 4) void prefill_mfma_wide_kernel(PrefillArgs 
 // ---------------------------------------------------------------------------------------------------------------
 template <typename MT, int D, bool CAUSAL>
 __global__ __launch_bounds__(512, 2) void prefill_mfma_pair_kernel(PrefillArgs a, int n_q_tiles, int n_bh_groups) {
+  request_args(a);
+  request_arg(n_q_tiles);
+  request_arg(n_bh_groups);
   using vec8 = typename MT::vec8;
   static_assert(!MT::kSplitP && !MT::kConvertV, "one weight fragment per V fragment, V tiles staged as they are: fp16");
   constexpr int NW = 8, BM = 256;

@@ -23,6 +23,7 @@ template <int DP> constexpr int keys_per_tile() { return DP > 128 ? 16 : 32; }
 
 template <typename E, int DP>
 __global__ __launch_bounds__(256) void prefill_valu_kernel(PrefillArgs a) {
+  request_args(a);
   using raw = typename E::raw;
   constexpr int NCH = DP / 16;  // float4 chunks per lane
   constexpr int kKeysPerTile = keys_per_tile<DP>();
